@@ -1,0 +1,182 @@
+/*
+ * ko.h - C ABI of the gfx950 (MI355X) operator library libko.so.
+ *
+ * Plain C: no HIP types, no C++ types.  Pointers named `in`, `out`, `A`, ...
+ * are DEVICE pointers unless the comment says host.  A stream is an opaque
+ * handle (a hipStream_t underneath; NULL is the default stream).  Every
+ * function returns a ko_status; 0 is success.  ko_last_error_string() returns
+ * a thread-local description of the last failure on the calling thread.
+ *
+ * The reference (donglinz/kernel_optimization) has no FFI: its seam is the
+ * `Tensor` class plus three `__global__` templates launched with
+ * <<<grid, block, smem, stream>>>.  Each entry point below names the reference
+ * interface it stands in for.
+ */
+#ifndef KO_H
+#define KO_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ko_stream_t;
+typedef void *ko_event_t;
+
+typedef enum ko_status {
+    KO_OK = 0,
+    KO_ERR_INVALID_ARGUMENT = 1,  /* null pointer, negative size, bad enum */
+    KO_ERR_UNSUPPORTED_SHAPE = 2, /* e.g. cols not a multiple of the vector width */
+    KO_ERR_RUNTIME = 3,           /* a HIP runtime call or a kernel launch failed */
+    KO_ERR_OUT_OF_MEMORY = 4,
+    KO_ERR_NO_DEVICE = 5
+} ko_status;
+
+/* Row-mapping policy: the reference's three implementations per operator.
+ * WARP  = row per (sub-)wavefront, row held in registers
+ *         (SoftMaxWarpImpl softmax.h:11-60, LayerNormWarpImpl layernorm.h:145-201)
+ * BLOCK = row per workgroup, row held on chip, LDS only for cross-wave partials
+ *         (SoftMaxBlockImpl softmax.h:62-113, LayerNormBlockImpl layernorm.h:204-252)
+ * BLOCK_NOCACHE = row per workgroup, row re-read from global memory
+ *         (SoftMaxBlockNoCacheImpl softmax.h:116-166, LayerNormBlockNoCacheImpl layernorm.h:254-300)
+ * AUTO  = chosen from the row length. */
+typedef enum ko_policy {
+    KO_POLICY_AUTO = 0,
+    KO_POLICY_WARP = 1,
+    KO_POLICY_BLOCK = 2,
+    KO_POLICY_BLOCK_NOCACHE = 3
+} ko_policy;
+
+typedef enum ko_dtype16 { KO_F16 = 0, KO_BF16 = 1 } ko_dtype16;
+typedef enum ko_layout { KO_ROW_MAJOR = 0, KO_COL_MAJOR = 1 } ko_layout;
+
+typedef struct ko_device_info_t {
+    char name[256];
+    char arch[64];              /* "gfx950..." */
+    int compute_units;
+    int wavefront_size;
+    int clock_khz;              /* peak engine clock */
+    int memory_clock_khz;
+    int memory_bus_bits;
+    int l2_bytes;
+    int lds_bytes_per_workgroup;
+    size_t hbm_bytes;
+} ko_device_info_t;
+
+/* ---- runtime: replaces the CUDA runtime calls made by common/tensor.cu:8-42,
+ *      checkCudaErrors (common/common.h:16-25) and the stream/event calls of the
+ *      benchmark drivers (nn_operators/softmax/main.cu:28-29,44-68). ---------- */
+const char *ko_last_error_string(void);
+const char *ko_status_name(int status);
+int ko_device_info(ko_device_info_t *info);
+
+int ko_malloc(void **device_ptr, size_t bytes);                 /* cudaMalloc, tensor.cu:10 */
+int ko_free(void *device_ptr);                                  /* cudaFree,   tensor.cu:25 */
+int ko_memset_async(void *device_ptr, int value, size_t bytes, ko_stream_t stream);
+int ko_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);                            /* tensor.cu:28-30 */
+int ko_memcpy_h2d_async(void *device_dst, const void *host_src, size_t bytes, ko_stream_t stream);  /* tensor.cu:32-34 */
+int ko_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes);                            /* tensor.cu:36-38 */
+int ko_memcpy_d2h_async(void *host_dst, const void *device_src, size_t bytes, ko_stream_t stream);  /* tensor.cu:40-42 */
+int ko_memcpy_d2d_async(void *device_dst, const void *device_src, size_t bytes, ko_stream_t stream);
+
+int ko_stream_create(ko_stream_t *stream);       /* cudaStreamCreateWithFlags(NonBlocking), softmax/main.cu:29 */
+int ko_stream_destroy(ko_stream_t stream);
+int ko_stream_synchronize(ko_stream_t stream);   /* softmax/main.cu:46,70 */
+int ko_device_synchronize(void);                 /* gemm/main.cu:152 */
+
+int ko_event_create(ko_event_t *event);                             /* softmax/main.cu:49-50 */
+int ko_event_record(ko_event_t event, ko_stream_t stream);          /* softmax/main.cu:57,61 */
+int ko_event_synchronize(ko_event_t event);                         /* softmax/main.cu:63 */
+int ko_event_elapsed_ms(float *ms, ko_event_t start, ko_event_t stop); /* softmax/main.cu:66 */
+int ko_event_destroy(ko_event_t event);
+
+/* ---- row softmax: replaces
+ *      softmax<K><<<grid, block, K::smem_in_bytes, stream>>>(T *in, T *out)
+ *      (nn_operators/softmax/softmax.h:168-174, launched at softmax/main.cu:58-60).
+ * in, out: row-major [rows, cols] fp32, contiguous; in == out is allowed.
+ * cols must be a multiple of 4 (the reference's static_assert, softmax.h:21).
+ * valid_len: NULL for no mask, else device int32[ceil(rows / rows_per_seq)];
+ * row r belongs to sequence r / rows_per_seq and every column
+ * j >= valid_len[seq] takes the value -10000 before the softmax. */
+int ko_softmax_f32(const float *in, float *out, int64_t rows, int64_t cols,
+                   const int32_t *valid_len, int64_t rows_per_seq, ko_stream_t stream);
+
+/* Same with the policy fixed by the caller (the three descriptor types). */
+int ko_softmax_f32_policy(const float *in, float *out, int64_t rows, int64_t cols,
+                          const int32_t *valid_len, int64_t rows_per_seq, int policy,
+                          ko_stream_t stream);
+
+/* ---- LayerNorm: replaces
+ *      layer_normalization<K><<<...>>>(Element *in, Element *out, Element epsilon,
+ *                                      Element *gamma = nullptr, Element *beta = nullptr)
+ *      (nn_operators/layernorm/layernorm.h:302-312, launched at layernorm/main.cu:57-59).
+ * in, out: row-major [rows, cols] fp32 (in == out allowed); gamma, beta: [cols]
+ * or NULL (each independently); mean, rstd: [rows] outputs or NULL.
+ * var divides by cols (unbiased == 0) or cols - 1 (unbiased != 0, the
+ * reference's intent at layernorm.h:48).  cols must be a multiple of 4. */
+int ko_layernorm_f32(const float *in, float *out, float *mean, float *rstd, const float *gamma,
+                     const float *beta, int64_t rows, int64_t cols, float eps, int unbiased,
+                     ko_stream_t stream);
+
+int ko_layernorm_f32_policy(const float *in, float *out, float *mean, float *rstd,
+                            const float *gamma, const float *beta, int64_t rows, int64_t cols,
+                            float eps, int unbiased, int policy, ko_stream_t stream);
+
+/* ---- SIMT-path SGEMM: replaces
+ *      gemm<GemmKernelSimt<...>><<<grid, K::thread_per_block, K::smem_total_size_in_bytes, stream>>>
+ *          (shape::GemmCoord problem_size, ElementA *A, ElementB *B, ElementC *C, ElementC *D)
+ *      (nn_operators/gemm/gemm.h:11-21, simt_gemm.h:299-374, launched at gemm/main.cu:111-117).
+ * D[m,n] = alpha * A[m,k] * B[k,n] + beta * C[m,n], all row-major fp32.
+ * C may be NULL (then beta is ignored); the reference's epilogue is alpha = beta = 1
+ * with C given, or D = A*B with C null (simt_gemm.h:325-373).
+ * m, n multiples of 4 are not required; any positive sizes are accepted. */
+int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
+                 float beta, const float *C, float *D, ko_stream_t stream);
+
+/* ---- tensor-core-path GEMM: replaces
+ *      gemm<GemmKernelTensorCore<half, half, half, ...>><<<...>>>(problem_size, A, B, C, D)
+ *      (nn_operators/gemm/tensor_core_gemm.h:341-399; its launch is commented out at gemm/main.cu:344).
+ * A [m,k] row-major; B logical [k,n], stored row-major (b_layout = KO_ROW_MAJOR,
+ * the reference's layout, tensor_core_gemm.h:178) or column-major (KO_COL_MAJOR:
+ * memory [n][k]); C, D [m,n] row-major.  Elements are binary16 or bfloat16
+ * (in_dtype); products accumulate in fp32 on the matrix cores; D is rounded once
+ * to the 16-bit type.  C may be NULL.  k must be a multiple of 8. */
+int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A, const void *B,
+                      int b_layout, float beta, const void *C, void *D, int in_dtype,
+                      ko_stream_t stream);
+
+/* ---- seeded device fills: replace the host RNG loops of the benchmark drivers
+ *      (softmax/main.cu:31-36, layernorm/main.cu:30-35, gemm/main.cu:46-66) with a
+ *      counter-based generator that gives the same tensor on host and device:
+ *      splitmix64(seed, counter) -> u in [0,1); uniform = lo + (hi-lo)*u;
+ *      normal = mean + std * sqrt(-2 ln(1-u(2i))) * cos(2 pi u(2i+1)); evaluated in
+ *      double, rounded once to the storage type.  `first` is the index of out[0]. */
+int ko_fill_normal_f32(float *out, int64_t n, uint64_t seed, double mean, double std,
+                       int64_t first, ko_stream_t stream);
+int ko_fill_uniform_f32(float *out, int64_t n, uint64_t seed, double lo, double hi, int64_t first,
+                        ko_stream_t stream);
+int ko_fill_uniform_16(void *out, int64_t n, uint64_t seed, double lo, double hi, int64_t first,
+                       int dtype, ko_stream_t stream);
+/* int32 lengths lo + floor((hi - lo + 1) * u), uniform on [lo, hi] */
+int ko_fill_lengths_i32(int32_t *out, int64_t n, uint64_t seed, int32_t lo, int32_t hi,
+                        ko_stream_t stream);
+
+/* ---- measurement helpers (no reference counterpart; used by the benchmark harness) */
+/* out[i] = in[i] for n floats, 128-bit accesses: the plain copy whose rate is the
+ * practical HBM ceiling the bandwidth kernels are compared with. */
+int ko_copy_f32(const float *in, float *out, int64_t n, ko_stream_t stream);
+/* Integer tuning knobs by name ("softmax.lanes_per_row", ...); value 0 restores the default.
+ * Unknown names return KO_ERR_INVALID_ARGUMENT. */
+int ko_set_tuning(const char *name, int value);
+int ko_get_tuning(const char *name, int *value);
+/* Cross-lane primitives check: each of the 64 lanes of one wavefront contributes
+ * in[lane]; out[lane] receives the all-reduce over its group of `group` lanes
+ * (group in {2,4,8,16,32,64}; op 0 = max, 1 = sum). */
+int ko_debug_wave_allreduce(const float *in, float *out, int group, int op, ko_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KO_H */

@@ -1,0 +1,106 @@
+"""Builds the native parts in-tree: libko.so (HIP kernels + C ABI, gfx950) and the
+pure C++ host layer (Tensor, benchmark drivers) that sits on top of the C ABI.
+
+Usage: python -m kernel_optimization_amd.build [--jobs N] [--only lib|host]
+"""
+import argparse
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+HOST = os.path.join(PKG, "host")
+LIB_DIR = os.path.join(PKG, "lib")
+BIN_DIR = os.path.join(PKG, "bin")
+OBJ_DIR = os.path.join(PKG, "build")
+LIB_PATH = os.path.join(LIB_DIR, "libko.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+
+# -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32 instructions.
+HIP_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    out = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines()
+                    if "packed-fp32-ops' is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def hip_sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def build_lib(jobs=4, verbose=False):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = []
+    cmds = []
+    for src in hip_sources():
+        obj = os.path.join(OBJ_DIR, src[:-4] + ".o")
+        objs.append(obj)
+        cmds.append([HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+    with concurrent.futures.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        for out in pool.map(_run, cmds):
+            if verbose and out.strip():
+                print(out)
+    out = _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+def build_host(verbose=False):
+    """Tensor + the three benchmark drivers: plain C++ (g++), linked against libko.so only."""
+    if not os.path.isdir(HOST):
+        return []
+    os.makedirs(BIN_DIR, exist_ok=True)
+    cxx = os.environ.get("CXX", "g++")
+    inc = os.path.join(ROOT, "include")
+    common = [cxx, "-O2", "-std=c++17", "-Wall", "-Wextra", "-I", inc]
+    tensor_obj = os.path.join(OBJ_DIR, "tensor.o")
+    _run(common + ["-fPIC", "-c", os.path.join(HOST, "tensor.cpp"), "-o", tensor_obj])
+    built = []
+    for name in ("softmax", "layernorm", "gemm", "host_selftest"):
+        src = os.path.join(HOST, name + "_main.cpp")
+        if not os.path.exists(src):
+            continue
+        exe = os.path.join(BIN_DIR, name)
+        _run(common + [src, tensor_obj, "-o", exe, "-L", LIB_DIR, "-lko", "-Wl,-rpath,$ORIGIN/../lib"])
+        built.append(exe)
+    return built
+
+
+def build_all(jobs=4, verbose=False):
+    lib = build_lib(jobs=jobs, verbose=verbose)
+    host = build_host(verbose=verbose)
+    return lib, host
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    ap.add_argument("--only", choices=["lib", "host"])
+    ap.add_argument("-v", "--verbose", action="store_true")
+    args = ap.parse_args(argv)
+    if args.only != "host":
+        print("built", build_lib(args.jobs, args.verbose))
+    if args.only != "lib":
+        for exe in build_host(args.verbose):
+            print("built", exe)
+
+
+if __name__ == "__main__":
+    main()

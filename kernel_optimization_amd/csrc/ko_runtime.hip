@@ -1,0 +1,247 @@
+// Runtime part of the C ABI: device memory, copies, streams, events, errors,
+// device query and the tuning table.  Stands in for the CUDA runtime calls of
+// the reference's common/tensor.cu:8-42 and benchmark drivers.
+#include "ko_internal.h"
+
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+namespace ko {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t err, const char *expr, const char *file, int line) {
+    int status = KO_ERR_RUNTIME;
+    if (err == hipErrorOutOfMemory) status = KO_ERR_OUT_OF_MEMORY;
+    if (err == hipErrorNoDevice || err == hipErrorInvalidDevice) status = KO_ERR_NO_DEVICE;
+    // Same information as the reference's checkCudaErrors line (common/common.h:19-21).
+    return fail(status, "HIP error at %s:%d code=%d(%s) \"%s\"", file, line, static_cast<int>(err),
+                hipGetErrorName(err), expr);
+}
+
+static std::mutex g_tuning_mutex;
+static std::map<std::string, int> &tuning_table() {
+    static std::map<std::string, int> t = {
+        {"softmax.lanes_per_row", 0}, {"softmax.blocks_per_cu", 0}, {"softmax.nontemporal", 0},
+        {"softmax.block_threads", 0},
+        {"layernorm.lanes_per_row", 0}, {"layernorm.blocks_per_cu", 0}, {"layernorm.nontemporal", 0},
+        {"layernorm.block_threads", 0},
+        {"sgemm.variant", 0}, {"gemm16.variant", 0}, {"copy.blocks_per_cu", 0},
+        {"copy.nontemporal", 0},
+    };
+    return t;
+}
+
+int tuning(const char *name) {
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    auto it = tuning_table().find(name);
+    return it == tuning_table().end() ? 0 : it->second;
+}
+
+int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+}  // namespace ko
+
+KO_EXPORT const char *ko_last_error_string(void) { return ko::g_last_error; }
+
+KO_EXPORT const char *ko_status_name(int status) {
+    switch (status) {
+        case KO_OK: return "KO_OK";
+        case KO_ERR_INVALID_ARGUMENT: return "KO_ERR_INVALID_ARGUMENT";
+        case KO_ERR_UNSUPPORTED_SHAPE: return "KO_ERR_UNSUPPORTED_SHAPE";
+        case KO_ERR_RUNTIME: return "KO_ERR_RUNTIME";
+        case KO_ERR_OUT_OF_MEMORY: return "KO_ERR_OUT_OF_MEMORY";
+        case KO_ERR_NO_DEVICE: return "KO_ERR_NO_DEVICE";
+        default: return "KO_ERR_UNKNOWN";
+    }
+}
+
+KO_EXPORT int ko_set_tuning(const char *name, int value) {
+    if (!name) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: null name");
+    std::lock_guard<std::mutex> lock(ko::g_tuning_mutex);
+    auto it = ko::tuning_table().find(name);
+    if (it == ko::tuning_table().end())
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: unknown knob \"%s\"", name);
+    it->second = value;
+    return KO_OK;
+}
+
+KO_EXPORT int ko_get_tuning(const char *name, int *value) {
+    if (!name || !value) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: null argument");
+    std::lock_guard<std::mutex> lock(ko::g_tuning_mutex);
+    auto it = ko::tuning_table().find(name);
+    if (it == ko::tuning_table().end())
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: unknown knob \"%s\"", name);
+    *value = it->second;
+    return KO_OK;
+}
+
+KO_EXPORT int ko_device_info(ko_device_info_t *info) {
+    if (!info) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_device_info: null info");
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) {
+        (void)hipGetLastError();
+        return ko::fail(KO_ERR_NO_DEVICE, "ko_device_info: no HIP device visible");
+    }
+    int dev = 0;
+    KO_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    KO_HIP(hipGetDeviceProperties(&prop, dev));
+    std::memset(info, 0, sizeof(*info));
+    std::strncpy(info->name, prop.name, sizeof(info->name) - 1);
+    std::strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->clock_khz = prop.clockRate;
+    info->memory_clock_khz = prop.memoryClockRate;
+    info->memory_bus_bits = prop.memoryBusWidth;
+    info->l2_bytes = prop.l2CacheSize;
+    info->lds_bytes_per_workgroup = static_cast<int>(prop.sharedMemPerBlock);
+    info->hbm_bytes = prop.totalGlobalMem;
+    return KO_OK;
+}
+
+KO_EXPORT int ko_malloc(void **device_ptr, size_t bytes) {
+    if (!device_ptr) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_malloc: null result pointer");
+    *device_ptr = nullptr;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMalloc(device_ptr, bytes));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_free(void *device_ptr) {
+    if (!device_ptr) return KO_OK;
+    KO_HIP(hipFree(device_ptr));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memset_async(void *device_ptr, int value, size_t bytes, ko_stream_t stream) {
+    if (bytes == 0) return KO_OK;
+    if (!device_ptr) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_memset_async: null pointer");
+    KO_HIP(hipMemsetAsync(device_ptr, value, bytes, ko::as_stream(stream)));
+    return KO_OK;
+}
+
+static int check_copy(const void *dst, const void *src, size_t bytes, const char *who) {
+    if (bytes && (!dst || !src)) return ko::fail(KO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes) {
+    if (int rc = check_copy(device_dst, host_src, bytes, "ko_memcpy_h2d")) return rc;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMemcpy(device_dst, host_src, bytes, hipMemcpyHostToDevice));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memcpy_h2d_async(void *device_dst, const void *host_src, size_t bytes,
+                                  ko_stream_t stream) {
+    if (int rc = check_copy(device_dst, host_src, bytes, "ko_memcpy_h2d_async")) return rc;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes) {
+    if (int rc = check_copy(host_dst, device_src, bytes, "ko_memcpy_d2h")) return rc;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMemcpy(host_dst, device_src, bytes, hipMemcpyDeviceToHost));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memcpy_d2h_async(void *host_dst, const void *device_src, size_t bytes,
+                                  ko_stream_t stream) {
+    if (int rc = check_copy(host_dst, device_src, bytes, "ko_memcpy_d2h_async")) return rc;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_memcpy_d2d_async(void *device_dst, const void *device_src, size_t bytes,
+                                  ko_stream_t stream) {
+    if (int rc = check_copy(device_dst, device_src, bytes, "ko_memcpy_d2d_async")) return rc;
+    if (bytes == 0) return KO_OK;
+    KO_HIP(hipMemcpyAsync(device_dst, device_src, bytes, hipMemcpyDeviceToDevice,
+                          ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_stream_create(ko_stream_t *stream) {
+    if (!stream) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_stream_create: null result pointer");
+    hipStream_t s = nullptr;
+    // Non-blocking with respect to the default stream, default priority.
+    KO_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = reinterpret_cast<ko_stream_t>(s);
+    return KO_OK;
+}
+
+KO_EXPORT int ko_stream_destroy(ko_stream_t stream) {
+    if (!stream) return KO_OK;
+    KO_HIP(hipStreamDestroy(ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_stream_synchronize(ko_stream_t stream) {
+    KO_HIP(hipStreamSynchronize(ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_device_synchronize(void) {
+    KO_HIP(hipDeviceSynchronize());
+    return KO_OK;
+}
+
+KO_EXPORT int ko_event_create(ko_event_t *event) {
+    if (!event) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_event_create: null result pointer");
+    hipEvent_t e = nullptr;
+    KO_HIP(hipEventCreate(&e));
+    *event = reinterpret_cast<ko_event_t>(e);
+    return KO_OK;
+}
+
+KO_EXPORT int ko_event_record(ko_event_t event, ko_stream_t stream) {
+    if (!event) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_event_record: null event");
+    KO_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), ko::as_stream(stream)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_event_synchronize(ko_event_t event) {
+    if (!event) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_event_synchronize: null event");
+    KO_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_event_elapsed_ms(float *ms, ko_event_t start, ko_event_t stop) {
+    if (!ms || !start || !stop)
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_event_elapsed_ms: null argument");
+    KO_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start),
+                               reinterpret_cast<hipEvent_t>(stop)));
+    return KO_OK;
+}
+
+KO_EXPORT int ko_event_destroy(ko_event_t event) {
+    if (!event) return KO_OK;
+    KO_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+    return KO_OK;
+}

@@ -1,0 +1,420 @@
+// Row softmax for gfx950: one pass over HBM (each element read once, written
+// once), fp32, optional per-sequence padding mask.
+//
+// Three mappings, the counterparts of the reference's three policies
+// (nn_operators/softmax/softmax.h):
+//   WARP          a row lives in the registers of a group of LPR lanes of one
+//                 wavefront (LPR in {8,16,32,64}; 64/LPR rows per wavefront),
+//                 VPL 128-bit vectors per lane; max and sum are DPP /
+//                 permlane-swap all-reduces; no LDS.      (SoftMaxWarpImpl, :11-60)
+//   BLOCK         a row lives in the registers of one workgroup; LDS carries only
+//                 the per-wave partials.                  (SoftMaxBlockImpl, :62-113)
+//   BLOCK_NOCACHE rows of any length: pass 1 keeps a running (max, sum) per
+//                 thread (online rescaling), pass 2 re-reads the row and writes:
+//                 two reads + one write instead of the reference's three reads.
+//                                                        (SoftMaxBlockNoCacheImpl, :116-166)
+//
+// Per row: m = max_j x_j (running max starts at -FLT_MAX, softmax.h:33),
+// e_j = exp(x_j - m), s = sum_j e_j, y_j = e_j / s  (softmax.h:35-57; the
+// intended x - m, not the x + m the reference's Subtract functor computes,
+// common/functors.h:168).
+//
+// Mask: columns j >= valid_len[row / rows_per_seq] take the value -10000.  Vectors
+// that lie wholly in the padded part are not loaded.
+#include "ko_internal.h"
+#include "wave64.h"
+
+#include <cfloat>
+
+namespace ko {
+namespace {
+
+constexpr float kMaskValue = -10000.0f;
+
+// Loads vector j (columns 4j..4j+3) of a row whose first `vlen` columns are valid.
+template <bool MASKED, bool NT>
+__device__ __forceinline__ float4v load_row_vec(const float *row, int j, int vlen) {
+    const int c = 4 * j;
+    if constexpr (!MASKED) {
+        return load4<NT>(row + c);
+    } else {
+        float4v v = {kMaskValue, kMaskValue, kMaskValue, kMaskValue};
+        if (c < vlen) {
+            float4v x = load4<NT>(row + c);
+            v[0] = x[0];
+            if (c + 1 < vlen) v[1] = x[1];
+            if (c + 2 < vlen) v[2] = x[2];
+            if (c + 3 < vlen) v[3] = x[3];
+        }
+        return v;
+    }
+}
+
+__device__ __forceinline__ int clamp_len(int v, int cols) { return v < 0 ? 0 : (v > cols ? cols : v); }
+
+// ---------------------------------------------------------------- WARP policy
+template <int LPR, int VPL, bool MASKED, bool NT>
+__global__ __launch_bounds__(256) void softmax_wave_kernel(const float *__restrict__ in,
+                                                           float *__restrict__ out, int64_t rows,
+                                                           int cols, const int32_t *__restrict__ valid_len,
+                                                           int64_t rows_per_seq) {
+    constexpr int RPW = 64 / LPR;  // rows per wavefront
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPR;
+    const int l = lane % LPR;
+    const int nvec = cols >> 2;
+    const int64_t waves_per_block = blockDim.x >> 6;
+    const int64_t wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * RPW;
+
+    for (int64_t row0 = wave * RPW; row0 < rows; row0 += stride) {
+        const int64_t row = row0 + sub;
+        const bool row_ok = row < rows;
+        const float *src = in + row * cols;
+        int vlen = cols;
+        if constexpr (MASKED) {
+            if (row_ok) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+        }
+
+        float4v v[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = l + k * LPR;
+            if (row_ok && j < nvec) {
+                v[k] = load_row_vec<MASKED, NT>(src, j, vlen);
+            } else {
+                v[k] = float4v{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+            }
+        }
+
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) m = fmaxf(fmaxf(fmaxf(m, v[k][0]), fmaxf(v[k][1], v[k][2])), v[k][3]);
+        m = wave::allreduce<LPR, wave::Max>(m);
+
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[k][e] = exp_nonpositive(v[k][e] - m);
+                s += v[k][e];
+            }
+        }
+        s = wave::allreduce<LPR, wave::Sum>(s);
+        const float inv = 1.0f / s;
+
+        float *dst = out + row * cols;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = l + k * LPR;
+            if (row_ok && j < nvec) store4<NT>(dst + 4 * j, v[k] * inv);
+        }
+    }
+}
+
+// --------------------------------------------------------------- BLOCK policy
+// Workgroup-wide all-reduce: wave all-reduce, then every thread folds the per-wave
+// partials from LDS in the same order (bit-identical result in every thread).
+template <int THREADS, class Op>
+__device__ __forceinline__ float block_allreduce(float v, float *lds, float identity) {
+    constexpr int WAVES = THREADS / 64;
+    v = wave::allreduce<64, Op>(v);
+    if constexpr (WAVES == 1) return v;
+    __syncthreads();  // previous use of lds finished
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = identity;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) r = Op()(r, lds[w]);
+    return r;
+}
+
+template <int THREADS, int VPL, bool MASKED, bool NT>
+__global__ __launch_bounds__(THREADS) void softmax_block_kernel(const float *__restrict__ in,
+                                                                float *__restrict__ out, int64_t rows,
+                                                                int cols,
+                                                                const int32_t *__restrict__ valid_len,
+                                                                int64_t rows_per_seq) {
+    __shared__ float lds[16];
+    const int nvec = cols >> 2;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const float *src = in + row * cols;
+        int vlen = cols;
+        if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+        float4v v[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            if (j < nvec) v[k] = load_row_vec<MASKED, NT>(src, j, vlen);
+            else v[k] = float4v{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+        }
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) m = fmaxf(fmaxf(fmaxf(m, v[k][0]), fmaxf(v[k][1], v[k][2])), v[k][3]);
+        m = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[k][e] = exp_nonpositive(v[k][e] - m);
+                s += v[k][e];
+            }
+        }
+        s = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
+        const float inv = 1.0f / s;
+        float *dst = out + row * cols;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            if (j < nvec) store4<NT>(dst + 4 * j, v[k] * inv);
+        }
+    }
+}
+
+// ------------------------------------------------------- BLOCK_NOCACHE policy
+// Online pair (m, s): s = sum exp(x - m) over the elements seen so far.
+__device__ __forceinline__ void online_add(float &m, float &s, float x) {
+    if (x > m) {
+        s = s * exp_nonpositive(m - x) + 1.0f;
+        m = x;
+    } else {
+        s += exp_nonpositive(x - m);
+    }
+}
+
+template <int THREADS, bool MASKED>
+__global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const float *__restrict__ in,
+                                                                  float *__restrict__ out,
+                                                                  int64_t rows, int cols,
+                                                                  const int32_t *__restrict__ valid_len,
+                                                                  int64_t rows_per_seq) {
+    __shared__ float lds[16];
+    const int nvec = cols >> 2;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const float *src = in + row * cols;
+        int vlen = cols;
+        if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+        float m = -FLT_MAX, s = 0.0f;
+        for (int j = threadIdx.x; j < nvec; j += THREADS) {
+            float4v x = load_row_vec<MASKED, false>(src, j, vlen);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) online_add(m, s, x[e]);
+        }
+        const float gm = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
+        s *= exp_nonpositive(m - gm);  // threads that saw nothing: s = 0
+        const float gs = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
+        const float inv = 1.0f / gs;
+        float *dst = out + row * cols;
+        for (int j = threadIdx.x; j < nvec; j += THREADS) {
+            float4v x = load_row_vec<MASKED, false>(src, j, vlen);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = exp_nonpositive(x[e] - gm) * inv;
+            store4<false>(dst + 4 * j, x);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ dispatch
+struct Args {
+    const float *in;
+    float *out;
+    int64_t rows;
+    int cols;
+    const int32_t *valid_len;
+    int64_t rows_per_seq;
+    hipStream_t stream;
+};
+
+template <int LPR, int VPL, bool MASKED, bool NT>
+int launch_wave(const Args &a) {
+    constexpr int RPW = 64 / LPR;
+    constexpr int kThreads = 256;
+    const int64_t rows_per_block = RPW * (kThreads / 64);
+    const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
+    int per_cu = tuning("softmax.blocks_per_cu");
+    if (per_cu <= 0) per_cu = 8;
+    int64_t grid = static_cast<int64_t>(compute_units()) * per_cu;
+    if (grid > needed) grid = needed;
+    softmax_wave_kernel<LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <int LPR, bool MASKED, bool NT>
+int launch_wave_vpl(const Args &a, int vpl) {
+    switch (vpl) {
+        case 1: return launch_wave<LPR, 1, MASKED, NT>(a);
+        case 2: return launch_wave<LPR, 2, MASKED, NT>(a);
+        case 3: return launch_wave<LPR, 3, MASKED, NT>(a);
+        case 4: return launch_wave<LPR, 4, MASKED, NT>(a);
+        case 5:
+        case 6: return launch_wave<LPR, 6, MASKED, NT>(a);
+        default: return launch_wave<LPR, 8, MASKED, NT>(a);
+    }
+}
+
+template <bool MASKED, bool NT>
+int launch_wave_lpr(const Args &a, int lpr) {
+    const int nvec = a.cols / 4;
+    const int vpl = (nvec + lpr - 1) / lpr;
+    switch (lpr) {
+        case 8: return launch_wave_vpl<8, MASKED, NT>(a, vpl);
+        case 16: return launch_wave_vpl<16, MASKED, NT>(a, vpl);
+        case 32: return launch_wave_vpl<32, MASKED, NT>(a, vpl);
+        default: return launch_wave_vpl<64, MASKED, NT>(a, vpl);
+    }
+}
+
+constexpr int kWaveMaxVpl = 8;
+constexpr int kWaveMaxCols = 64 * kWaveMaxVpl * 4;    // 2048
+constexpr int kBlockMaxCols = 1024 * 8 * 4;           // 32768
+
+// Lanes per row for the WARP policy: the widest group whose lanes each hold at least
+// two vectors (more bytes in flight per lane), never so narrow that a lane would
+// need more than kWaveMaxVpl vectors.
+int default_lanes_per_row(int cols) {
+    const int nvec = cols / 4;
+    int lpr = 64;
+    while (lpr > 8 && nvec < 2 * lpr) lpr >>= 1;
+    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    return lpr;
+}
+
+template <bool MASKED>
+int launch_wave_any(const Args &a) {
+    int lpr = tuning("softmax.lanes_per_row");
+    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(a.cols);
+    while (lpr < 64 && (a.cols / 4 + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    if (tuning("softmax.nontemporal") == 1) return launch_wave_lpr<MASKED, true>(a, lpr);
+    return launch_wave_lpr<MASKED, false>(a, lpr);
+}
+
+template <int THREADS, bool MASKED>
+int launch_block_threads(const Args &a) {
+    const int nvec = a.cols / 4;
+    const int vpl = (nvec + THREADS - 1) / THREADS;
+    int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
+    if (grid > a.rows) grid = a.rows;
+    dim3 g(static_cast<unsigned>(grid)), b(THREADS);
+#define KO_SM_BLOCK(V)                                                                         \
+    softmax_block_kernel<THREADS, V, MASKED, false><<<g, b, 0, a.stream>>>(                      \
+        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq)
+    if (vpl <= 1) KO_SM_BLOCK(1);
+    else if (vpl <= 2) KO_SM_BLOCK(2);
+    else if (vpl <= 4) KO_SM_BLOCK(4);
+    else KO_SM_BLOCK(8);
+#undef KO_SM_BLOCK
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <bool MASKED>
+int launch_block(const Args &a) {
+    const int nvec = a.cols / 4;
+    int threads = tuning("softmax.block_threads");
+    if (threads != 256 && threads != 512 && threads != 1024) {
+        threads = 256;
+        while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;
+    }
+    while (threads < 1024 && (nvec + threads - 1) / threads > 8) threads <<= 1;
+    if (threads == 256) return launch_block_threads<256, MASKED>(a);
+    if (threads == 512) return launch_block_threads<512, MASKED>(a);
+    return launch_block_threads<1024, MASKED>(a);
+}
+
+template <bool MASKED>
+int launch_nocache(const Args &a) {
+    constexpr int kThreads = 1024;
+    int64_t grid = static_cast<int64_t>(compute_units()) * 4;
+    if (grid > a.rows) grid = a.rows;
+    softmax_nocache_kernel<kThreads, MASKED><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <bool MASKED>
+int dispatch(const Args &a, int policy) {
+    if (policy == KO_POLICY_AUTO) {
+        policy = a.cols <= kWaveMaxCols ? KO_POLICY_WARP
+                 : a.cols <= kBlockMaxCols ? KO_POLICY_BLOCK
+                                           : KO_POLICY_BLOCK_NOCACHE;
+    }
+    switch (policy) {
+        case KO_POLICY_WARP:
+            if (a.cols > kWaveMaxCols)
+                return fail(KO_ERR_UNSUPPORTED_SHAPE,
+                            "softmax: WARP policy holds at most %d columns per row, got %d", kWaveMaxCols,
+                            a.cols);
+            return launch_wave_any<MASKED>(a);
+        case KO_POLICY_BLOCK:
+            if (a.cols > kBlockMaxCols)
+                return fail(KO_ERR_UNSUPPORTED_SHAPE,
+                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxCols,
+                            a.cols);
+            return launch_block<MASKED>(a);
+        case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<MASKED>(a);
+        default: return fail(KO_ERR_INVALID_ARGUMENT, "softmax: unknown policy %d", policy);
+    }
+}
+
+}  // namespace
+}  // namespace ko
+
+KO_EXPORT int ko_softmax_f32_policy(const float *in, float *out, int64_t rows, int64_t cols,
+                                    const int32_t *valid_len, int64_t rows_per_seq, int policy,
+                                    ko_stream_t stream) {
+    if (rows < 0 || cols <= 0)
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: rows=%lld cols=%lld", (long long)rows,
+                        (long long)cols);
+    if (cols % 4 != 0)
+        return ko::fail(KO_ERR_UNSUPPORTED_SHAPE,
+                        "softmax: cols=%lld is not a multiple of the vector width 4", (long long)cols);
+    if (cols > (1 << 30)) return ko::fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld too large", (long long)cols);
+    if (rows == 0) return KO_OK;
+    if (!in || !out) return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: null in/out pointer");
+    if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15)
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be 16-byte aligned");
+    if (valid_len && rows_per_seq <= 0)
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: valid_len given but rows_per_seq=%lld",
+                        (long long)rows_per_seq);
+    ko::Args a{in, out, rows, static_cast<int>(cols), valid_len, rows_per_seq, ko::as_stream(stream)};
+    return valid_len ? ko::dispatch<true>(a, policy) : ko::dispatch<false>(a, policy);
+}
+
+KO_EXPORT int ko_softmax_f32(const float *in, float *out, int64_t rows, int64_t cols,
+                             const int32_t *valid_len, int64_t rows_per_seq, ko_stream_t stream) {
+    return ko_softmax_f32_policy(in, out, rows, cols, valid_len, rows_per_seq, KO_POLICY_AUTO, stream);
+}
+
+// ---- cross-lane primitive check (see ko.h)
+namespace ko {
+namespace {
+template <int G>
+__global__ void wave_allreduce_kernel(const float *in, float *out, int op) {
+    float v = in[threadIdx.x];
+    out[threadIdx.x] = op == 0 ? wave::allreduce<G, wave::Max>(v) : wave::allreduce<G, wave::Sum>(v);
+}
+}  // namespace
+}  // namespace ko
+
+KO_EXPORT int ko_debug_wave_allreduce(const float *in, float *out, int group, int op,
+                                      ko_stream_t stream) {
+    if (!in || !out) return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: null pointer");
+    if (op != 0 && op != 1) return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: op=%d", op);
+    hipStream_t s = ko::as_stream(stream);
+    switch (group) {
+        case 2: ko::wave_allreduce_kernel<2><<<1, 64, 0, s>>>(in, out, op); break;
+        case 4: ko::wave_allreduce_kernel<4><<<1, 64, 0, s>>>(in, out, op); break;
+        case 8: ko::wave_allreduce_kernel<8><<<1, 64, 0, s>>>(in, out, op); break;
+        case 16: ko::wave_allreduce_kernel<16><<<1, 64, 0, s>>>(in, out, op); break;
+        case 32: ko::wave_allreduce_kernel<32><<<1, 64, 0, s>>>(in, out, op); break;
+        case 64: ko::wave_allreduce_kernel<64><<<1, 64, 0, s>>>(in, out, op); break;
+        default: return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: group=%d", group);
+    }
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}

@@ -1,0 +1,167 @@
+// Cross-lane primitives for 64-wide wavefronts on gfx950.
+//
+// The reference reduces over 32-lane warps with a __shfl_down_sync tree whose
+// result is valid in lane 0 and is then broadcast with __shfl_sync
+// (common/common.h:37-46, nn_operators/softmax/softmax.h:41-42).  Here every
+// step is a symmetric exchange (lane i pairs with a lane j that pairs back
+// with i), so after log2(G) steps every lane of a G-lane group holds the same
+// bits and no broadcast is needed:
+//   xor 1, xor 2        DPP quad_perm          (inside a quad)
+//   i <-> 7-i           DPP row_half_mirror    (quad 0 <-> quad 1 of an 8-lane half row)
+//   i <-> 15-i          DPP row_mirror         (the two halves of a 16-lane row)
+//   row 2k <-> row 2k+1 v_permlane16_swap      (gfx950)
+//   lanes 0-31 <-> 32-63 v_permlane32_swap     (gfx950)
+// No LDS is touched.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace ko {
+namespace wave {
+
+constexpr int kDppQuadXor1 = 0xB1;      // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;      // quad_perm:[2,3,0,1]
+constexpr int kDppRowMirror = 0x140;
+constexpr int kDppRowHalfMirror = 0x141;
+
+template <int Ctrl>
+__device__ __forceinline__ float dpp(float v) {
+    int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, Ctrl, 0xf, 0xf, true));
+}
+
+// Partner value across adjacent 16-lane rows (row 0 <-> 1, row 2 <-> 3).
+// v_permlane16_swap exchanges the odd rows of its first operand with the even
+// rows of its second; starting from two copies of v, the first result holds
+// the even row of each pair in both rows, the second the odd row in both.
+__device__ __forceinline__ void swap16(float v, float &even_rows, float &odd_rows) {
+    unsigned u = __builtin_bit_cast(unsigned, v);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    even_rows = __builtin_bit_cast(float, r[0]);
+    odd_rows = __builtin_bit_cast(float, r[1]);
+}
+
+// Same for the two 32-lane halves: first result = lower half's values in both
+// halves, second = upper half's.
+__device__ __forceinline__ void swap32(float v, float &lower, float &upper) {
+    unsigned u = __builtin_bit_cast(unsigned, v);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    lower = __builtin_bit_cast(float, r[0]);
+    upper = __builtin_bit_cast(float, r[1]);
+}
+
+struct Max {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct Sum {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+
+// All-reduce over aligned groups of G lanes (G in {1,2,4,8,16,32,64}).  Op must be
+// commutative; the result is bit-identical in every lane of the group.
+template <int G, class Op>
+__device__ __forceinline__ float allreduce(float v, Op op = Op()) {
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "");
+    if constexpr (G >= 2) v = op(v, dpp<kDppQuadXor1>(v));
+    if constexpr (G >= 4) v = op(v, dpp<kDppQuadXor2>(v));
+    if constexpr (G >= 8) v = op(v, dpp<kDppRowHalfMirror>(v));
+    if constexpr (G >= 16) v = op(v, dpp<kDppRowMirror>(v));
+    if constexpr (G >= 32) {
+        float a, b;
+        swap16(v, a, b);
+        v = op(a, b);
+    }
+    if constexpr (G >= 64) {
+        float a, b;
+        swap32(v, a, b);
+        v = op(a, b);
+    }
+    return v;
+}
+
+// Welford triplet (count, mean, M2).  The merge is Chan's pairwise update
+// (nn_operators/layernorm/layernorm.h:36-47, without the division of M2 by
+// count-1 at :48), written so that merge(a,b) and merge(b,a) give the same bits:
+//   n = na + nb;  mean = (na*ma + nb*mb)/n;  M2 = (M2a + M2b) + (mb-ma)^2 * na*nb/n
+// An empty side (count 0) is the identity; two empty sides stay empty.
+struct Welford {
+    float count, mean, m2;
+};
+
+__device__ __forceinline__ Welford welford_merge(const Welford &a, const Welford &b) {
+    Welford r;
+    r.count = a.count + b.count;
+    const float n = r.count > 0.0f ? r.count : 1.0f;  // both sides empty: 0/1 keeps the triplet at zero
+    r.mean = (a.count * a.mean + b.count * b.mean) / n;
+    const float d = b.mean - a.mean;
+    r.m2 = (a.m2 + b.m2) + d * d * (a.count * b.count / n);
+    return r;
+}
+
+template <int Ctrl>
+__device__ __forceinline__ Welford welford_dpp_step(const Welford &w) {
+    Welford o{dpp<Ctrl>(w.count), dpp<Ctrl>(w.mean), dpp<Ctrl>(w.m2)};
+    return welford_merge(w, o);
+}
+
+template <int G>
+__device__ __forceinline__ Welford welford_allreduce(Welford w) {
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "");
+    if constexpr (G >= 2) w = welford_dpp_step<kDppQuadXor1>(w);
+    if constexpr (G >= 4) w = welford_dpp_step<kDppQuadXor2>(w);
+    if constexpr (G >= 8) w = welford_dpp_step<kDppRowHalfMirror>(w);
+    if constexpr (G >= 16) w = welford_dpp_step<kDppRowMirror>(w);
+    if constexpr (G >= 32) {
+        Welford a, b;
+        swap16(w.count, a.count, b.count);
+        swap16(w.mean, a.mean, b.mean);
+        swap16(w.m2, a.m2, b.m2);
+        w = welford_merge(a, b);
+    }
+    if constexpr (G >= 64) {
+        Welford a, b;
+        swap32(w.count, a.count, b.count);
+        swap32(w.mean, a.mean, b.mean);
+        swap32(w.m2, a.m2, b.m2);
+        w = welford_merge(a, b);
+    }
+    return w;
+}
+
+}  // namespace wave
+
+// 128-bit global accesses, optionally non-temporal (streaming: data is touched once).
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <bool NT>
+__device__ __forceinline__ float4v load4(const float *p) {
+    const float4v *q = reinterpret_cast<const float4v *>(p);
+    if constexpr (NT) return __builtin_nontemporal_load(q);
+    return *q;
+}
+
+template <bool NT>
+__device__ __forceinline__ void store4(float *p, float4v v) {
+    float4v *q = reinterpret_cast<float4v *>(p);
+    if constexpr (NT) __builtin_nontemporal_store(v, q);
+    else *q = v;
+}
+
+// exp(d) for d <= 0, about 1 ulp: d*log2(e) is formed as a rounded product plus its
+// exact residual and the low part of log2(e), the integer part is split off and
+// applied with ldexp, and the hardware base-2 exponential (v_exp_f32) only sees a
+// fraction in [-0.5, 0.5].  Arguments below -128 are clamped (the result is 0 either way).
+__device__ __forceinline__ float exp_nonpositive(float d) {
+    const float kLog2eHi = 0x1.715476p+0f;
+    const float kLog2eLo = 0x1.4ae0cp-26f;
+    d = fmaxf(d, -128.0f);
+    float y = d * kLog2eHi;
+    float r = __builtin_fmaf(d, kLog2eHi, -y);
+    r = __builtin_fmaf(d, kLog2eLo, r);
+    float n = __builtin_rintf(y);
+    float f = (y - n) + r;
+    float e = __builtin_amdgcn_exp2f(f);
+    return __builtin_ldexpf(e, static_cast<int>(n));
+}
+
+}  // namespace ko

@@ -1,0 +1,183 @@
+"""GPU parity: ko_sgemm_f32 and ko_gemm_f16f32acc (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+from kernel_optimization_amd import inputs
+from tolerances import assert_gemm16_close, assert_sgemm_close
+
+pytestmark = pytest.mark.gpu
+
+SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5]
+GEMM16_VARIANTS = [0, 1, 2, 3, 4, 5]
+
+
+@pytest.fixture
+def sgemm_variant(ko, request):
+    ko.set_tuning("sgemm.variant", request.param)
+    yield request.param
+    ko.set_tuning("sgemm.variant", 0)
+
+
+@pytest.fixture
+def gemm16_variant(ko, request):
+    ko.set_tuning("gemm16.variant", request.param)
+    yield request.param
+    ko.set_tuning("gemm16.variant", 0)
+
+
+# ------------------------------------------------------------------------------------ SGEMM
+
+@pytest.mark.parametrize("sgemm_variant", SGEMM_VARIANTS, indirect=True)
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 256, 96), (200, 136, 40), (1, 4, 4), (65, 129, 33),
+                                   (37, 50, 7)])
+def test_sgemm_matches_oracle(ko, sgemm_variant, m, n, k):
+    A = inputs.uniform_f32((m, k), 11 + m)
+    B = inputs.uniform_f32((k, n), 13 + n)
+    ref, ap = oracle.sgemm(A, B, want_absprod=True)
+    assert_sgemm_close(ko.sgemm_host(A, B), ref, ap, k)
+
+
+def test_sgemm_cfg3_full(ko):
+    """1024^3, U(-1,1), alpha=1, beta=0, C null: the whole output against the oracle, with the
+    reference's own abs <= 1e-3 gate (nn_operators/gemm/main.cu:169-170) as well."""
+    c = inputs.make_inputs(3)
+    ref, ap = oracle.sgemm(c["A"], c["B"], want_absprod=True)
+    assert_sgemm_close(ko.sgemm_host(c["A"], c["B"]), ref, ap, 1024, reference_gate=True)
+
+
+def test_sgemm_epilogue(ko):
+    """D = acc + C (the reference's epilogue with C given, simt_gemm.h:325-354) and alpha/beta."""
+    m, n, k = 96, 160, 72
+    A, B = inputs.uniform_f32((m, k), 1), inputs.uniform_f32((k, n), 2)
+    C = inputs.normal_f32((m, n), 3)
+    for alpha, beta in ((1.0, 1.0), (0.5, -2.0), (2.0, 0.0)):
+        ref, ap = oracle.sgemm(A, B, C, alpha, beta, want_absprod=True)
+        bound_scale = abs(alpha) * ap + abs(beta) * np.abs(C)
+        assert_sgemm_close(ko.sgemm_host(A, B, C, alpha, beta), ref, bound_scale + 1e-6, k)
+
+
+def test_sgemm_exact_cases(ko):
+    """Identity known-answer test of the reference (A[idx] = idx/1024, B = I, gemm/main.cu:219,226),
+    all-ones -> exactly K, and small integers -> bit-exact for any summation order."""
+    n = 256
+    A = (np.arange(n * n) // 1024).astype(np.float32).reshape(n, n)
+    np.testing.assert_array_equal(ko.sgemm_host(A, np.eye(n, dtype=np.float32)), A)
+    np.testing.assert_array_equal(ko.sgemm_host(np.ones((64, 512), np.float32), np.ones((512, 128), np.float32)),
+                                  np.full((64, 128), 512, np.float32))
+    rng = np.random.default_rng(5)
+    Ai = rng.integers(-4, 5, (130, 1024)).astype(np.float32)
+    Bi = rng.integers(-4, 5, (1024, 72)).astype(np.float32)
+    np.testing.assert_array_equal(ko.sgemm_host(Ai, Bi), (Ai.astype(np.float64) @ Bi.astype(np.float64)))
+
+
+def test_sgemm_errors(ko):
+    buf = ko.DeviceBuffer(1 << 16)
+    with pytest.raises(ko.KoError) as e:
+        ko.sgemm(16, 16, 16, None, buf, buf)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    with pytest.raises(ko.KoError) as e:
+        ko.sgemm(-1, 16, 16, buf, buf, buf)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    ko.sgemm(0, 16, 16, buf, buf, buf)  # empty problem
+
+
+# ----------------------------------------------------------------------------------- GEMM16
+
+def _bits16(shape, seed, bf16):
+    if bf16:
+        return inputs.uniform_bf16_bits(shape, seed)
+    return inputs.uniform_f16(shape, seed).view(np.uint16)
+
+
+def _to_f64(bits, bf16):
+    return oracle.bf16_to_f64(bits) if bf16 else oracle.f16_to_f64(bits)
+
+
+@pytest.mark.parametrize("gemm16_variant", GEMM16_VARIANTS, indirect=True)
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768)])
+def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
+    A = _bits16((m, k), 21 + m, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 23 + n, bf16)
+    _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16)
+    got = ko.gemm16_host(A, B, m, n, k, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR,
+                         dtype=ko.BF16 if bf16 else ko.F16)
+    assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+
+
+def test_gemm16_odd_n(ko):
+    """n not a multiple of 4: the element-wise store path."""
+    m, n, k = 70, 45, 40
+    A, B = _bits16((m, k), 1, False), _bits16((n, k), 2, False)
+    _, ref64, ap = oracle.gemm16(A, B, m, n, k)
+    assert_gemm16_close(_to_f64(ko.gemm16_host(A, B, m, n, k), False), ref64, ap, k)
+
+
+def test_gemm16_epilogue(ko):
+    m, n, k = 160, 192, 64
+    A, B = _bits16((m, k), 4, False), _bits16((n, k), 5, False)
+    C = inputs.uniform_f16((m, n), 6, -2.0, 2.0).view(np.uint16)
+    for alpha, beta in ((1.0, 1.0), (0.5, -1.5)):
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, C_bits=C, alpha=alpha, beta=beta)
+        got = ko.gemm16_host(A, B, m, n, k, C_bits=C, alpha=alpha, beta=beta)
+        scale = abs(alpha) * ap + abs(beta) * np.abs(oracle.f16_to_f64(C))
+        assert_gemm16_close(_to_f64(got, False), ref64, scale, k)
+
+
+def test_gemm16_exact_cases(ko):
+    """Reference known-answer inputs (A[idx] = idx/1024, B = I, C = 0; gemm/main.cu:219,226,233) and
+    small integers (every partial sum < 2^11 is exact in fp32 and in binary16)."""
+    n = 256
+    A = (np.arange(n * n) // 1024).astype(np.float16)
+    I = np.eye(n, dtype=np.float16)
+    for layout in (ko.COL_MAJOR, ko.ROW_MAJOR):
+        got = ko.gemm16_host(A.view(np.uint16), I.view(np.uint16), n, n, n, b_layout=layout)
+        np.testing.assert_array_equal(got.view(np.float16), A.reshape(n, n))
+    rng = np.random.default_rng(9)
+    Ai = rng.integers(-2, 3, (96, 128)).astype(np.float16)
+    Bi = rng.integers(-2, 3, (200, 128)).astype(np.float16)  # [n][k]
+    got = ko.gemm16_host(Ai.view(np.uint16), Bi.view(np.uint16), 96, 200, 128).view(np.float16)
+    np.testing.assert_array_equal(got.astype(np.float64), Ai.astype(np.float64) @ Bi.astype(np.float64).T)
+
+
+def test_gemm16_cfg4_sampled(ko):
+    """BERT FFN up-projection at full size (16384 x 3072 x 768, fp16, column-major B), operands filled on
+    the device: 192 sampled rows of D against the oracle on the bytes the kernel read, and linearity
+    over the whole output (D(2A) == 2 D(A) bit for bit: scaling by 2 is exact in fp16 and fp32)."""
+    m, n, k = 16384, 3072, 768
+    dA, dB, dD = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(m * n * 2)
+    ko.fill_uniform_16(dA, m * k, inputs.tensor_seed(4, 0))
+    ko.fill_uniform_16(dB, n * k, inputs.tensor_seed(4, 1))
+    ko.gemm16(m, n, k, dA, dB, dD)
+    ko.synchronize()
+    A = dA.download(np.uint16, (m, k))
+    B = dB.download(np.uint16, (n, k))
+    D = dD.download(np.uint16, (m, n))
+    hostA = inputs.uniform_f16((8, k), inputs.tensor_seed(4, 0)).view(np.uint16)
+    np.testing.assert_array_equal(hostA, A[:8])  # device fill == host generator, bit for bit
+    idx = np.sort(np.concatenate([np.random.default_rng(1).choice(m, 184, replace=False),
+                                  [0, 1, 255, 256, m - 257, m - 256, m - 2, m - 1]]))
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k)
+    assert_gemm16_close(oracle.f16_to_f64(D[idx]), ref64, ap, k)
+    assert np.all(np.isfinite(D.view(np.float16)))
+    dA2 = ko.DeviceBuffer.from_numpy((A.view(np.float16) * np.float16(2)).view(np.uint16))
+    dD2 = ko.DeviceBuffer(m * n * 2)
+    ko.gemm16(m, n, k, dA2, dB, dD2)
+    ko.synchronize()
+    D2 = dD2.download(np.uint16, (m, n)).view(np.float16)
+    np.testing.assert_array_equal(D2, D.view(np.float16) * np.float16(2))
+
+
+def test_gemm16_errors(ko):
+    buf = ko.DeviceBuffer(1 << 16)
+    with pytest.raises(ko.KoError) as e:
+        ko.gemm16(16, 16, 12, buf, buf, buf)  # k % 8 != 0
+    assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
+    with pytest.raises(ko.KoError) as e:
+        ko.gemm16(16, 16, 16, buf, buf, buf, dtype=7)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    with pytest.raises(ko.KoError) as e:
+        ko.gemm16(16, 16, 16, buf, None, buf)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT

@@ -1,0 +1,143 @@
+"""GPU parity: ko_softmax_f32 (through the C ABI) against the CPU oracle on identical seeded inputs."""
+import numpy as np
+import pytest
+
+import oracle
+from kernel_optimization_amd import inputs
+from tolerances import assert_softmax_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_wave_allreduce_primitives(ko):
+    """DPP / permlane-swap all-reduce: every lane of a group ends with the group's max / sum."""
+    rng = np.random.default_rng(7)
+    x = rng.integers(-50, 50, 64).astype(np.float32)  # integers: sums are exact in any order
+    dx, dy = ko.DeviceBuffer.from_numpy(x), ko.DeviceBuffer(256)
+    for g in (2, 4, 8, 16, 32, 64):
+        for op, fn in ((0, np.max), (1, np.sum)):
+            ko.check(ko.lib().ko_debug_wave_allreduce(dx.ptr, dy.ptr, g, op, None))
+            ko.synchronize()
+            got = dy.download(np.float32, (64,))
+            want = np.repeat(fn(x.reshape(64 // g, g), axis=1), g)
+            np.testing.assert_array_equal(got, want, err_msg="group %d op %d" % (g, op))
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 128), (1024, 128), (1000, 128), (7, 4), (33, 36), (64, 512),
+                                       (129, 768), (5, 2048), (77, 1000), (3, 260)])
+def test_softmax_matches_oracle(ko, rows, cols):
+    x = inputs.normal_f32((rows, cols), 1234 + rows * 7 + cols, 0.0, 4.0)
+    assert_softmax_close(ko.softmax_host(x), oracle.softmax(x))
+
+
+@pytest.mark.parametrize("lpr", [8, 16, 32, 64])
+@pytest.mark.parametrize("cols", [128, 512])
+def test_softmax_every_lane_mapping(ko, lpr, cols):
+    x = inputs.normal_f32((515, cols), 99 + lpr, 0.0, 4.0)
+    ref = oracle.softmax(x)
+    ko.set_tuning("softmax.lanes_per_row", lpr)
+    try:
+        for nt in (0, 1):
+            ko.set_tuning("softmax.nontemporal", nt)
+            assert_softmax_close(ko.softmax_host(x), ref)
+    finally:
+        ko.set_tuning("softmax.lanes_per_row", 0)
+        ko.set_tuning("softmax.nontemporal", 0)
+
+
+@pytest.mark.parametrize("policy,rows,cols", [
+    (2, 37, 128), (2, 19, 1024), (2, 9, 4096), (2, 5, 8192), (2, 3, 32768), (2, 11, 5000),
+    (3, 37, 128), (3, 19, 1024), (3, 4, 40000), (3, 2, 131072),
+    (0, 3, 4096), (0, 2, 65536)])
+def test_softmax_block_policies(ko, policy, rows, cols):
+    """Row-per-workgroup (BLOCK) and re-read (BLOCK_NOCACHE) policies, and AUTO on long rows."""
+    x = inputs.normal_f32((rows, cols), 4321 + cols, 0.0, 4.0)
+    assert_softmax_close(ko.softmax_host(x, policy=policy), oracle.softmax(x))
+
+
+@pytest.mark.parametrize("policy", [0, 1, 2, 3])
+def test_masked_softmax_matches_oracle(ko, policy):
+    """cfg5 shape in small: 3 sequences x 40 rows x 512 columns, lengths in [64, 512] plus the edge lengths."""
+    rows_per_seq, cols = 40, 512
+    vl = np.concatenate([inputs.valid_lengths(3, 5), np.array([0, 1, 3, 4, 5, 255, 256, 257, 511, 512, 600, -3],
+                                                              np.int32)])
+    rows = rows_per_seq * len(vl) - 13  # last sequence is ragged
+    x = inputs.normal_f32((rows, cols), 55, 0.0, 4.0)
+    got = ko.softmax_host(x, valid_len=vl, rows_per_seq=rows_per_seq, policy=policy)
+    ref = oracle.softmax(x, valid_len=vl, rows_per_seq=rows_per_seq)
+    assert_softmax_close(got, ref)
+    # padded columns are exactly zero when at least one column is valid
+    for s, L in enumerate(vl):
+        L = int(np.clip(L, 0, cols))
+        blk = got[s * rows_per_seq:(s + 1) * rows_per_seq]
+        if 0 < L < cols:
+            assert np.all(blk[:, L:] == 0.0)
+        if L == 0:
+            np.testing.assert_array_equal(blk, np.full_like(blk, 1.0 / cols))
+
+
+def test_softmax_properties(ko):
+    cols = 128
+    # constant row -> exactly 1/C; one-hot dominance; large magnitudes stay finite (max subtraction)
+    x = np.zeros((4, cols), np.float32)
+    x[0] = 3.25
+    x[1, 0] = 100.0
+    x[2] = np.linspace(-80, 80, cols)
+    x[3] = 80.0
+    x[3, 5] = -80.0
+    y = ko.softmax_host(x)
+    np.testing.assert_array_equal(y[0], np.full(cols, 1.0 / cols, np.float32))
+    assert y[1, 0] == 1.0 and np.all(y[1, 1:] < 1e-40)
+    assert np.all(np.isfinite(y))
+    assert_softmax_close(y, oracle.softmax(x))
+    # shift invariance on exactly representable shifts, rows sum to 1
+    x = inputs.normal_f32((256, cols), 3, 0.0, 4.0)
+    xq = np.round(x * 64) / 64
+    a, b = ko.softmax_host(xq), ko.softmax_host(xq + np.float32(16.0))
+    np.testing.assert_array_equal(a, b)
+    assert np.abs(a.sum(1, dtype=np.float64) - 1).max() <= cols * 2.0 ** -24
+
+
+def test_softmax_in_place_and_empty(ko):
+    x = inputs.normal_f32((300, 512), 8, 0.0, 4.0)
+    assert_softmax_close(ko.softmax_host(x, in_place=True), oracle.softmax(x))
+    ko.softmax(None, None, 0, 128)  # zero rows: nothing to do, no error
+
+
+def test_softmax_errors(ko):
+    buf = ko.DeviceBuffer(4096)
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(buf, buf, 4, 130)  # cols % 4 != 0: the reference's static_assert (softmax.h:21)
+    assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(None, buf, 4, 128)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(buf, buf, 4, 128, valid_len=buf, rows_per_seq=0)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(buf, buf, 1, 4096, policy=1)  # WARP policy holds at most 2048 columns
+    assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert "WARP" in str(e.value)
+
+
+def test_softmax_full_size_cfg1_properties(ko):
+    """[196608,128] at full size, inputs filled on the device: sampled rows against the oracle on the
+    very bytes the kernel read, plus size-independent properties over the whole output."""
+    rows, cols = 196608, 128
+    n = rows * cols
+    dx, dy = ko.DeviceBuffer(n * 4), ko.DeviceBuffer(n * 4)
+    ko.fill_normal_f32(dx, n, inputs.tensor_seed(1, 0), 0.0, 4.0)
+    ko.softmax(dx, dy, rows, cols)
+    ko.synchronize()
+    x = dx.download(np.float32, (rows, cols))
+    y = dy.download(np.float32, (rows, cols))
+    assert np.all(np.isfinite(y)) and y.min() >= 0
+    assert np.abs(y.sum(1, dtype=np.float64) - 1).max() <= cols * 2.0 ** -24
+    assert np.array_equal(y[np.arange(rows), x.argmax(1)], y.max(1))  # order preserved at the top
+    idx = np.random.default_rng(0).choice(rows, 4096, replace=False)
+    idx = np.concatenate([idx, [0, 1, 2, 3, rows - 4, rows - 3, rows - 2, rows - 1]])
+    assert_softmax_close(y[idx], oracle.softmax(x[idx]))
+    # the device fill is the same generator as the host one
+    host = inputs.normal_f32((64, cols), inputs.tensor_seed(1, 0), 0.0, 4.0)
+    assert np.all(np.abs(host - x[:64]) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))
