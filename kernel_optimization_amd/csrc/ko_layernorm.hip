@@ -10,6 +10,13 @@
 // common/functors.h:168, and its merge divides M2 by count-1 at every step,
 // layernorm.h:48 - neither is reproduced).
 //
+// The statistics are taken of x - x0, x0 being the row's first element: fp32
+// Welford/Chan arithmetic rounds every partial mean to an ulp of the data's
+// magnitude, which costs a few 1e-5 of the variance when |mean| is 1e4 times the
+// standard deviation.  After the shift the partial means are of the size of the
+// spread, not of the offset, and x - x0 itself is exact or nearly so.
+// mean = x0 + mean(x - x0); its error is relative to the spread of the row.
+//
 // Mappings as in the reference: WARP (LayerNormWarpImpl :145-201) = row in the
 // registers of LPR lanes of a wavefront; BLOCK (LayerNormBlockImpl :204-252) =
 // row in the registers of a workgroup, per-wave triplets through LDS;
@@ -54,8 +61,8 @@ struct Args {
 
 // ---------------------------------------------------------------- WARP policy
 template <int LPR, int VPL, bool NT>
-__global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *__restrict__ in,
-                                                             float *__restrict__ out,
+__global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
+                                                             float *out,
                                                              float *__restrict__ mean_out,
                                                              float *__restrict__ rstd_out,
                                                              const float *__restrict__ gamma,
@@ -97,10 +104,12 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *__rest
             else v[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
         }
 
+        const float x0 = wave::broadcast_group_first<LPR>(v[0][0]);
         wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
+            v[k] = v[k] - x0;
             if (j < nvec) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) welford_update(w, v[k][e], rcp.v[4 * k + e + 1]);
@@ -108,7 +117,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *__rest
         }
         w = wave::welford_allreduce<LPR>(w);
 
-        const float mean = w.mean;
+        const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
 
         float *dst = out + row * cols;
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *__rest
             }
         }
         if (row_ok && l == 0) {
-            if (mean_out) mean_out[row] = mean;
+            if (mean_out) mean_out[row] = x0 + mean;
             if (rstd_out) rstd_out[row] = rstd;
         }
     }
@@ -152,8 +161,8 @@ __device__ __forceinline__ wave::Welford block_welford_allreduce(wave::Welford w
 }
 
 template <int THREADS, int VPL>
-__global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *__restrict__ in,
-                                                                  float *__restrict__ out,
+__global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *in,
+                                                                  float *out,
                                                                   float *__restrict__ mean_out,
                                                                   float *__restrict__ rstd_out,
                                                                   const float *__restrict__ gamma,
@@ -172,17 +181,19 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *_
             if (j < nvec) v[k] = load4<false>(src + 4 * j);
             else v[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
         }
+        const float x0 = src[0];
         wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
+            v[k] = v[k] - x0;
             if (j < nvec) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) welford_update(w, v[k][e], rcp.v[4 * k + e + 1]);
             }
         }
         w = block_welford_allreduce<THREADS>(w, lds);
-        const float mean = w.mean;
+        const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
         float *dst = out + row * cols;
 #pragma unroll
@@ -201,7 +212,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *_
             }
         }
         if (threadIdx.x == 0) {
-            if (mean_out) mean_out[row] = mean;
+            if (mean_out) mean_out[row] = x0 + mean;
             if (rstd_out) rstd_out[row] = rstd;
         }
     }
@@ -209,8 +220,8 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *_
 
 // ------------------------------------------------------- BLOCK_NOCACHE policy
 template <int THREADS>
-__global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float *__restrict__ in,
-                                                                    float *__restrict__ out,
+__global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float *in,
+                                                                    float *out,
                                                                     float *__restrict__ mean_out,
                                                                     float *__restrict__ rstd_out,
                                                                     const float *__restrict__ gamma,
@@ -221,9 +232,10 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float 
     const int nvec = cols >> 2;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const float *src = in + row * cols;
+        const float x0 = src[0];
         wave::Welford w{0.0f, 0.0f, 0.0f};
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load4<false>(src + 4 * j);
+            float4v x = load4<false>(src + 4 * j) - x0;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 // streaming update with a true division: the count is not a compile-time constant here
@@ -234,11 +246,11 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float 
             }
         }
         w = block_welford_allreduce<THREADS>(w, lds);
-        const float mean = w.mean;
+        const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
         float *dst = out + row * cols;
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load4<false>(src + 4 * j);
+            float4v x = load4<false>(src + 4 * j) - x0;
             float4v y;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -250,7 +262,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float 
             store4<false>(dst + 4 * j, y);
         }
         if (threadIdx.x == 0) {
-            if (mean_out) mean_out[row] = mean;
+            if (mean_out) mean_out[row] = x0 + mean;
             if (rstd_out) rstd_out[row] = rstd;
         }
     }

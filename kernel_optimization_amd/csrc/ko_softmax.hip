@@ -54,8 +54,8 @@ __device__ __forceinline__ int clamp_len(int v, int cols) { return v < 0 ? 0 : (
 
 // ---------------------------------------------------------------- WARP policy
 template <int LPR, int VPL, bool MASKED, bool NT>
-__global__ __launch_bounds__(256) void softmax_wave_kernel(const float *__restrict__ in,
-                                                           float *__restrict__ out, int64_t rows,
+__global__ __launch_bounds__(256) void softmax_wave_kernel(const float *in,
+                                                           float *out, int64_t rows,
                                                            int cols, const int32_t *__restrict__ valid_len,
                                                            int64_t rows_per_seq) {
     constexpr int RPW = 64 / LPR;  // rows per wavefront
@@ -131,8 +131,8 @@ __device__ __forceinline__ float block_allreduce(float v, float *lds, float iden
 }
 
 template <int THREADS, int VPL, bool MASKED, bool NT>
-__global__ __launch_bounds__(THREADS) void softmax_block_kernel(const float *__restrict__ in,
-                                                                float *__restrict__ out, int64_t rows,
+__global__ __launch_bounds__(THREADS) void softmax_block_kernel(const float *in,
+                                                                float *out, int64_t rows,
                                                                 int cols,
                                                                 const int32_t *__restrict__ valid_len,
                                                                 int64_t rows_per_seq) {
@@ -185,8 +185,8 @@ __device__ __forceinline__ void online_add(float &m, float &s, float x) {
 }
 
 template <int THREADS, bool MASKED>
-__global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const float *__restrict__ in,
-                                                                  float *__restrict__ out,
+__global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const float *in,
+                                                                  float *out,
                                                                   int64_t rows, int cols,
                                                                   const int32_t *__restrict__ valid_len,
                                                                   int64_t rows_per_seq) {

@@ -32,22 +32,38 @@ __device__ __forceinline__ float dpp(float v) {
 
 // Partner value across adjacent 16-lane rows (row 0 <-> 1, row 2 <-> 3).
 // v_permlane16_swap exchanges the odd rows of its first operand with the even
-// rows of its second; starting from two copies of v, the first result holds
-// the even row of each pair in both rows, the second the odd row in both.
+// rows of its second; starting from two copies of v, the first operand ends up
+// holding the even row of each pair in both rows, the second the odd row in both.
+// Written as inline assembly: with this compiler the two results of
+// __builtin_amdgcn_permlane16_swap / permlane32_swap come back in one register.
+// The s_nop before covers the wait states the instruction needs after a VALU write
+// of its operands (the compiler cannot see inside the asm to insert them).
 __device__ __forceinline__ void swap16(float v, float &even_rows, float &odd_rows) {
-    unsigned u = __builtin_bit_cast(unsigned, v);
-    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    even_rows = __builtin_bit_cast(float, r[0]);
-    odd_rows = __builtin_bit_cast(float, r[1]);
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    even_rows = a;
+    odd_rows = b;
 }
 
 // Same for the two 32-lane halves: first result = lower half's values in both
 // halves, second = upper half's.
 __device__ __forceinline__ void swap32(float v, float &lower, float &upper) {
-    unsigned u = __builtin_bit_cast(unsigned, v);
-    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    lower = __builtin_bit_cast(float, r[0]);
-    upper = __builtin_bit_cast(float, r[1]);
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lower = a;
+    upper = b;
+}
+
+// Value held by the first lane of each aligned group of G lanes, in every lane of the group.
+template <int G>
+__device__ __forceinline__ float broadcast_group_first(float v) {
+    const int bits = __builtin_bit_cast(int, v);
+    if constexpr (G == 64) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(bits));
+    } else {
+        const int lane = static_cast<int>(threadIdx.x) & 63;
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane & ~(G - 1)) << 2, bits));
+    }
 }
 
 struct Max {

@@ -145,7 +145,8 @@ def test_gemm16_exact_cases(ko):
 def test_gemm16_cfg4_sampled(ko):
     """BERT FFN up-projection at full size (16384 x 3072 x 768, fp16, column-major B), operands filled on
     the device: 192 sampled rows of D against the oracle on the bytes the kernel read, and linearity
-    over the whole output (D(2A) == 2 D(A) bit for bit: scaling by 2 is exact in fp16 and fp32)."""
+    over the whole output (D(2A) == 2 D(A) bit for bit wherever the result is a normal fp16 number:
+    scaling by 2 is exact in fp16 and fp32)."""
     m, n, k = 16384, 3072, 768
     dA, dB, dD = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(m * n * 2)
     ko.fill_uniform_16(dA, m * k, inputs.tensor_seed(4, 0))
@@ -167,7 +168,10 @@ def test_gemm16_cfg4_sampled(ko):
     ko.gemm16(m, n, k, dA2, dB, dD2)
     ko.synchronize()
     D2 = dD2.download(np.uint16, (m, n)).view(np.float16)
-    np.testing.assert_array_equal(D2, D.view(np.float16) * np.float16(2))
+    want = D.view(np.float16) * np.float16(2)
+    normal = np.abs(want) >= 2.0 ** -13  # subnormal results round on a fixed grid, so scaling is exact only above it
+    np.testing.assert_array_equal(D2[normal], want[normal])
+    assert np.abs(D2[~normal].astype(np.float64) - want[~normal].astype(np.float64)).max(initial=0.0) <= 2.0 ** -23
 
 
 def test_gemm16_errors(ko):

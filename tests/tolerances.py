@@ -1,7 +1,11 @@
 """Parity gates between the HIP kernels and the CPU oracle (the tolerances are part of the tests).
 
 softmax   |d| <= 1e-6  and  |d| <= 1e-5 * |ref| wherever |ref| >= FLT_MIN
-LayerNorm |dy| <= 1e-5 * max(|ref|, 1);  mean: |d| <= 1e-5 * max(|ref|, 1e-3);  rstd: |d| <= 1e-5 * |ref|
+LayerNorm |dy| <= 1e-5 * max(|ref|, 1);  rstd: |d| <= 1e-5 * |ref|;
+          mean: |d| <= 1e-5 * max(|ref mean|, ref std) with ref std = 1/ref rstd.  The mean is a sum with
+          cancellation: its fp32 partial sums are of the size of the row's spread, so an error relative to
+          |mean| alone is out of reach of any fp32 reduction when |mean| << std (partial sums of size
+          std*sqrt(n) carry an ulp of about 1e-7*std each)
 SGEMM     |d| <= 2 K 2^-24 * sum_k |a_ik||b_kj|   (any summation order), plus the reference's own
           gate |d| <= 1e-3 (nn_operators/gemm/main.cu:169-170) where the test says so
 GEMM16    |d| <= 2^-11 |ref| + K 2^-24 sum_k |a_ik||b_kj| + 2^-24   (one rounding to 16 bits + fp32 sums);
@@ -33,7 +37,8 @@ def assert_layernorm_close(got, ref):
     assert dy.max() <= 1e-5, "layernorm y err %.3e > 1e-5" % dy.max()
     if mean is not None:
         mean, rmean = np.asarray(mean, np.float64), np.asarray(rmean, np.float64)
-        dm = np.abs(mean - rmean) / np.maximum(np.abs(rmean), 1e-3)
+        scale = np.maximum(np.abs(rmean), 1.0 / np.asarray(rrstd, np.float64))
+        dm = np.abs(mean - rmean) / scale
         assert dm.max() <= 1e-5, "layernorm mean err %.3e > 1e-5" % dm.max()
     if rstd is not None:
         rstd, rrstd = np.asarray(rstd, np.float64), np.asarray(rrstd, np.float64)
