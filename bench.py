@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all/--no-all]
+
+A step is one launch of the operator over one batch of synthetic, seeded input that is
+already resident in HBM.  The headline workload is the masked row softmax
+[786432, 512] (3.2 GB of traffic: past the 256 MB Infinity Cache by itself); the other four
+configurations are measured as well (rotating buffer sets so that they, too, run out of
+HBM rather than out of the cache) and reported under "workloads".
+
+Prints ONE JSON line.  `value` is algorithmic bytes per second over the wall-clock of the K
+timed steps; `roofline.achieved` is the same algorithmic bytes over the average launch
+duration measured with HIP events on the launch stream.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import kernel_optimization_amd as ko  # noqa: E402
+from kernel_optimization_amd import inputs  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}
+WORKLOADS = {c["name"]: k for k, c in inputs.CONFIGS.items()}
+HEADLINE = 5
+
+
+def _traffic(name):
+    """HBM bytes per launch measured offline with rocprofv3 --pmc (profiles/hbm_traffic.json), or None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        return None
+
+
+def _time_steps(launch, steps, warmup):
+    """warmup untimed launches, then `steps` launches: wall clock bracketed by device syncs, and a
+    HIP event pair on the launch stream around the same launches."""
+    for i in range(warmup):
+        launch(i)
+    ko.synchronize()
+    e0, e1 = ko.Event(), ko.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        launch(warmup + i)
+    e1.record()
+    ko.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) / steps, e0.elapsed_ms(e1) * 1e-3 / steps
+
+
+def _vendor():
+    path = os.path.join(ROOT, "kernel_optimization_amd", "lib", "libko_vendor.so")
+    if not os.path.exists(path):
+        return None
+    V = ctypes.CDLL(path)
+    i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+    V.kov_gemm16.argtypes = [i64, i64, i64, vp, vp, ci, vp, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
+                             ctypes.POINTER(ci)]
+    V.kov_sgemm.argtypes = [i64, i64, i64, vp, vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ci)]
+    return V
+
+
+# ------------------------------------------------------------------------------ workloads
+
+def bench_softmax(cfg, steps, warmup):
+    c = inputs.CONFIGS[cfg]
+    rows, cols = c["rows"], c["cols"]
+    n = rows * cols
+    work = inputs.algorithmic_work(cfg)
+    nsets = max(1, -(-(1 << 30) // work))  # rotate through > 1 GiB of buffers unless one set is that big
+    xs = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    ys = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    for x in xs:
+        ko.fill_normal_f32(x, n, inputs.tensor_seed(cfg, 0), 0.0, 4.0)
+    vl, rps = None, 0
+    if "n_seq" in c:
+        vl, rps = ko.DeviceBuffer(c["n_seq"] * 4), c["rows_per_seq"]
+        ko.fill_lengths_i32(vl, c["n_seq"], inputs.tensor_seed(cfg, 1), c["len_lo"], c["len_hi"])
+    wall, dev = _time_steps(lambda i: ko.softmax(xs[i % nsets], ys[i % nsets], rows, cols, vl, rps), steps, warmup)
+    res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
+               ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
+               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
+               algorithmic_bytes=work, kernel_us=dev * 1e6)
+    keep = dict(x=xs[0], y=ys[0], vl=vl, rows=rows, cols=cols, rps=rps)
+    return res, keep
+
+
+def bench_layernorm(cfg, steps, warmup):
+    c = inputs.CONFIGS[cfg]
+    rows, cols = c["rows"], c["cols"]
+    n = rows * cols
+    work = inputs.algorithmic_work(cfg)
+    nsets = max(1, -(-(1 << 30) // work))
+    xs = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    ys = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    ms = [ko.DeviceBuffer(rows * 4) for _ in range(nsets)]
+    rs = [ko.DeviceBuffer(rows * 4) for _ in range(nsets)]
+    g, b = ko.DeviceBuffer(cols * 4), ko.DeviceBuffer(cols * 4)
+    for x in xs:
+        ko.fill_normal_f32(x, n, inputs.tensor_seed(cfg, 0), 0.5, 2.0)
+    ko.fill_normal_f32(g, cols, inputs.tensor_seed(cfg, 1), 1.0, 0.1)
+    ko.fill_normal_f32(b, cols, inputs.tensor_seed(cfg, 2), 0.0, 0.1)
+    wall, dev = _time_steps(lambda i: ko.layernorm(xs[i % nsets], ys[i % nsets], rows, cols, ms[i % nsets],
+                                                   rs[i % nsets], g, b, c["eps"]), steps, warmup)
+    return dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
+                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
+                roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                              frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
+                algorithmic_bytes=work, kernel_us=dev * 1e6), None
+
+
+def bench_sgemm(cfg, steps, warmup, vendor):
+    c = inputs.CONFIGS[cfg]
+    m, n, k = c["m"], c["n"], c["k"]
+    flops = inputs.algorithmic_work(cfg)
+    nsets = 32  # 12 MB per set: rotate through 400 MB
+    As = [ko.DeviceBuffer(m * k * 4) for _ in range(nsets)]
+    Bs = [ko.DeviceBuffer(k * n * 4) for _ in range(nsets)]
+    Ds = [ko.DeviceBuffer(m * n * 4) for _ in range(nsets)]
+    for a, b in zip(As, Bs):
+        ko.fill_uniform_f32(a, m * k, inputs.tensor_seed(cfg, 0))
+        ko.fill_uniform_f32(b, k * n, inputs.tensor_seed(cfg, 1))
+    wall, dev = _time_steps(lambda i: ko.sgemm(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
+    res = dict(workload=c["name"], metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
+               ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
+               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f32"], unit="TFLOP/s",
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=None),
+               flops=flops, kernel_us=dev * 1e6)
+    if vendor is not None:
+        us, na = ctypes.c_float(), ctypes.c_int()
+        tmp = ko.DeviceBuffer(m * n * 4)
+        if vendor.kov_sgemm(m, n, k, As[0].ptr, Bs[0].ptr, tmp.ptr, 16, 50, ctypes.byref(us), ctypes.byref(na)) == 0:
+            res["hipblaslt_tflops"] = flops / us.value / 1e6
+            res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
+            ref = tmp.download(np.float32, (m, n))
+            res["max_abs_diff_vs_hipblaslt"] = float(np.abs(Ds[0].download(np.float32, (m, n)) - ref).max())
+    return res, None
+
+
+def bench_gemm16(cfg, steps, warmup, vendor):
+    c = inputs.CONFIGS[cfg]
+    m, n, k = c["m"], c["n"], c["k"]
+    flops = inputs.algorithmic_work(cfg)
+    nsets = 4  # 130 MB per set
+    As = [ko.DeviceBuffer(m * k * 2) for _ in range(nsets)]
+    Bs = [ko.DeviceBuffer(k * n * 2) for _ in range(nsets)]
+    Ds = [ko.DeviceBuffer(m * n * 2) for _ in range(nsets)]
+    for a, b in zip(As, Bs):
+        ko.fill_uniform_16(a, m * k, inputs.tensor_seed(cfg, 0))
+        ko.fill_uniform_16(b, k * n, inputs.tensor_seed(cfg, 1))
+    wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
+    res = dict(workload=c["name"], metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
+               ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
+               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=None),
+               flops=flops, kernel_us=dev * 1e6)
+    if vendor is not None:
+        us, na = ctypes.c_float(), ctypes.c_int()
+        tmp = ko.DeviceBuffer(m * n * 2)
+        if vendor.kov_gemm16(m, n, k, As[0].ptr, Bs[0].ptr, 1, tmp.ptr, 0, 16, 20, ctypes.byref(us),
+                             ctypes.byref(na)) == 0:
+            res["hipblaslt_tflops"] = flops / us.value / 1e6
+            res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
+            ref = tmp.download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
+            got = Ds[0].download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
+            res["max_abs_diff_vs_hipblaslt"] = float(np.abs(got - ref).max())
+    return res, None
+
+
+def run_workload(cfg, steps, warmup, vendor):
+    op = inputs.CONFIGS[cfg]["op"]
+    if op == "softmax":
+        return bench_softmax(cfg, steps, warmup)
+    if op == "layernorm":
+        return bench_layernorm(cfg, steps, warmup)
+    if op == "sgemm":
+        return bench_sgemm(cfg, steps, warmup, vendor)
+    return bench_gemm16(cfg, steps, warmup, vendor)
+
+
+# ---------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline_softmax(keep, cfg):
+    """The CPU oracle (a port: the reference has no CPU softmax) on the first quarter of the rows the GPU
+    just processed, all host threads, best of 3; also checks the GPU rows against it."""
+    import oracle  # test infrastructure: used here as the timed CPU baseline and checker only
+    c = inputs.CONFIGS[cfg]
+    rows = keep["rows"] // 4
+    if keep["rps"]:
+        rows -= rows % keep["rps"]
+    cols = keep["cols"]
+    x = keep["x"].download(np.float32, (rows, cols))
+    y = keep["y"].download(np.float32, (rows, cols))
+    vl = keep["vl"].download(np.int32, (c["n_seq"],)) if keep["vl"] is not None else None
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ref = oracle.softmax(x, vl, keep["rps"])
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    d = np.abs(y.astype(np.float64) - ref)
+    sel = ref >= np.finfo(np.float32).tiny
+    parity = dict(rows_checked=rows, max_abs_err=float(d.max()), max_rel_err=float((d[sel] / ref[sel]).max()),
+                  gate="abs<=1e-6 and rel<=1e-5", ok=bool(d.max() <= 1e-6 and (d[sel] / ref[sel]).max() <= 1e-5))
+    return dict(value=2 * rows * cols * 4 / best / 1e9, unit="GB/s", cores=oracle.max_threads(), kind="port",
+                sample="first %d of %d rows (x %d cols) of the same device-resident input, best of 3; "
+                       "host cpus visible: %d" % (rows, keep["rows"], cols, os.cpu_count() or 0),
+                seconds=best), parity
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS))
+    ap.add_argument("--all", dest="all", action="store_true", default=True,
+                    help="also measure the other four configurations (default)")
+    ap.add_argument("--no-all", dest="all", action="store_false")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (every operator here shards by rows with no "
+                 "communication); run with --gpus 1")
+    ko.lib()
+    info = ko.device_info()  # raises without a GPU: there is no CPU fallback
+    vendor = _vendor()
+
+    cfg = WORKLOADS[args.workload]
+    head, keep = run_workload(cfg, args.steps, args.warmup, vendor)
+    cpu, parity = (None, None)
+    if not args.no_cpu and keep is not None:
+        cpu, parity = cpu_baseline_softmax(keep, cfg)
+    del keep
+
+    others = []
+    if args.all:
+        for other in sorted(inputs.CONFIGS):
+            if other == cfg:
+                continue
+            res, k2 = run_workload(other, args.steps, args.warmup, vendor)
+            del k2
+            others.append(res)
+
+    line = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic (seeded counter-based generator, filled on the device)",
+        "config": {"workload": head["workload"], "buffer_sets": head["buffer_sets"],
+                   "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
+        "roofline": head["roofline"], "cpu_baseline": cpu, "parity": parity,
+        "kernel_us": head["kernel_us"],
+        "workloads": others,
+    }
+    for key in ("hipblaslt_tflops", "vs_hipblaslt", "max_abs_diff_vs_hipblaslt"):
+        if key in head:
+            line[key] = head[key]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

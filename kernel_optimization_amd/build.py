@@ -62,6 +62,18 @@ def build_lib(jobs=4, verbose=False):
     return LIB_PATH
 
 
+def build_vendor(verbose=False):
+    """libko_vendor.so: hipBLASLt timed on the same buffers (comparison harness, not product)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    out_path = os.path.join(LIB_DIR, "libko_vendor.so")
+    out = _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-x", "hip",
+                f"--offload-arch={ARCH}", os.path.join(PKG, "vendor", "ko_vendor.cpp"), "-o", out_path,
+                "-lhipblaslt"])
+    if verbose and out.strip():
+        print(out)
+    return out_path
+
+
 def build_host(verbose=False):
     """Tensor + the three benchmark drivers: plain C++ (g++), linked against libko.so only."""
     if not os.path.isdir(HOST):
@@ -85,19 +97,22 @@ def build_host(verbose=False):
 
 def build_all(jobs=4, verbose=False):
     lib = build_lib(jobs=jobs, verbose=verbose)
+    vendor = build_vendor(verbose=verbose)
     host = build_host(verbose=verbose)
-    return lib, host
+    return lib, vendor, host
 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    ap.add_argument("--only", choices=["lib", "host"])
+    ap.add_argument("--only", choices=["lib", "host", "vendor"])
     ap.add_argument("-v", "--verbose", action="store_true")
     args = ap.parse_args(argv)
-    if args.only != "host":
+    if args.only in (None, "lib"):
         print("built", build_lib(args.jobs, args.verbose))
-    if args.only != "lib":
+    if args.only in (None, "vendor"):
+        print("built", build_vendor(args.verbose))
+    if args.only in (None, "host"):
         for exe in build_host(args.verbose):
             print("built", exe)
 

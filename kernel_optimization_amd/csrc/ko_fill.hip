@@ -153,16 +153,17 @@ KO_EXPORT int ko_copy_f32(const float *in, float *out, int64_t n, ko_stream_t st
     if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15)
         return ko::fail(KO_ERR_INVALID_ARGUMENT, "copy_f32: pointers must be 16-byte aligned");
     const int64_t nvec = n / 4;
-    int per_cu = ko::tuning("copy.blocks_per_cu");
-    if (per_cu <= 0) per_cu = 8;
-    int64_t grid = static_cast<int64_t>(ko::compute_units()) * per_cu;
     const int64_t needed = (nvec + 255) / 256 > 0 ? (nvec + 255) / 256 : 1;
-    if (grid > needed) grid = needed;
+    int64_t grid = needed;  // one vector per thread unless the knob caps the grid
+    const int per_cu = ko::tuning("copy.blocks_per_cu");
+    if (per_cu > 0 && grid > static_cast<int64_t>(ko::compute_units()) * per_cu)
+        grid = static_cast<int64_t>(ko::compute_units()) * per_cu;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     hipStream_t s = ko::as_stream(stream);
-    if (ko::tuning("copy.nontemporal") == 1)
-        ko::copy_f32_kernel<true><<<dim3(static_cast<unsigned>(grid)), 256, 0, s>>>(in, out, nvec, n);
-    else
+    if (ko::tuning("copy.nontemporal") == 2)
         ko::copy_f32_kernel<false><<<dim3(static_cast<unsigned>(grid)), 256, 0, s>>>(in, out, nvec, n);
+    else
+        ko::copy_f32_kernel<true><<<dim3(static_cast<unsigned>(grid)), 256, 0, s>>>(in, out, nvec, n);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }

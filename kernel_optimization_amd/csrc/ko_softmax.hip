@@ -233,10 +233,13 @@ int launch_wave(const Args &a) {
     constexpr int kThreads = 256;
     const int64_t rows_per_block = RPW * (kThreads / 64);
     const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
-    int per_cu = tuning("softmax.blocks_per_cu");
-    if (per_cu <= 0) per_cu = 8;
-    int64_t grid = static_cast<int64_t>(compute_units()) * per_cu;
-    if (grid > needed) grid = needed;
+    // One row batch per wavefront by default (measured faster than a persistent grid-stride
+    // launch: the hardware keeps more loads in flight); a positive knob caps the grid instead.
+    int64_t grid = needed;
+    const int per_cu = tuning("softmax.blocks_per_cu");
+    if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
+        grid = static_cast<int64_t>(compute_units()) * per_cu;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     softmax_wave_kernel<LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
     KO_CHECK_LAUNCH();
@@ -272,14 +275,13 @@ constexpr int kWaveMaxVpl = 8;
 constexpr int kWaveMaxCols = 64 * kWaveMaxVpl * 4;    // 2048
 constexpr int kBlockMaxCols = 1024 * 8 * 4;           // 32768
 
-// Lanes per row for the WARP policy: the widest group whose lanes each hold at least
-// two vectors (more bytes in flight per lane), never so narrow that a lane would
-// need more than kWaveMaxVpl vectors.
+// Lanes per row for the WARP policy: the narrowest group that gives every lane at most
+// one vector, so that one load instruction of the group covers the row contiguously;
+// rows longer than 64 vectors take the whole wavefront and several vectors per lane.
 int default_lanes_per_row(int cols) {
     const int nvec = cols / 4;
-    int lpr = 64;
-    while (lpr > 8 && nvec < 2 * lpr) lpr >>= 1;
-    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    int lpr = 8;
+    while (lpr < 64 && lpr < nvec) lpr <<= 1;
     return lpr;
 }
 
@@ -288,8 +290,9 @@ int launch_wave_any(const Args &a) {
     int lpr = tuning("softmax.lanes_per_row");
     if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(a.cols);
     while (lpr < 64 && (a.cols / 4 + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
-    if (tuning("softmax.nontemporal") == 1) return launch_wave_lpr<MASKED, true>(a, lpr);
-    return launch_wave_lpr<MASKED, false>(a, lpr);
+    // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off.
+    if (tuning("softmax.nontemporal") == 2) return launch_wave_lpr<MASKED, false>(a, lpr);
+    return launch_wave_lpr<MASKED, true>(a, lpr);
 }
 
 template <int THREADS, bool MASKED>

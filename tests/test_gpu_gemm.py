@@ -9,7 +9,7 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5]
-GEMM16_VARIANTS = [0, 1, 2, 3, 4, 5]
+GEMM16_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8]
 
 
 @pytest.fixture

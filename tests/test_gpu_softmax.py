@@ -37,7 +37,7 @@ def test_softmax_every_lane_mapping(ko, lpr, cols):
     ref = oracle.softmax(x)
     ko.set_tuning("softmax.lanes_per_row", lpr)
     try:
-        for nt in (0, 1):
+        for nt in (1, 2):  # streaming accesses on / off
             ko.set_tuning("softmax.nontemporal", nt)
             assert_softmax_close(ko.softmax_host(x), ref)
     finally:
