@@ -181,6 +181,20 @@ def bench_gemm16(cfg, steps, warmup, vendor):
     return res, None
 
 
+def bench_copy(steps, warmup, nbytes=1 << 30):
+    """Plain out[i] = in[i] copy of `nbytes` in and `nbytes` out: the practical ceiling of a read+write
+    stream on this device, and the calibration kernel for the HBM traffic counters."""
+    n = nbytes // 4
+    x, y = ko.DeviceBuffer(n * 4), ko.DeviceBuffer(n * 4)
+    ko.fill_uniform_f32(x, n, 1)
+    wall, dev = _time_steps(lambda i: ko.copy_f32(x, y, n), steps, warmup)
+    return dict(workload="copy_f32_%dMiB" % (nbytes >> 20), metric="hbm_gbytes_per_s", unit="GB/s",
+                value=2 * n * 4 / wall / 1e9, ms_per_step=wall * 1e3, dtype="f32", buffer_sets=1,
+                roofline=dict(bound="hbm", achieved=2 * n * 4 / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                              frac=2 * n * 4 / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
+                algorithmic_bytes=2 * n * 4, kernel_us=dev * 1e6)
+
+
 def run_workload(cfg, steps, warmup, vendor):
     op = inputs.CONFIGS[cfg]["op"]
     if op == "softmax":
@@ -195,11 +209,11 @@ def run_workload(cfg, steps, warmup, vendor):
 # ---------------------------------------------------------------------------- CPU baseline
 
 def cpu_baseline_softmax(keep, cfg):
-    """The CPU oracle (a port: the reference has no CPU softmax) on the first quarter of the rows the GPU
-    just processed, all host threads, best of 3; also checks the GPU rows against it."""
+    """The CPU oracle (a port: the reference has no CPU softmax) on the rows the GPU just processed, all
+    host threads, best of 3 (about 15-25 core-seconds in all); also checks the GPU rows against it."""
     import oracle  # test infrastructure: used here as the timed CPU baseline and checker only
     c = inputs.CONFIGS[cfg]
-    rows = keep["rows"] // 4
+    rows = keep["rows"]
     if keep["rps"]:
         rows -= rows % keep["rps"]
     cols = keep["cols"]
@@ -217,8 +231,8 @@ def cpu_baseline_softmax(keep, cfg):
     parity = dict(rows_checked=rows, max_abs_err=float(d.max()), max_rel_err=float((d[sel] / ref[sel]).max()),
                   gate="abs<=1e-6 and rel<=1e-5", ok=bool(d.max() <= 1e-6 and (d[sel] / ref[sel]).max() <= 1e-5))
     return dict(value=2 * rows * cols * 4 / best / 1e9, unit="GB/s", cores=oracle.max_threads(), kind="port",
-                sample="first %d of %d rows (x %d cols) of the same device-resident input, best of 3; "
-                       "host cpus visible: %d" % (rows, keep["rows"], cols, os.cpu_count() or 0),
+                sample="all %d rows x %d cols of the same device-resident input, %d threads, best of 3; "
+                       "host cpus visible: %d" % (rows, cols, oracle.max_threads(), os.cpu_count() or 0),
                 seconds=best), parity
 
 
@@ -227,7 +241,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS) + ["copy_f32"])
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
     ap.add_argument("--no-all", dest="all", action="store_false")
@@ -240,6 +254,9 @@ def main():
     info = ko.device_info()  # raises without a GPU: there is no CPU fallback
     vendor = _vendor()
 
+    if args.workload == "copy_f32":  # calibration run for the traffic counters
+        print(json.dumps(bench_copy(args.steps, args.warmup)))
+        return
     cfg = WORKLOADS[args.workload]
     head, keep = run_workload(cfg, args.steps, args.warmup, vendor)
     cpu, parity = (None, None)
@@ -248,7 +265,9 @@ def main():
     del keep
 
     others = []
+    copy = None
     if args.all:
+        copy = bench_copy(args.steps, args.warmup)
         for other in sorted(inputs.CONFIGS):
             if other == cfg:
                 continue
@@ -265,6 +284,8 @@ def main():
                    "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
         "roofline": head["roofline"], "cpu_baseline": cpu, "parity": parity,
         "kernel_us": head["kernel_us"],
+        "copy_ceiling": None if copy is None else {"GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"],
+                                                   "workload": copy["workload"]},
         "workloads": others,
     }
     for key in ("hipblaslt_tflops", "vs_hipblaslt", "max_abs_diff_vs_hipblaslt"):

@@ -1,0 +1,55 @@
+// LayerNorm: the reference's descriptor types (nn_operators/layernorm/layernorm.h:145-300)
+// and its kernel entry (:302-312) as host-side types over the C ABI.
+//
+// Reference:   layer_normalization<K><<<grid, block, K::smem_in_bytes, stream>>>(in, out, epsilon, gamma, beta);
+// Here:        layer_normalization<K>(grid, block, K::smem_in_bytes, stream, in, out, epsilon, gamma, beta);
+//
+// With K::elementwise_affine == false gamma and beta are not applied, as in the reference
+// (layernorm.h:189).  The extended overload also returns the per-row mean and rstd and
+// selects the variance denominator (N by default; N-1 is what layernorm.h:48 aims at).
+#ifndef KERNEL_OPTIMIZATION_LAYERNORM_H
+#define KERNEL_OPTIMIZATION_LAYERNORM_H
+
+#include <type_traits>
+
+#include "../../common/common.h"
+
+#define KO_LAYERNORM_DESCRIPTOR(NAME, POLICY, SMEM)                                                      \
+    template <typename _Element, int _vec_len, int _num_row, int _num_column, bool _elementwise_affine> \
+    struct NAME {                                                                                        \
+        using Element = _Element;                                                                        \
+        static const int vec_len = _vec_len;                                                             \
+        static const int num_row = _num_row;                                                             \
+        static const int num_column = _num_column;                                                       \
+        static const bool elementwise_affine = _elementwise_affine;                                      \
+        static const int smem_in_bytes = (SMEM);                                                         \
+        static const int policy = (POLICY);                                                              \
+        static_assert(_num_column % _vec_len == 0, "Unaligned vectorized access");                       \
+    }
+
+KO_LAYERNORM_DESCRIPTOR(LayerNormWarpImpl, KO_POLICY_WARP, 0);                                                 // :145-201
+KO_LAYERNORM_DESCRIPTOR(LayerNormBlockImpl, KO_POLICY_BLOCK,
+                        _num_column * sizeof(_Element) + 32 * 3 * sizeof(_Element));                            // :204-252
+KO_LAYERNORM_DESCRIPTOR(LayerNormBlockNoCacheImpl, KO_POLICY_BLOCK_NOCACHE, 32 * 3 * sizeof(_Element));         // :254-300
+#undef KO_LAYERNORM_DESCRIPTOR
+
+template <typename LayerNormKernel>
+void layer_normalization(int grid_dim, int block_dim, int smem_in_bytes, ko_stream_t stream,
+                         typename LayerNormKernel::Element *in_data, typename LayerNormKernel::Element *out_data,
+                         typename LayerNormKernel::Element epsilon,
+                         typename LayerNormKernel::Element *gamma = nullptr,
+                         typename LayerNormKernel::Element *beta = nullptr,
+                         typename LayerNormKernel::Element *mean = nullptr,
+                         typename LayerNormKernel::Element *rstd = nullptr, bool unbiased = false) {
+    static_assert(std::is_same<typename LayerNormKernel::Element, float>::value, "libko provides the fp32 LayerNorm");
+    (void)grid_dim;
+    (void)block_dim;
+    (void)smem_in_bytes;
+    const bool affine = LayerNormKernel::elementwise_affine;
+    checkKoErrors(ko_layernorm_f32_policy(in_data, out_data, mean, rstd, affine ? gamma : nullptr,
+                                          affine ? beta : nullptr, LayerNormKernel::num_row,
+                                          LayerNormKernel::num_column, epsilon, unbiased ? 1 : 0,
+                                          LayerNormKernel::policy, stream));
+}
+
+#endif  // KERNEL_OPTIMIZATION_LAYERNORM_H

@@ -1,0 +1,98 @@
+// LayerNorm benchmark driver: the counterpart of nn_operators/layernorm/main.cu
+// (run_benchmark :21-73, main :74-79) written against the C ABI.
+#include <cmath>
+#include <cstdio>
+
+#include "kernel_optimization/common/common.h"
+#include "kernel_optimization/common/random.h"
+#include "kernel_optimization/common/tensor.h"
+#include "kernel_optimization/nn_operators/layernorm/layernorm.h"
+
+template <int grid_dim, int block_dim, typename T, template <typename, int, int, int, bool> class LayerNorm,
+          int vec_len, int num_row, int num_column, bool affine>
+void run_benchmark(float epsilon) {
+    using LayerNormKernel = LayerNorm<T, vec_len, num_row, num_column, affine>;
+    const size_t count = static_cast<size_t>(num_row) * num_column;
+
+    Tensor in_data(count * sizeof(T));
+    Tensor out_data(count * sizeof(T));
+    Tensor gamma(num_column * sizeof(T)), beta(num_column * sizeof(T));
+    Tensor mean(num_row * sizeof(T)), rstd(num_row * sizeof(T));
+
+    ko_stream_t stream;
+    checkKoErrors(ko_stream_create(&stream));
+
+    for (size_t idx = 0; idx < count; ++idx)
+        in_data.template host_ref<T>()[idx] = T(ko_random::normal(ko_random::tensor_seed(2, 0), idx, 0.5, 2.0));
+    for (int c = 0; c < num_column; ++c) {
+        gamma.template host_ref<T>()[c] = T(ko_random::normal(ko_random::tensor_seed(2, 1), c, 1.0, 0.1));
+        beta.template host_ref<T>()[c] = T(ko_random::normal(ko_random::tensor_seed(2, 2), c, 0.0, 0.1));
+    }
+    in_data.host_to_device_async(stream);
+    gamma.host_to_device_async(stream);
+    beta.host_to_device_async(stream);
+    checkKoErrors(ko_stream_synchronize(stream));
+
+    ko_event_t _start, _stop;
+    checkKoErrors(ko_event_create(&_start));
+    checkKoErrors(ko_event_create(&_stop));
+
+    const int n_warm = 3, n_iter = 20;
+    auto launch = [&]() {
+        layer_normalization<LayerNormKernel>(grid_dim, block_dim, LayerNormKernel::smem_in_bytes, stream,
+                                             in_data.template device_ref<T>(), out_data.template device_ref<T>(),
+                                             epsilon, gamma.template device_ref<T>(), beta.template device_ref<T>(),
+                                             mean.template device_ref<T>(), rstd.template device_ref<T>());
+    };
+    for (int idx = 0; idx < n_warm; ++idx) launch();
+    checkKoErrors(ko_event_record(_start, stream));
+    for (int idx = 0; idx < n_iter; ++idx) launch();
+    checkKoErrors(ko_event_record(_stop, stream));
+    checkKoErrors(ko_event_synchronize(_stop));
+    float time_in_ms = 0;
+    checkKoErrors(ko_event_elapsed_ms(&time_in_ms, _start, _stop));
+
+    printf("======Num row %d, num column %d======\n", num_row, num_column);
+    printf("Average time %.2fms\n", time_in_ms / n_iter);
+    printf("Algorithmic bandwidth %.0f GB/s\n", 2.0 * count * sizeof(T) / (time_in_ms / n_iter * 1e-3) / 1e9);
+
+    // Sampled rows against a two-pass computation in double.
+    out_data.device_to_host_async(stream);
+    mean.device_to_host_async(stream);
+    rstd.device_to_host_async(stream);
+    checkKoErrors(ko_stream_synchronize(stream));
+    double worst = 0;
+    for (int r = 0; r < num_row; r += 509) {
+        const T *x = in_data.template host_ref<T>() + static_cast<size_t>(r) * num_column;
+        const T *y = out_data.template host_ref<T>() + static_cast<size_t>(r) * num_column;
+        double s = 0, m2 = 0;
+        for (int c = 0; c < num_column; ++c) s += x[c];
+        const double mu = s / num_column;
+        for (int c = 0; c < num_column; ++c) m2 += (x[c] - mu) * (x[c] - mu);
+        const double rs = 1.0 / std::sqrt(m2 / num_column + epsilon);
+        for (int c = 0; c < num_column; ++c) {
+            double ref = (x[c] - mu) * rs;
+            if (affine) ref = ref * gamma.template host_ref<T>()[c] + beta.template host_ref<T>()[c];
+            const double err = std::fabs(y[c] - ref) / (std::fabs(ref) > 1.0 ? std::fabs(ref) : 1.0);
+            worst = err > worst ? err : worst;
+        }
+        const double erstd = std::fabs(rstd.template host_ref<T>()[r] - rs) / rs;
+        worst = erstd > worst ? erstd : worst;
+    }
+    printf("max error over sampled rows: %.3g %s\n", worst, worst <= 1e-5 ? "Passed." : "FAILED");
+
+    checkKoErrors(ko_event_destroy(_start));
+    checkKoErrors(ko_event_destroy(_stop));
+    checkKoErrors(ko_stream_destroy(stream));
+    if (worst > 1e-5) exit(-1);
+}
+
+int main() {
+    // The reference's two runs (affine off, eps 1e-4; layernorm/main.cu:75-76) ...
+    run_benchmark<40 * 8, 128, float, LayerNormWarpImpl, 4, 128 * 128, 768, false>(0.0001f);
+    run_benchmark<40 * 16, 64, float, LayerNormBlockImpl, 4, 128 * 128, 768, false>(0.0001f);
+    // ... and the BERT-base hidden-state configuration with gamma/beta, eps 1e-5.
+    run_benchmark<40 * 8, 128, float, LayerNormWarpImpl, 4, 128 * 128, 768, true>(0.00001f);
+    run_benchmark<40 * 8, 128, float, LayerNormBlockNoCacheImpl, 4, 49152, 1024, true>(0.00001f);
+    return 0;
+}

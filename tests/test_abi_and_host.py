@@ -1,0 +1,139 @@
+"""CPU-side checks of the boundary: libko.so loads without a GPU and exports every symbol that
+include/ko.h declares; the ctypes table covers the same set; error paths that need no device; the
+C++ host layer (Tensor, descriptors, 16-bit types) builds with a plain C++ compiler and passes its
+self test."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import kernel_optimization_amd as ko
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "kernel_optimization_amd", "bin")
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ko.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ko_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 30
+    out = subprocess.run(["nm", "-D", "--defined-only", ko.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = set(re.findall(r"\sT\s+(ko_[a-z0-9_]+)", out))
+    assert set(names) <= exported, sorted(set(names) - exported)
+    assert exported <= set(names), "exported but not declared in ko.h: %s" % sorted(exported - set(names))
+    assert set(ko.SIGNATURES) == set(names)
+    lib = ko.lib()
+    for n in names:
+        getattr(lib, n)
+
+
+def test_header_is_plain_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "ko.h"\nint main(void) { return (int)KO_OK + (int)sizeof(ko_device_info_t) * 0; }\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), "-c",
+                    str(src), "-o", str(tmp_path / "t.o")], check=True)
+
+
+def test_status_names_and_argument_errors_without_device():
+    assert ko.status_name(0) == "KO_OK" and ko.status_name(2) == "KO_ERR_UNSUPPORTED_SHAPE"
+    lib = ko.lib()
+    # argument validation happens before anything touches the device
+    assert lib.ko_softmax_f32(None, None, 4, 130, None, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert "multiple of the vector width" in ko.last_error()
+    assert lib.ko_softmax_f32(None, None, -1, 128, None, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
+    assert lib.ko_layernorm_f32(None, None, None, None, None, None, 4, 770, 1e-5, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert lib.ko_sgemm_f32(-1, 1, 1, 1.0, None, None, 0.0, None, None, None) == ko.KO_ERR_INVALID_ARGUMENT
+    assert lib.ko_gemm_f16f32acc(8, 8, 12, 1.0, 1, 1, 1, 0.0, None, 1, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert lib.ko_set_tuning(b"no.such.knob", 1) == ko.KO_ERR_INVALID_ARGUMENT
+    ko.set_tuning("softmax.lanes_per_row", 16)
+    assert ko.get_tuning("softmax.lanes_per_row") == 16
+    ko.set_tuning("softmax.lanes_per_row", 0)
+    with pytest.raises(ko.KoError):
+        ko.check(ko.KO_ERR_RUNTIME)
+
+
+def test_no_cpu_fallback():
+    """Without a GPU the operators report an error: nothing is computed on the host."""
+    if ko.device_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax_host(np.zeros((4, 128), np.float32))
+    assert e.value.status in (ko.KO_ERR_NO_DEVICE, ko.KO_ERR_RUNTIME, ko.KO_ERR_OUT_OF_MEMORY)
+
+
+def test_host_layer_selftest(tmp_path):
+    exe = os.path.join(BIN, "host_selftest")
+    if not os.path.exists(exe):
+        from kernel_optimization_amd import build
+        build.build_host()
+    dump = tmp_path / "half.bin"
+    out = subprocess.run([exe, str(dump)], capture_output=True, text=True)
+    assert out.returncode == 0 and "host selftest ok" in out.stdout, out.stdout + out.stderr
+    d = np.fromfile(dump, dtype=np.dtype([("u", "<u4"), ("b", "<u2")]))
+    with np.errstate(over="ignore"):
+        want = d["u"].view(np.float32).astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(d["b"], want)  # ko_half(float) rounds like IEEE binary16
+
+
+def test_input_generators():
+    from kernel_optimization_amd import inputs
+    # splitmix64 known answers (seed 0: the published first outputs of the generator)
+    z = inputs.splitmix64(0, np.arange(3, dtype=np.uint64))
+    assert [int(v) for v in z] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+    x = inputs.normal_f64(200000, 7, 0.0, 1.0)
+    assert abs(x.mean()) < 0.01 and abs(x.std() - 1) < 0.01
+    u = inputs.uniform_f64(200000, 8, -1.0, 1.0)
+    assert u.min() >= -1 and u.max() < 1 and abs(u.mean()) < 0.01
+    np.testing.assert_array_equal(inputs.normal_f32((4, 8), 3)[2], inputs.normal_f64(8, 3, 0, 1, start=16).astype(np.float32))
+    vl = inputs.valid_lengths(4096, 9)
+    assert vl.min() >= 64 and vl.max() <= 512 and vl.max() > 500 and vl.min() < 76
+    assert inputs.algorithmic_work(1) == 201326592 and inputs.algorithmic_work(2) == 100800512
+    assert inputs.algorithmic_work(5) == 3221225472 and inputs.algorithmic_work(4) == 77309411328
+
+
+@pytest.mark.gpu
+def test_host_layer_on_gpu():
+    out = subprocess.run([os.path.join(BIN, "host_selftest"), "gpu"], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0 and "host selftest ok (with gpu)" in out.stdout, out.stdout + out.stderr
+
+
+@pytest.mark.gpu
+def test_gemm_driver_on_gpu():
+    """The GEMM driver prints the reference's lines and 'Passed.' for both paths."""
+    out = subprocess.run([os.path.join(BIN, "gemm")], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.count("Passed.") == 2
+    assert "======Problem size {1024,1024,1024} block shape: {64,64,8} warp shape {32,32,8}======" in out.stdout
+    assert "Average time" in out.stdout
+
+
+@pytest.mark.gpu
+def test_device_fill_matches_host_generator(ko):
+    from kernel_optimization_amd import inputs
+    n = 1 << 16
+    buf = ko.DeviceBuffer(n * 4)
+    ko.fill_uniform_f32(buf, n, 42, -1.0, 1.0)
+    ko.synchronize()
+    np.testing.assert_array_equal(buf.download(np.float32, (n,)), inputs.uniform_f32((n,), 42))
+    ko.fill_uniform_16(buf, n, 43, -1.0, 1.0, dtype=ko.F16)
+    ko.synchronize()
+    np.testing.assert_array_equal(buf.download(np.uint16, (n,)), inputs.uniform_f16((n,), 43).view(np.uint16))
+    ko.fill_uniform_16(buf, n, 44, -1.0, 1.0, dtype=ko.BF16)
+    ko.synchronize()
+    np.testing.assert_array_equal(buf.download(np.uint16, (n,)), inputs.uniform_bf16_bits((n,), 44))
+    ko.fill_lengths_i32(buf, 128, inputs.tensor_seed(5, 1), 64, 512)
+    ko.synchronize()
+    np.testing.assert_array_equal(buf.download(np.int32, (128,)), inputs.valid_lengths(128, inputs.tensor_seed(5, 1)))
+    ko.fill_normal_f32(buf, n, 45, 0.5, 2.0, first=1000)
+    ko.synchronize()
+    host = inputs.normal_f64(n, 45, 0.5, 2.0, start=1000).astype(np.float32)
+    dev = buf.download(np.float32, (n,))
+    assert np.all(np.abs(dev - host) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))  # libm vs device log/cos: <= 1 ulp
+    assert (dev != host).mean() < 0.01
