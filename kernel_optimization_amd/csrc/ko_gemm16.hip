@@ -102,15 +102,152 @@ struct Params {
     float alpha, beta;
     int tiles_n;
     int nblocks;
+    unsigned long long *trace;  // tuning aid: per-step timestamps of workgroup 0 (null in normal use)
 };
 
 // EDGE = false: M % BM == 0, N % BN == 0 and K % 64 == 0, so no load or store needs a bounds check.
+// Writes one wave's WTM x WTN accumulator tile to D (rows row0.., columns col0..).
+// acc[i][j][4q + e] is D[m][n] with m = 32i + lane % 32 and n = 32j + 8q + 4*(lane / 32) + e:
+// four consecutive columns per (i, j, q).  `region` is this wave's own piece of LDS, free for reuse.
+// The LDS transpose runs in PARTS passes over WTM / PARTS rows each, so that a wave needs
+// only WTM * WTN * 2 / PARTS bytes of LDS.
+template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1>
+__device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
+                                           int lane, int row0, int col0) {
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    const int M = p.M, N = p.N;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const float alpha = p.alpha, beta = p.beta;
+    const bool use_c = p.C != nullptr && beta != 0.0f;
+
+    if (!EDGE && !use_c) {
+        // Full tiles, no C: each wave transposes its own tile through LDS (free now: the last
+        // barrier of the K loop is behind every wave) and writes whole 16-byte chunks, a
+        // contiguous WTN*2-byte run per row.  8-byte units of a row are XOR-swizzled with the
+        // row index: the accumulator writes (32 consecutive rows, one unit) and the row reads
+        // (all chunks of a row) are then both free of bank conflicts; a chunk read from an odd
+        // row has its two units swapped.
+        constexpr int ROW_CHUNKS = WTN / 8;         // 16-byte chunks per row of the wave tile
+        constexpr int ROWS_PER_ITER = 64 / ROW_CHUNKS;
+        constexpr int SWZ = (2 * ROW_CHUNKS < 16 ? 2 * ROW_CHUNKS : 16) - 1;  // swizzle stays inside the row
+        // rows of WTN*2 = 128 bytes pair up into one 64-bank line: then the row pair index drives the swizzle
+        auto erow = [](int row) { return (SWIZZLE == 1 && WTN * 2 <= 128) ? (row >> 1) : row; };
+        constexpr int PTM = TM / PARTS;             // 32-row blocks per pass
+        constexpr int PROWS = WTM / PARTS;          // rows per pass
+        static_assert(TM % PARTS == 0, "");
+        u32x2 *region8 = reinterpret_cast<u32x2 *>(region);
+        const u32x4 *region16 = reinterpret_cast<const u32x4 *>(region8);
+        const int c = lane % ROW_CHUNKS;
+#pragma unroll
+        for (int part = 0; part < PARTS; ++part) {
+            if (part > 0) wave_lds_fence();  // the previous pass has read its rows
+#pragma unroll
+            for (int ii = 0; ii < PTM; ++ii) {
+                const int i = part * PTM + ii;
+                const int row = ii * 32 + frow;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int unit = j * 8 + 2 * q + fhalf;
+                        u32x2 o;
+                        o[0] = from_float<BF16>(alpha * acc[i][j][4 * q]) |
+                               (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 1])) << 16);
+                        o[1] = from_float<BF16>(alpha * acc[i][j][4 * q + 2]) |
+                               (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 3])) << 16);
+                        region8[row * (2 * ROW_CHUNKS) + (unit ^ (erow(row) & SWZ))] = o;
+                    }
+                }
+            }
+            wave_lds_fence();
+#pragma unroll
+            for (int it = 0; it < PROWS / ROWS_PER_ITER; ++it) {
+                const int row = it * ROWS_PER_ITER + lane / ROW_CHUNKS;
+                u32x4 v = region16[row * ROW_CHUNKS + (c ^ ((erow(row) & SWZ) >> 1))];
+                if (erow(row) & 1) v = u32x4{v[2], v[3], v[0], v[1]};
+                const int gm = row0 + part * PROWS + row;
+                const int gn = col0 + c * 8;
+                *reinterpret_cast<u32x4 *>(p.D + static_cast<int64_t>(gm) * N + gn) = v;
+            }
+        }
+        return;
+    }
+
+    const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = row0 + i * 32 + frow;
+        if (EDGE && m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = col0 + j * 32 + 8 * q + 4 * fhalf;
+                if (EDGE && n >= N) continue;
+                const int64_t off = static_cast<int64_t>(m) * N + n;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][4 * q + e];
+                if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
+                    if (use_c) {
+                        const u32x2 c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            v[e] += beta * to_float<BF16>(static_cast<uint16_t>(c2[e >> 1] >> ((e & 1) * 16)));
+                    }
+                    u32x2 o;
+                    o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
+                    o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
+                    *reinterpret_cast<u32x2 *>(p.D + off) = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e < N) {
+                            float t = v[e];
+                            if (use_c) t += beta * to_float<BF16>(p.C[off + e]);
+                            p.D[off + e] = from_float<BF16>(t);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Tiling of one kernel instantiation.
 // REG_STAGES = 2: global loads run two K tiles ahead (two sets of staging registers);
 // REG_STAGES = 1: one tile ahead.  FRAG_DB: fragments of the next K step are read into a
-// second register set while the MFMAs of the current step run.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int REG_STAGES, bool FRAG_DB, bool BF16, bool B_ROW_MAJOR,
-          bool EDGE>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Params p) {
+// second register set while the MFMAs of the current step run.  SWIZZLE selects the row
+// function XOR-ed into the chunk index of the LDS stages: 0 = row % 8 (conflict free for 8
+// consecutive rows when two rows share a bank line of 32 banks), 1 = (row / 2) % 8 (conflict
+// free for 16 consecutive rows on 64 banks, where two 128-byte rows make one bank line).
+// L2_AHEAD (direct-to-LDS kernels): every wave also touches, with one 4-byte load per lane, the
+// cache lines of the K tile that lies L2_AHEAD steps ahead, so that the first-touch miss of a
+// line is taken well before the load that fills LDS with it.
+// SCHED = 1 pins the order of the inner loop with scheduling-group directives: one fragment
+// read of the next K step after each of the first MFMAs of the current one.
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_, int L2_AHEAD_ = 0,
+          int SCHED_ = 0>
+struct Tiling {
+    static constexpr int L2_AHEAD = L2_AHEAD_;
+    static constexpr int SCHED = SCHED_;
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, REG_STAGES = REG_STAGES_;
+    static constexpr bool FRAG_DB = FRAG_DB_;
+    static constexpr int SWIZZLE = SWIZZLE_;
+    static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+};
+
+template <int SWIZZLE>
+__device__ __forceinline__ int swz(int row) {
+    if constexpr (SWIZZLE == 1) return (row >> 1) & 7;
+    else return row & 7;
+}
+
+template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
+__global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
+    constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N, REG_STAGES = T::REG_STAGES;
+    constexpr bool FRAG_DB = T::FRAG_DB;
+    constexpr int SWIZZLE = T::SWIZZLE;
     constexpr int THREADS = 64 * WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -138,6 +275,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
     // while the tile one step ahead waits to be written to LDS.
     u32x4 ra[REG_STAGES][A_ITERS], rb[REG_STAGES][B_ITERS];
 
+    // Full tiles: the address of a 16-byte chunk is a wave-uniform base (tile origin, step i
+    // and K tile: scalar registers) plus a per-lane byte offset that never changes, so the
+    // loads need one offset register instead of a 64-bit pointer each.
+    constexpr int ROWS_PER_ITER = THREADS / kChunks;  // rows covered by one load instruction of the workgroup
+    const uint32_t lane_off_a = static_cast<uint32_t>((tid / kChunks) * K + (tid % kChunks) * 8) * 2u;
+
     auto load_global = [&](int kt, auto slot) {
         constexpr int S = decltype(slot)::value;
         const int k0 = kt * kBK;
@@ -153,7 +296,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
                 if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.A + static_cast<int64_t>(gr) * K + kc);
                 ra[S][i] = v;
             } else {
-                ra[S][i] = *reinterpret_cast<const u32x4 *>(p.A + static_cast<int64_t>(gr) * K + kc);
+                const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + i * ROWS_PER_ITER) * K + k0);
+                ra[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
             }
         }
         if constexpr (!B_ROW_MAJOR) {
@@ -169,7 +313,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
                     if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.B + static_cast<int64_t>(gr) * K + kc);
                     rb[S][i] = v;
                 } else {
-                    rb[S][i] = *reinterpret_cast<const u32x4 *>(p.B + static_cast<int64_t>(gr) * K + kc);
+                    const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + i * ROWS_PER_ITER) * K + k0);
+                    rb[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
                 }
             }
         } else {
@@ -207,14 +352,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
         for (int i = 0; i < A_ITERS; ++i) {
             const int idx = tid + i * THREADS;
             const int row = idx / kChunks, c = idx % kChunks;
-            sa[row * kChunks + (c ^ (row & 7))] = ra[S][i];
+            sa[row * kChunks + (c ^ swz<SWIZZLE>(row))] = ra[S][i];
         }
         if constexpr (!B_ROW_MAJOR) {
 #pragma unroll
             for (int i = 0; i < B_ITERS; ++i) {
                 const int idx = tid + i * THREADS;
                 const int row = idx / kChunks, c = idx % kChunks;
-                sb[row * kChunks + (c ^ (row & 7))] = rb[S][i];
+                sb[row * kChunks + (c ^ swz<SWIZZLE>(row))] = rb[S][i];
             }
         } else {
             uint16_t *sb16 = reinterpret_cast<uint16_t *>(sb);
@@ -227,7 +372,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
                 for (int e = 0; e < 8; ++e) {
                     const int n = c * 8 + e;
                     const uint16_t h = static_cast<uint16_t>(rb[S][i][e >> 1] >> ((e & 1) * 16));
-                    const int chunk = (kr >> 3) ^ (n & 7);
+                    const int chunk = (kr >> 3) ^ swz<SWIZZLE>(n);
                     sb16[(n * kChunks + chunk) * 8 + (kr & 7)] = h;
                 }
             }
@@ -255,12 +400,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int row = wm * WTM + i * 32 + frow;
-                af[slot][i] = sa[row * kChunks + (chunk ^ (row & 7))];
+                af[slot][i] = sa[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const int row = wn * WTN + j * 32 + frow;
-                bf[slot][j] = sb[row * kChunks + (chunk ^ (row & 7))];
+                bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
             }
         };
         if constexpr (FRAG_DB) read_frags(0, 0);
@@ -303,102 +448,597 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_kernel(const Pa
         if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
     }
 
-    // Epilogue.  acc[i][j][4q + e] is D[m][n] with m = tile row (lane % 32) and
-    // n = 8q + 4*(lane / 32) + e: four consecutive columns per (i, j, q).
-    const float alpha = p.alpha, beta = p.beta;
-    const bool use_c = p.C != nullptr && beta != 0.0f;
+    store_tile<WTM, WTN, SWIZZLE, BF16, EDGE>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+}
 
-    if (!EDGE && !use_c) {
-        // Full tiles, no C: each wave transposes its own tile through LDS (free now: the last
-        // barrier of the K loop is behind every wave) and writes whole 16-byte chunks, a
-        // contiguous WTN*2-byte run per row.  8-byte units of a row are XOR-swizzled with the
-        // row index: the accumulator writes (32 consecutive rows, one unit) and the row reads
-        // (all chunks of a row) are then both free of bank conflicts; a chunk read from an odd
-        // row has its two units swapped.
-        constexpr int ROW_CHUNKS = WTN / 8;         // 16-byte chunks per row of the wave tile
-        constexpr int ROWS_PER_ITER = 64 / ROW_CHUNKS;
-        constexpr int SWZ = (2 * ROW_CHUNKS < 16 ? 2 * ROW_CHUNKS : 16) - 1;  // swizzle stays inside the row
-        static_assert(BM * BN * 2 <= 2 * STAGE * 16, "epilogue tile must fit the pipeline LDS");
-        u32x2 *region8 = reinterpret_cast<u32x2 *>(lds) + wave * (WTM * WTN / 4);
+// Direct-to-LDS variant for full tiles with K-contiguous operands (column-major B):
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS
+// (lane l of a wave-level load fills the l-th 16-byte slot after the wave-uniform LDS
+// base), so the staging registers and the ds_write instructions of the register pipeline
+// disappear.  The XOR swizzle is applied on the global side: the lane that fills slot
+// (row, p) fetches chunk p ^ swz(row) of that row, still one 128-byte segment per 8 lanes.
+// Each wave-level load covers 8 tile rows; wave w issues loads w, w + WAVES, ...
+// One K tile ahead is in flight while the current one is multiplied; a wave waits for its
+// own loads (vmcnt) before the barrier that publishes the stage.
+template <class T, bool BF16>
+__global__ __launch_bounds__(T::THREADS) void gemm16_dtl_kernel(const Params p) {
+    constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
+    constexpr bool FRAG_DB = T::FRAG_DB;
+    constexpr int SWIZZLE = T::SWIZZLE;
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_CHUNKS = BM * kChunks, B_CHUNKS = BN * kChunks;
+    constexpr int STAGE = A_CHUNKS + B_CHUNKS;
+    constexpr int A_LOADS = A_CHUNKS / 64 / WAVES, B_LOADS = B_CHUNKS / 64 / WAVES;  // per wave and K tile
+    static_assert(WAVES % 2 == 0 && A_CHUNKS % (64 * WAVES) == 0 && B_CHUNKS % (64 * WAVES) == 0, "");
+
+    extern __shared__ u32x4 lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int tile = xcd_remap(blockIdx.x, p.nblocks);
+    const int m0 = (tile / p.tiles_n) * BM;
+    const int n0 = (tile % p.tiles_n) * BN;
+    const int K = p.K;
+    const int KT = K / kBK;
+
+    // This lane's byte offset inside an 8-row group: row lane/8, chunk (lane%8) ^ swz(row).  The
+    // swizzle of row 8g + lane/8 depends on g only through its parity, which is the wave's.
+    const int row_in = lane >> 3;
+    const uint32_t lane_off =
+        static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<SWIZZLE>(8 * wave + row_in)) << 3)) * 2u;
+
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+
+    auto issue = [&](int kt, int stage) {
+        const int k0 = kt * kBK;
+        u32x4 *dst = lds + stage * STAGE;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int row = i * 32 + frow;
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + 64 * g), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + A_CHUNKS + 64 * g), 16, 0, 0);
+        }
+    };
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+
+    auto compute_tile = [&](int cur) {
+        const u32x4 *sa = lds + cur * STAGE;
+        const u32x4 *sb = sa + A_CHUNKS;
+        constexpr int SLOTS = FRAG_DB ? 2 : 1;
+        u32x4 af[SLOTS][TM], bf[SLOTS][TN];
+        auto read_frags = [&](int ks, int slot) {
+            const int chunk = 2 * ks + fhalf;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wm * WTM + i * 32 + frow;
+                af[slot][i] = sa[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int unit = j * 8 + 2 * q + fhalf;
-                    u32x2 o;
-                    o[0] = from_float<BF16>(alpha * acc[i][j][4 * q]) |
-                           (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 1])) << 16);
-                    o[1] = from_float<BF16>(alpha * acc[i][j][4 * q + 2]) |
-                           (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 3])) << 16);
-                    region8[row * (2 * ROW_CHUNKS) + (unit ^ (row & SWZ))] = o;
-                }
+                const int row = wn * WTN + j * 32 + frow;
+                bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
             }
-        }
-        wave_lds_fence();
-        const u32x4 *region16 = reinterpret_cast<const u32x4 *>(region8);
-        const int c = lane % ROW_CHUNKS;
+        };
+        if constexpr (FRAG_DB) read_frags(0, 0);
 #pragma unroll
-        for (int it = 0; it < WTM / ROWS_PER_ITER; ++it) {
-            const int row = it * ROWS_PER_ITER + lane / ROW_CHUNKS;
-            u32x4 v = region16[row * ROW_CHUNKS + (c ^ ((row & SWZ) >> 1))];
-            if (row & 1) v = u32x4{v[2], v[3], v[0], v[1]};
-            const int gm = m0 + wm * WTM + row;
-            const int gn = n0 + wn * WTN + c * 8;
-            *reinterpret_cast<u32x4 *>(p.D + static_cast<int64_t>(gm) * N + gn) = v;
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            if constexpr (FRAG_DB) {
+                if (ks + 1 < kBK / 16) read_frags(ks + 1, (ks + 1) & 1);
+            } else {
+                read_frags(ks, 0);
+            }
+            const int slot = FRAG_DB ? (ks & 1) : 0;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
         }
-        return;
-    }
+    };
 
-    const bool vec_ok = (N & 3) == 0;
+    issue(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) issue(kt + 1, cur ^ 1);
+        compute_tile(cur);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+    }
+    store_tile<WTM, WTN, SWIZZLE, BF16, false>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+}
+
+// Persistent form of the direct-to-LDS kernel: one workgroup per compute unit walks over
+// its tiles, and the K tiles of all of them form one stream through the two LDS stages.
+// While the last K tile of an output tile is multiplied, the first K tile of the next
+// output tile is already in flight into the other stage; the epilogue then transposes
+// through the stage that was just consumed (in two passes, half of LDS), and its global
+// stores drain while the next tile's main loop runs.
+template <class T, bool BF16>
+__global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Params p) {
+    constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
+    constexpr bool FRAG_DB = T::FRAG_DB;
+    constexpr int SWIZZLE = T::SWIZZLE;
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_CHUNKS = BM * kChunks, B_CHUNKS = BN * kChunks;
+    constexpr int STAGE = A_CHUNKS + B_CHUNKS;
+    constexpr int A_LOADS = A_CHUNKS / 64 / WAVES, B_LOADS = B_CHUNKS / 64 / WAVES;
+    constexpr int EPI_PARTS = (BM * BN * 2) / (STAGE * 16);  // passes so that the transpose fits one stage
+    static_assert(WAVES % 2 == 0 && A_CHUNKS % (64 * WAVES) == 0 && B_CHUNKS % (64 * WAVES) == 0, "");
+    static_assert(EPI_PARTS >= 1 && TM % EPI_PARTS == 0, "");
+
+    extern __shared__ u32x4 lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int K = p.K;
+    const int KT = K / kBK;
+    const int grid = gridDim.x;
+    const int my_tiles = (p.nblocks - static_cast<int>(blockIdx.x) + grid - 1) / grid;
+    const int total = my_tiles * KT;
+
+    const int row_in = lane >> 3;
+    const uint32_t lane_off =
+        static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<SWIZZLE>(8 * wave + row_in)) << 3)) * 2u;
+
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+
+    auto tile_origin = [&](int t, int &m0, int &n0) {
+        const int tile = xcd_remap(static_cast<int>(blockIdx.x) + grid * t, p.nblocks);
+        m0 = (tile / p.tiles_n) * BM;
+        n0 = (tile % p.tiles_n) * BN;
+    };
+
+    auto issue = [&](int step, int stage) {
+        const int t = step / KT, kt = step - t * KT;
+        int m0, n0;
+        tile_origin(t, m0, n0);
+        const int k0 = kt * kBK;
+        u32x4 *dst = lds + stage * STAGE;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm * WTM + i * 32 + frow;
-        if (EDGE && m >= M) continue;
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + 64 * g), 16, 0, 0);
+        }
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int i = 0; i < B_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + A_CHUNKS + 64 * g), 16, 0, 0);
+        }
+    };
+
+    // One 4-byte load per lane into a scratch corner of LDS: lane l of wave w touches the 128-byte
+    // line of row (BM + BN) / WAVES * w + l of the stage that `step` will load (A rows first, then B).
+    constexpr int L2_AHEAD = T::L2_AHEAD;
+    constexpr int TOUCH_ROWS = (BM + BN) / WAVES;   // rows a wave touches per K tile
+    constexpr int TOUCH_LOADS = TOUCH_ROWS / 64;
+    static_assert(L2_AHEAD == 0 || (TOUCH_ROWS % 64 == 0 && BM % TOUCH_ROWS == 0), "");
+    auto touch = [&](int step) {
+        const int t = step / KT, kt = step - t * KT;
+        int m0, n0;
+        tile_origin(t, m0, n0);
+        const int k0 = kt * kBK;
+        uint32_t *scratch = reinterpret_cast<uint32_t *>(lds + 2 * STAGE) + wave * 64;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * fhalf;
-                if (EDGE && n >= N) continue;
-                const int64_t off = static_cast<int64_t>(m) * N + n;
-                float v[4];
+        for (int i = 0; i < TOUCH_LOADS; ++i) {
+            const int r = TOUCH_ROWS * wave + 64 * i;  // first row of this load, wave-uniform
+            const uint16_t *base = r < BM ? p.A + static_cast<int64_t>(m0 + r) * K + k0
+                                          : p.B + static_cast<int64_t>(n0 + r - BM) * K + k0;
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + static_cast<int64_t>(lane) * K), (lptr_t)scratch, 4, 0, 0);
+        }
+    };
+
+    float16v acc[TM][TN];
+    auto clear_acc = [&]() {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][4 * q + e];
-                if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
-                    if (use_c) {
-                        const u32x2 c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            v[e] += beta * to_float<BF16>(static_cast<uint16_t>(c2[e >> 1] >> ((e & 1) * 16)));
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    };
+    clear_acc();
+
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+
+    auto compute_tile = [&](int cur) {
+        const u32x4 *sa = lds + cur * STAGE;
+        const u32x4 *sb = sa + A_CHUNKS;
+        constexpr int SLOTS = FRAG_DB ? 2 : 1;
+        u32x4 af[SLOTS][TM], bf[SLOTS][TN];
+        auto read_frags = [&](int ks, int slot) {
+            const int chunk = 2 * ks + fhalf;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wm * WTM + i * 32 + frow;
+                af[slot][i] = sa[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int row = wn * WTN + j * 32 + frow;
+                bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
+            }
+        };
+        if constexpr (FRAG_DB) read_frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            if constexpr (FRAG_DB) {
+                if (ks + 1 < kBK / 16) read_frags(ks + 1, (ks + 1) & 1);
+            } else {
+                read_frags(ks, 0);
+            }
+            const int slot = FRAG_DB ? (ks & 1) : 0;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
+            if constexpr (T::SCHED == 1 && FRAG_DB) {
+                // MFMA, read, MFMA, read, ... for the TM + TN reads of the next step, then the remaining MFMAs
+                constexpr int READS = TM + TN;
+                if (ks + 1 < kBK / 16) {
+                    // the reads go early in the step: two after each of the first MFMAs
+#pragma unroll
+                    for (int r = 0; r < READS / 2; ++r) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
                     }
-                    u32x2 o;
-                    o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
-                    o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
-                    *reinterpret_cast<u32x2 *>(p.D + off) = o;
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - READS / 2, 0);
                 } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (n + e < N) {
-                            float t = v[e];
-                            if (use_c) t += beta * to_float<BF16>(p.C[off + e]);
-                            p.D[off + e] = from_float<BF16>(t);
-                        }
-                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
                 }
             }
+        }
+    };
+
+    if (total == 0) return;
+    issue(0, 0);
+    if constexpr (L2_AHEAD > 0) {
+        for (int a = 1; a < L2_AHEAD && a < total; ++a) touch(a);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+    int kt = 0, t = 0;
+    for (int step = 0; step < total; ++step) {
+        const int cur = step & 1;
+        const bool tracing = p.trace != nullptr && blockIdx.x == 0 && lane == 0;
+        unsigned long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+        if (tracing) t0 = __builtin_amdgcn_s_memtime();
+        if (step + 1 < total) issue(step + 1, cur ^ 1);
+        bool touched = false;
+        if constexpr (L2_AHEAD > 0) {
+            if (step + L2_AHEAD < total) {
+                touch(step + L2_AHEAD);
+                touched = true;
+            }
+        }
+        compute_tile(cur);
+        if (tracing) t1 = __builtin_amdgcn_s_memtime();
+        // Loads complete in order: the touch loads are the youngest, so leaving them outstanding
+        // still guarantees that this step's LDS fills have landed.
+        if (touched) {
+            if constexpr (TOUCH_LOADS == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        if (tracing) t2 = __builtin_amdgcn_s_memtime();
+        lds_barrier();
+        if (tracing) {
+            t3 = __builtin_amdgcn_s_memtime();
+            unsigned long long *dst = p.trace + (static_cast<size_t>(wave) * 64 + step) * 4;
+            if (step < 64) {
+                dst[0] = t0;
+                dst[1] = t1;
+                dst[2] = t2;
+                dst[3] = t3;
+            }
+        }
+        if (++kt == KT) {
+            int m0, n0;
+            tile_origin(t, m0, n0);
+            // stage `cur` is free (every wave is past the barrier); stage cur^1 holds the next tile's first K tile
+            store_tile<WTM, WTN, SWIZZLE, BF16, false, EPI_PARTS>(
+                p, acc, lds + cur * STAGE + wave * (WTM * WTN / 8 / EPI_PARTS), lane, m0 + wm * WTM, n0 + wn * WTN);
+            clear_acc();
+            lds_barrier();  // the next step loads into stage `cur`
+            kt = 0;
+            ++t;
         }
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int REG_STAGES, bool FRAG_DB, bool BF16, bool B_ROW_MAJOR,
-          bool EDGE>
+// Second form of the persistent kernel, written to keep the inner loop's register needs small:
+// LDS holds [A stage 0][A stage 1][B stage 0][B stage 1]; the byte offset of a lane's fragment for
+// K step ks is precomputed once (4 registers for A, 4 for B: the swizzle term depends on the lane
+// only), and the stage, the 32-row block and the operand enter as immediate offsets of ds_read_b128.
+// The K loop is unrolled by two so that the stage is a compile-time constant.
+template <class T, bool BF16>
+__global__ __launch_bounds__(T::THREADS) void gemm16_persistent2_kernel(const Params p) {
+    constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int KS = kBK / 16;
+    constexpr int A_BYTES = BM * kBK * 2, B_BYTES = BN * kBK * 2;  // per stage
+    constexpr int A_LOADS = A_BYTES / 1024 / WAVES, B_LOADS = B_BYTES / 1024 / WAVES;
+    constexpr int EPI_PARTS = (BM * BN * 2) / (A_BYTES + B_BYTES);
+    static_assert(T::SWIZZLE == 1, "this kernel uses the 64-bank swizzle");
+    static_assert(WAVES % 2 == 0 && A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0, "");
+    static_assert(2 * A_BYTES + B_BYTES + (TN - 1) * 4096 < 65536 + 65536, "");
+    static_assert(EPI_PARTS >= 1 && TM % EPI_PARTS == 0, "");
+    static_assert((A_BYTES % (WAVES / 2 * (WTM * WTN * 2 / EPI_PARTS))) == 0 || true, "");
+
+    extern __shared__ u32x4 lds[];
+    char *const lds_bytes = reinterpret_cast<char *>(lds);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int K = p.K;
+    const int KT = K / kBK;
+    const int grid = gridDim.x;
+    const int my_tiles = (p.nblocks - static_cast<int>(blockIdx.x) + grid - 1) / grid;
+    const int total = my_tiles * KT;
+    if (total == 0) return;
+
+    const int row_in = lane >> 3;
+    const uint32_t lane_off =
+        static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<1>(8 * wave + row_in)) << 3)) * 2u;
+
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+
+    auto tile_origin = [&](int t, int &m0, int &n0) {
+        const int tile = xcd_remap(static_cast<int>(blockIdx.x) + grid * t, p.nblocks);
+        m0 = (tile / p.tiles_n) * BM;
+        n0 = (tile % p.tiles_n) * BN;
+    };
+
+    auto issue = [&](int step, int stage) {
+        const int t = step / KT, kt = step - t * KT;
+        int m0, n0;
+        tile_origin(t, m0, n0);
+        const int k0 = kt * kBK;
+        char *dst_a = lds_bytes + stage * A_BYTES;
+        char *dst_b = lds_bytes + 2 * A_BYTES + stage * B_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst_a + 1024 * g), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const int g = wave + WAVES * i;
+            const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst_b + 1024 * g), 16, 0, 0);
+        }
+    };
+
+    // Fragment addresses: row (lane % 32) of a 32-row block, chunk (2 ks + lane / 32) ^ swizzle(row).
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+    const int sw = (frow >> 1) & 7;  // 32-row blocks start at multiples of 16 rows: the swizzle sees only frow
+    uint32_t off_a[KS], off_b[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const uint32_t o = static_cast<uint32_t>(frow * 128 + (((2 * ks + fhalf) ^ sw) << 4));
+        off_a[ks] = o + wm * WTM * 128;
+        off_b[ks] = o + 2 * A_BYTES + wn * WTN * 128;
+    }
+
+    float16v acc[TM][TN];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    };
+    clear_acc();
+
+    auto compute_tile = [&](auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        u32x4 af[2][TM], bf[2][TN];
+        auto read_frags = [&](int ks, int slot) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[slot][i] = *reinterpret_cast<const u32x4 *>(lds_bytes + off_a[ks] + (S * A_BYTES + i * 4096));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bf[slot][j] = *reinterpret_cast<const u32x4 *>(lds_bytes + off_b[ks] + (S * B_BYTES + j * 4096));
+        };
+        read_frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + 1 < KS) read_frags(ks + 1, (ks + 1) & 1);
+            const int slot = ks & 1;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
+            if constexpr (T::SCHED == 1) {
+                constexpr int READS = TM + TN;
+                if (ks + 1 < KS) {
+#pragma unroll
+                    for (int r = 0; r < READS / 2; ++r) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - READS / 2, 0);
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+                }
+            }
+        }
+    };
+
+    // K tiles come in pairs (the launcher takes this kernel for an even number of K tiles only), so
+    // every output tile starts in stage 0 and the stage is a compile-time constant of each half step.
+    auto step_fn = [&](int step, auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        const bool tracing = p.trace != nullptr && blockIdx.x == 0 && lane == 0;
+        unsigned long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+        if (tracing) t0 = __builtin_amdgcn_s_memtime();
+        if (step + 1 < total) issue(step + 1, S ^ 1);
+        compute_tile(stage_c);
+        if (tracing) t1 = __builtin_amdgcn_s_memtime();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (tracing) t2 = __builtin_amdgcn_s_memtime();
+        lds_barrier();
+        if (tracing) {
+            t3 = __builtin_amdgcn_s_memtime();
+            unsigned long long *dst = p.trace + (static_cast<size_t>(wave) * 64 + step) * 4;
+            if (step < 64) {
+                dst[0] = t0;
+                dst[1] = t1;
+                dst[2] = t2;
+                dst[3] = t3;
+            }
+        }
+    };
+
+    issue(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+    int step = 0;
+    for (int t = 0; t < my_tiles; ++t) {
+        for (int kt = 0; kt < KT; kt += 2, step += 2) {
+            step_fn(step, std::integral_constant<int, 0>{});
+            step_fn(step + 1, std::integral_constant<int, 1>{});
+        }
+        int m0, n0;
+        tile_origin(t, m0, n0);
+        // Stage 1 was consumed last and is free; stage 0 already holds the next tile's first K tile.
+        // The transpose regions of the first half of the waves lie in stage 1's A part, those of the
+        // second half in its B part.
+        constexpr int REGION = WTM * WTN * 2 / EPI_PARTS;  // bytes per wave
+        static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
+        char *region = wave < WAVES / 2 ? lds_bytes + A_BYTES + wave * REGION
+                                        : lds_bytes + 2 * A_BYTES + B_BYTES + (wave - WAVES / 2) * REGION;
+        store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane, m0 + wm * WTM,
+                                                        n0 + wn * WTN);
+        clear_acc();
+        lds_barrier();  // the next step loads into stage 1
+    }
+}
+
+template <class T, bool BF16>
+int launch_persistent2(Params p, hipStream_t stream) {
+    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
+    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
+    auto kernel = gemm16_persistent2_kernel<T, BF16>;
+    static bool configured = false;
+    if (!configured) {
+        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        configured = true;
+    }
+    p.tiles_n = p.N / T::BN;
+    p.nblocks = (p.M / T::BM) * p.tiles_n;
+    int grid = compute_units() / 8 * 8;
+    if (grid > p.nblocks) grid = p.nblocks;
+    kernel<<<dim3(static_cast<unsigned>(grid)), dim3(T::THREADS), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <class T, bool BF16, bool B_ROW_MAJOR>
+int launch_persistent2_experimental(const Params &p, hipStream_t stream) {
+    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_persistent2<T, BF16>(p, stream);
+    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
+}
+
+template <class T, bool BF16>
+int launch_persistent(Params p, hipStream_t stream) {
+    // two stages plus 256 bytes per wave of scratch for the cache-line touches
+    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t) + (T::L2_AHEAD > 0 ? T::THREADS * 4 : 0);
+    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the persistent variant needs full tiles");
+    auto kernel = gemm16_persistent_kernel<T, BF16>;
+    static bool configured = false;
+    if (!configured) {
+        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        configured = true;
+    }
+    p.tiles_n = p.N / T::BN;
+    p.nblocks = (p.M / T::BM) * p.tiles_n;
+    int grid = compute_units() / 8 * 8;  // a multiple of the XCD count keeps a workgroup's tiles on its XCD's band
+    if (grid > p.nblocks) grid = p.nblocks;
+    kernel<<<dim3(static_cast<unsigned>(grid)), dim3(T::THREADS), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <class T, bool BF16, bool B_ROW_MAJOR>
+int launch_persistent_experimental(const Params &p, hipStream_t stream) {
+    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_persistent<T, BF16>(p, stream);
+    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
+}
+
+template <class T, bool BF16>
+int launch_dtl(Params p, hipStream_t stream) {
+    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
+    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the direct-to-LDS variant needs full tiles");
+    auto kernel = gemm16_dtl_kernel<T, BF16>;
+    static bool configured = false;
+    if (!configured) {
+        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        configured = true;
+    }
+    p.tiles_n = p.N / T::BN;
+    p.nblocks = (p.M / T::BM) * p.tiles_n;
+    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(T::THREADS), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+template <class T, bool BF16, bool B_ROW_MAJOR>
+int launch_dtl_experimental(const Params &p, hipStream_t stream) {
+    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_dtl<T, BF16>(p, stream);
+    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
+}
+
+template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
 int launch_edge(const Params &p, hipStream_t stream) {
-    constexpr int THREADS = 64 * WAVES_M * WAVES_N;
-    constexpr size_t lds_bytes = 2u * (BM + BN) * kBK * sizeof(uint16_t);
-    auto kernel = gemm16_kernel<BM, BN, WAVES_M, WAVES_N, REG_STAGES, FRAG_DB, BF16, B_ROW_MAJOR, EDGE>;
+    constexpr int THREADS = T::THREADS;
+    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
+    auto kernel = gemm16_kernel<T, BF16, B_ROW_MAJOR, EDGE>;
     static bool configured = false;  // per instantiation
     if (!configured) {
         KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -410,39 +1050,72 @@ int launch_edge(const Params &p, hipStream_t stream) {
     return KO_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int REG_STAGES, bool FRAG_DB, bool BF16, bool B_ROW_MAJOR>
+template <class T, bool BF16, bool B_ROW_MAJOR>
 int launch(Params p, hipStream_t stream) {
-    const int tiles_m = (p.M + BM - 1) / BM;
-    p.tiles_n = (p.N + BN - 1) / BN;
+    const int tiles_m = (p.M + T::BM - 1) / T::BM;
+    p.tiles_n = (p.N + T::BN - 1) / T::BN;
     p.nblocks = tiles_m * p.tiles_n;
-    const bool edge = (p.M % BM) != 0 || (p.N % BN) != 0 || (p.K % kBK) != 0;
-    if (edge) return launch_edge<BM, BN, WAVES_M, WAVES_N, REG_STAGES, FRAG_DB, BF16, B_ROW_MAJOR, true>(p, stream);
-    return launch_edge<BM, BN, WAVES_M, WAVES_N, REG_STAGES, FRAG_DB, BF16, B_ROW_MAJOR, false>(p, stream);
+    const bool edge = (p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0;
+    if (edge) return launch_edge<T, BF16, B_ROW_MAJOR, true>(p, stream);
+    return launch_edge<T, BF16, B_ROW_MAJOR, false>(p, stream);
 }
+
+// Variants that exist for tuning only are built for the binary16, column-major-B case.
+template <class T, bool BF16, bool B_ROW_MAJOR>
+int launch_experimental(const Params &p, hipStream_t stream) {
+    if constexpr (!BF16 && !B_ROW_MAJOR) return launch<T, BF16, B_ROW_MAJOR>(p, stream);
+    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
+}
+
+using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 128x64
+using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
 
 template <bool BF16, bool B_ROW_MAJOR>
 int launch_variant(const Params &p, hipStream_t stream) {
-    int variant = tuning("gemm16.variant");
+    const int variant = tuning("gemm16.variant");
     if (variant <= 0) {
-        // Large problems: 256x256 tiles; small ones: 128x128 so that the grid still fills the chip.
+        // Enough 256x256 tiles to fill the chip: the big tiling - as the persistent direct-to-LDS kernel
+        // when the tiles are full and both operands are K-contiguous, else as the register pipeline.
+        // Fewer: 128x128 tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
-        variant = big_tiles >= compute_units() ? 6 : 3;
+        if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+        if constexpr (!B_ROW_MAJOR) {
+            if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) return launch_persistent<TileBig, BF16>(p, stream);
+        }
+        return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
     }
-    switch (variant) {
-        case 1: return launch<256, 256, 2, 2, 1, true, BF16, B_ROW_MAJOR>(p, stream);
-        case 2: return launch<256, 256, 2, 4, 2, false, BF16, B_ROW_MAJOR>(p, stream);
-        case 3: return launch<128, 128, 2, 2, 2, true, BF16, B_ROW_MAJOR>(p, stream);
-        case 4: return launch<256, 128, 2, 2, 2, true, BF16, B_ROW_MAJOR>(p, stream);
-        case 5: return launch<128, 256, 2, 2, 2, true, BF16, B_ROW_MAJOR>(p, stream);
-        case 6: return launch<256, 256, 2, 4, 1, true, BF16, B_ROW_MAJOR>(p, stream);
-        case 7: return launch<256, 256, 4, 2, 2, false, BF16, B_ROW_MAJOR>(p, stream);
-        case 8: return launch<256, 128, 2, 4, 2, true, BF16, B_ROW_MAJOR>(p, stream);
+    switch (variant) {  // explicit choices, for tuning and for the tests
+        case 3: return launch<Tiling<128, 128, 2, 2, 2, true, 0>, BF16, B_ROW_MAJOR>(p, stream);
+        case 6: return launch<Tiling<256, 256, 2, 4, 1, true, 0>, BF16, B_ROW_MAJOR>(p, stream);
+        case 9: return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
+        case 10: return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+        case 20: return launch_dtl_experimental<TileBig, BF16, B_ROW_MAJOR>(p, stream);
+        case 23: return launch_dtl_experimental<Tiling<256, 256, 4, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
+        case 30:
+            if constexpr (!B_ROW_MAJOR) return launch_persistent<TileBig, BF16>(p, stream);
+            else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: the persistent variant needs column-major B");
+        case 31: return launch_persistent_experimental<Tiling<256, 256, 4, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
+        case 36: return launch_persistent_experimental<Tiling<256, 256, 2, 4, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
+        case 41: return launch_persistent2_experimental<Tiling<256, 256, 2, 4, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
+        case 42: return launch_persistent2_experimental<Tiling<256, 256, 4, 2, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
 
 }  // namespace
 }  // namespace ko
+
+namespace ko {
+namespace {
+unsigned long long *g_trace = nullptr;
+}
+}  // namespace ko
+
+// Tuning aid (not declared in ko.h): device buffer of 8 * 64 * 4 uint64 that the persistent
+// kernels fill with per-step timestamps of workgroup 0, or null to switch tracing off.
+extern "C" __attribute__((visibility("default"))) void ko_internal_gemm16_trace(void *buf) {
+    ko::g_trace = static_cast<unsigned long long *>(buf);
+}
 
 KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
                                 const void *B, int b_layout, float beta, const void *C, void *D,
@@ -465,7 +1138,7 @@ KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, co
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: C and D must be 8-byte aligned");
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
-             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0};
+             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, g_trace};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);

@@ -9,7 +9,7 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5]
-GEMM16_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8]
+GEMM16_VARIANTS = [0, 3, 6, 9, 10, 20, 23, 30, 31, 36, 41, 42]
 
 
 @pytest.fixture
@@ -97,14 +97,66 @@ def _to_f64(bits, bf16):
 @pytest.mark.parametrize("gemm16_variant", GEMM16_VARIANTS, indirect=True)
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("b_col_major", [True, False])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768), (512, 768, 192)])
 def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
+    if gemm16_variant not in (0, 3, 6, 9, 10, 30) and (bf16 or not b_col_major):
+        pytest.skip("tuning variants are built for f16 with column-major B only")
+    if gemm16_variant == 30 and not b_col_major:
+        pytest.skip("the persistent kernel takes column-major B")
+    if gemm16_variant >= 20 and (m % 256 or n % 256 or k % 64):
+        pytest.skip("the direct-to-LDS variants take full tiles only")
+    if gemm16_variant >= 40 and k % 128:
+        pytest.skip("this persistent variant takes an even number of K tiles")
     A = _bits16((m, k), 21 + m, bf16)
     B = _bits16((n, k) if b_col_major else (k, n), 23 + n, bf16)
     _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16)
     got = ko.gemm16_host(A, B, m, n, k, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR,
                          dtype=ko.BF16 if bf16 else ko.F16)
     assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+
+
+@pytest.mark.parametrize("m,n,k", [(8192, 4096, 192), (2048, 1024, 64), (16384, 3072, 768)])
+def test_gemm16_variants_agree_bitwise(ko, m, n, k):
+    """Every tiling accumulates in the same K order with the same matrix instruction, so all variants
+    must give the same bits; the persistent variants walk several tiles per workgroup here (and an odd
+    number of K tiles, which flips the LDS stage parity from tile to tile).  Sampled rows also go
+    against the oracle."""
+    dA, dB = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2)
+    ko.fill_uniform_16(dA, m * k, 77)
+    ko.fill_uniform_16(dB, n * k, 78)
+    outs = {}
+    try:
+        for v in GEMM16_VARIANTS[1:]:
+            if v >= 40 and k % 128:
+                continue
+            ko.set_tuning("gemm16.variant", v)
+            dD = ko.DeviceBuffer(m * n * 2)
+            ko.gemm16(m, n, k, dA, dB, dD)
+            ko.synchronize()
+            outs[v] = dD.download(np.uint16, (m, n))
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+    base = outs[3]
+    for v, d in outs.items():
+        np.testing.assert_array_equal(d, base, err_msg="variant %d differs from variant 3" % v)
+    idx = np.sort(np.random.default_rng(3).choice(m, 48, replace=False))
+    A = dA.download(np.uint16, (m, k))[idx]
+    B = dB.download(np.uint16, (n, k))
+    _, ref64, ap = oracle.gemm16(A, B, len(idx), n, k)
+    assert_gemm16_close(oracle.f16_to_f64(base[idx]), ref64, ap, k)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm16_default_path_big(ko, bf16):
+    """Large enough for the default dispatch to take the persistent direct-to-LDS kernel (512 tiles of
+    256 x 256, 5 K tiles: several tiles per workgroup, odd K-tile count), both 16-bit types."""
+    m, n, k = 8192, 4096, 320
+    A = _bits16((m, k), 31, bf16)
+    B = _bits16((n, k), 32, bf16)
+    got = ko.gemm16_host(A, B, m, n, k, dtype=ko.BF16 if bf16 else ko.F16)
+    idx = np.sort(np.random.default_rng(4).choice(m, 64, replace=False))
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, bf16=bf16)
+    assert_gemm16_close(_to_f64(got[idx], bf16), ref64, ap, k, bf16=bf16)
 
 
 def test_gemm16_odd_n(ko):
