@@ -32,6 +32,7 @@
 #include "ko_internal.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace ko {
 namespace {
@@ -102,8 +103,28 @@ struct Params {
     float alpha, beta;
     int tiles_n;
     int nblocks;
-    unsigned long long *trace;  // tuning aid: per-step timestamps of workgroup 0 (null in normal use)
+    int band_rows;              // persistent kernels: > 0 selects the blocked tile order (see tile_of)
+    int block_cols;
 };
+
+// Persistent kernels: tile number t (0, 1, ...) of workgroup b when the grid has `grid` workgroups.
+// Workgroup b runs on XCD b % 8 and is the (b / 8)-th of the workgroups there.  With band_rows > 0
+// each XCD owns band_rows consecutive rows of tiles and walks them in blocks of block_cols columns:
+// the workgroups that are resident on one XCD at a time cover a band_rows x block_cols block of
+// tiles, the most compact footprint (fewest distinct A and B panels) their shared L2 can be given,
+// and the A panels of the band are reused from block to block.  Otherwise tiles are dealt in
+// row-major order from one contiguous range per XCD.
+__device__ __forceinline__ void tile_of(const Params &p, int b, int grid, int t, int &tile_m, int &tile_n) {
+    if (p.band_rows > 0) {
+        const int x = b & 7, j = b >> 3;
+        tile_m = x * p.band_rows + j % p.band_rows;
+        tile_n = t * p.block_cols + j / p.band_rows;
+    } else {
+        const int tile = xcd_remap(b + grid * t, p.nblocks);
+        tile_m = tile / p.tiles_n;
+        tile_n = tile % p.tiles_n;
+    }
+}
 
 // EDGE = false: M % BM == 0, N % BN == 0 and K % 64 == 0, so no load or store needs a bounds check.
 // Writes one wave's WTM x WTN accumulator tile to D (rows row0.., columns col0..).
@@ -221,16 +242,8 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 // function XOR-ed into the chunk index of the LDS stages: 0 = row % 8 (conflict free for 8
 // consecutive rows when two rows share a bank line of 32 banks), 1 = (row / 2) % 8 (conflict
 // free for 16 consecutive rows on 64 banks, where two 128-byte rows make one bank line).
-// L2_AHEAD (direct-to-LDS kernels): every wave also touches, with one 4-byte load per lane, the
-// cache lines of the K tile that lies L2_AHEAD steps ahead, so that the first-touch miss of a
-// line is taken well before the load that fills LDS with it.
-// SCHED = 1 pins the order of the inner loop with scheduling-group directives: one fragment
-// read of the next K step after each of the first MFMAs of the current one.
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_, int L2_AHEAD_ = 0,
-          int SCHED_ = 0>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_>
 struct Tiling {
-    static constexpr int L2_AHEAD = L2_AHEAD_;
-    static constexpr int SCHED = SCHED_;
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, REG_STAGES = REG_STAGES_;
     static constexpr bool FRAG_DB = FRAG_DB_;
     static constexpr int SWIZZLE = SWIZZLE_;
@@ -261,7 +274,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets address math run on the scalar unit
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     const int tile = xcd_remap(blockIdx.x, p.nblocks);
@@ -451,7 +464,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
     store_tile<WTM, WTN, SWIZZLE, BF16, EDGE>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
 }
 
-// Direct-to-LDS variant for full tiles with K-contiguous operands (column-major B):
+// Direct-to-LDS kernels for full tiles with K-contiguous operands (column-major B):
 // global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS
 // (lane l of a wave-level load fills the l-th 16-byte slot after the wave-uniform LDS
 // base), so the staging registers and the ds_write instructions of the register pipeline
@@ -460,116 +473,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
 // Each wave-level load covers 8 tile rows; wave w issues loads w, w + WAVES, ...
 // One K tile ahead is in flight while the current one is multiplied; a wave waits for its
 // own loads (vmcnt) before the barrier that publishes the stage.
-template <class T, bool BF16>
-__global__ __launch_bounds__(T::THREADS) void gemm16_dtl_kernel(const Params p) {
-    constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
-    constexpr bool FRAG_DB = T::FRAG_DB;
-    constexpr int SWIZZLE = T::SWIZZLE;
-    constexpr int WAVES = WAVES_M * WAVES_N;
-    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-    constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int A_CHUNKS = BM * kChunks, B_CHUNKS = BN * kChunks;
-    constexpr int STAGE = A_CHUNKS + B_CHUNKS;
-    constexpr int A_LOADS = A_CHUNKS / 64 / WAVES, B_LOADS = B_CHUNKS / 64 / WAVES;  // per wave and K tile
-    static_assert(WAVES % 2 == 0 && A_CHUNKS % (64 * WAVES) == 0 && B_CHUNKS % (64 * WAVES) == 0, "");
-
-    extern __shared__ u32x4 lds[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    const int tile = xcd_remap(blockIdx.x, p.nblocks);
-    const int m0 = (tile / p.tiles_n) * BM;
-    const int n0 = (tile % p.tiles_n) * BN;
-    const int K = p.K;
-    const int KT = K / kBK;
-
-    // This lane's byte offset inside an 8-row group: row lane/8, chunk (lane%8) ^ swz(row).  The
-    // swizzle of row 8g + lane/8 depends on g only through its parity, which is the wave's.
-    const int row_in = lane >> 3;
-    const uint32_t lane_off =
-        static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<SWIZZLE>(8 * wave + row_in)) << 3)) * 2u;
-
-    typedef const __attribute__((address_space(1))) void *gptr_t;
-    typedef __attribute__((address_space(3))) void *lptr_t;
-
-    auto issue = [&](int kt, int stage) {
-        const int k0 = kt * kBK;
-        u32x4 *dst = lds + stage * STAGE;
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            const int g = wave + WAVES * i;
-            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * g) * K + k0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + 64 * g), 16, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) {
-            const int g = wave + WAVES * i;
-            const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + A_CHUNKS + 64 * g), 16, 0, 0);
-        }
-    };
-
-    float16v acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    const int frow = lane & 31;
-    const int fhalf = lane >> 5;
-
-    auto compute_tile = [&](int cur) {
-        const u32x4 *sa = lds + cur * STAGE;
-        const u32x4 *sb = sa + A_CHUNKS;
-        constexpr int SLOTS = FRAG_DB ? 2 : 1;
-        u32x4 af[SLOTS][TM], bf[SLOTS][TN];
-        auto read_frags = [&](int ks, int slot) {
-            const int chunk = 2 * ks + fhalf;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int row = wm * WTM + i * 32 + frow;
-                af[slot][i] = sa[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int row = wn * WTN + j * 32 + frow;
-                bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
-            }
-        };
-        if constexpr (FRAG_DB) read_frags(0, 0);
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            if constexpr (FRAG_DB) {
-                if (ks + 1 < kBK / 16) read_frags(ks + 1, (ks + 1) & 1);
-            } else {
-                read_frags(ks, 0);
-            }
-            const int slot = FRAG_DB ? (ks & 1) : 0;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
-        }
-    };
-
-    issue(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    lds_barrier();
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) issue(kt + 1, cur ^ 1);
-        compute_tile(cur);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        lds_barrier();
-    }
-    store_tile<WTM, WTN, SWIZZLE, BF16, false>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
-}
-
-// Persistent form of the direct-to-LDS kernel: one workgroup per compute unit walks over
+//
+// Persistent form: one workgroup per compute unit walks over
 // its tiles, and the K tiles of all of them form one stream through the two LDS stages.
 // While the last K tile of an output tile is multiplied, the first K tile of the next
 // output tile is already in flight into the other stage; the epilogue then transposes
@@ -594,7 +499,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets address math run on the scalar unit
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int K = p.K;
     const int KT = K / kBK;
@@ -632,27 +537,6 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
             const int g = wave + WAVES * i;
             const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
             __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst + A_CHUNKS + 64 * g), 16, 0, 0);
-        }
-    };
-
-    // One 4-byte load per lane into a scratch corner of LDS: lane l of wave w touches the 128-byte
-    // line of row (BM + BN) / WAVES * w + l of the stage that `step` will load (A rows first, then B).
-    constexpr int L2_AHEAD = T::L2_AHEAD;
-    constexpr int TOUCH_ROWS = (BM + BN) / WAVES;   // rows a wave touches per K tile
-    constexpr int TOUCH_LOADS = TOUCH_ROWS / 64;
-    static_assert(L2_AHEAD == 0 || (TOUCH_ROWS % 64 == 0 && BM % TOUCH_ROWS == 0), "");
-    auto touch = [&](int step) {
-        const int t = step / KT, kt = step - t * KT;
-        int m0, n0;
-        tile_origin(t, m0, n0);
-        const int k0 = kt * kBK;
-        uint32_t *scratch = reinterpret_cast<uint32_t *>(lds + 2 * STAGE) + wave * 64;
-#pragma unroll
-        for (int i = 0; i < TOUCH_LOADS; ++i) {
-            const int r = TOUCH_ROWS * wave + 64 * i;  // first row of this load, wave-uniform
-            const uint16_t *base = r < BM ? p.A + static_cast<int64_t>(m0 + r) * K + k0
-                                          : p.B + static_cast<int64_t>(n0 + r - BM) * K + k0;
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + static_cast<int64_t>(lane) * K), (lptr_t)scratch, 4, 0, 0);
         }
     };
 
@@ -701,67 +585,20 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
-            if constexpr (T::SCHED == 1 && FRAG_DB) {
-                // MFMA, read, MFMA, read, ... for the TM + TN reads of the next step, then the remaining MFMAs
-                constexpr int READS = TM + TN;
-                if (ks + 1 < kBK / 16) {
-                    // the reads go early in the step: two after each of the first MFMAs
-#pragma unroll
-                    for (int r = 0; r < READS / 2; ++r) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - READS / 2, 0);
-                } else {
-                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
-                }
-            }
         }
     };
 
     if (total == 0) return;
     issue(0, 0);
-    if constexpr (L2_AHEAD > 0) {
-        for (int a = 1; a < L2_AHEAD && a < total; ++a) touch(a);
-    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
     int kt = 0, t = 0;
     for (int step = 0; step < total; ++step) {
         const int cur = step & 1;
-        const bool tracing = p.trace != nullptr && blockIdx.x == 0 && lane == 0;
-        unsigned long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-        if (tracing) t0 = __builtin_amdgcn_s_memtime();
         if (step + 1 < total) issue(step + 1, cur ^ 1);
-        bool touched = false;
-        if constexpr (L2_AHEAD > 0) {
-            if (step + L2_AHEAD < total) {
-                touch(step + L2_AHEAD);
-                touched = true;
-            }
-        }
         compute_tile(cur);
-        if (tracing) t1 = __builtin_amdgcn_s_memtime();
-        // Loads complete in order: the touch loads are the youngest, so leaving them outstanding
-        // still guarantees that this step's LDS fills have landed.
-        if (touched) {
-            if constexpr (TOUCH_LOADS == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-        if (tracing) t2 = __builtin_amdgcn_s_memtime();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
-        if (tracing) {
-            t3 = __builtin_amdgcn_s_memtime();
-            unsigned long long *dst = p.trace + (static_cast<size_t>(wave) * 64 + step) * 4;
-            if (step < 64) {
-                dst[0] = t0;
-                dst[1] = t1;
-                dst[2] = t2;
-                dst[3] = t3;
-            }
-        }
         if (++kt == KT) {
             int m0, n0;
             tile_origin(t, m0, n0);
@@ -776,13 +613,48 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
     }
 }
 
-// Second form of the persistent kernel, written to keep the inner loop's register needs small:
-// LDS holds [A stage 0][A stage 1][B stage 0][B stage 1]; the byte offset of a lane's fragment for
-// K step ks is precomputed once (4 registers for A, 4 for B: the swizzle term depends on the lane
-// only), and the stage, the 32-row block and the operand enter as immediate offsets of ds_read_b128.
-// The K loop is unrolled by two so that the stage is a compile-time constant.
+// Persistent direct-to-LDS kernel with a pinned inner loop.  LDS holds
+// [A stage 0][A stage 1][B stage 0][B stage 1]; the byte offset of a lane's fragment for K step ks
+// is precomputed once (4 registers for A, 4 for B: the swizzle term depends on the lane only), and
+// the stage, the 32-row block and the operand enter as immediate offsets of ds_read_b128.  The K
+// loop is unrolled by two so that the stage is a compile-time constant (hence K % 128 == 0), and
+// the loads walk the K tiles with a cursor instead of dividing the step number.
+// The inner loop is a fixed sequence of inline-assembly instructions so that its order is exactly
+// the one below (left to itself the compiler folds the two fragment register sets into one and
+// waits for every LDS read right after issuing it).  Per K tile held in stage S:
+//
+//   K step 0..2 : MFMA, 2 reads, MFMA, 2 reads, MFMA, 2 reads, 5 MFMA    (reads = next step's fragments)
+//   wait for the LDS reads and for this wave's direct-to-LDS loads, barrier
+//                                 -> stage S^1 (next K tile) is published, stage S is free
+//   start the direct-to-LDS loads of the K tile after next into stage S
+//   K step 3    : the same pattern, the reads being step 0 of the next K tile out of stage S^1
+//
+// so neither the barrier nor the first fragment reads of a K tile stand between two MFMAs.
+// At the last K tile of an output tile the loads into stage S start only after the epilogue
+// has used that stage for its transpose.
+template <int IMM>
+__device__ __forceinline__ void lds_read16(u32x4 &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(IMM));
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <bool BF16>
+__device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u32x4 &b) {
+    if constexpr (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+
 template <class T, bool BF16>
-__global__ __launch_bounds__(T::THREADS) void gemm16_persistent2_kernel(const Params p) {
+__global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -791,18 +663,18 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent2_kernel(const Pa
     constexpr int A_BYTES = BM * kBK * 2, B_BYTES = BN * kBK * 2;  // per stage
     constexpr int A_LOADS = A_BYTES / 1024 / WAVES, B_LOADS = B_BYTES / 1024 / WAVES;
     constexpr int EPI_PARTS = (BM * BN * 2) / (A_BYTES + B_BYTES);
-    static_assert(T::SWIZZLE == 1, "this kernel uses the 64-bank swizzle");
+    constexpr int READS = TM + TN;
+    static_assert(T::SWIZZLE == 1 && KS == 4, "");
     static_assert(WAVES % 2 == 0 && A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0, "");
-    static_assert(2 * A_BYTES + B_BYTES + (TN - 1) * 4096 < 65536 + 65536, "");
-    static_assert(EPI_PARTS >= 1 && TM % EPI_PARTS == 0, "");
-    static_assert((A_BYTES % (WAVES / 2 * (WTM * WTN * 2 / EPI_PARTS))) == 0 || true, "");
+    static_assert(A_BYTES + (TM - 1) * 4096 < 65536 && B_BYTES + (TN - 1) * 4096 < 65536, "");
+    static_assert(EPI_PARTS >= 1 && TM % EPI_PARTS == 0 && READS % 2 == 0 && TM * TN > READS / 2, "");
 
     extern __shared__ u32x4 lds[];
     char *const lds_bytes = reinterpret_cast<char *>(lds);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets address math run on the scalar unit
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int K = p.K;
     const int KT = K / kBK;
@@ -819,42 +691,49 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent2_kernel(const Pa
     typedef __attribute__((address_space(3))) void *lptr_t;
 
     auto tile_origin = [&](int t, int &m0, int &n0) {
-        const int tile = xcd_remap(static_cast<int>(blockIdx.x) + grid * t, p.nblocks);
-        m0 = (tile / p.tiles_n) * BM;
-        n0 = (tile % p.tiles_n) * BN;
+        int tile_m, tile_n;
+        tile_of(p, static_cast<int>(blockIdx.x), grid, t, tile_m, tile_n);
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
     };
 
-    auto issue = [&](int step, int stage) {
-        const int t = step / KT, kt = step - t * KT;
-        int m0, n0;
-        tile_origin(t, m0, n0);
-        const int k0 = kt * kBK;
+    // The loads walk the K tiles of this workgroup's output tiles in order; the cursor holds the
+    // next one to fetch, so no division is needed per step.
+    int ld_kt = 0, ld_t = 0, ld_m0, ld_n0;
+    tile_origin(0, ld_m0, ld_n0);
+    auto issue_next = [&](int stage) {
+        const int k0 = ld_kt * kBK;
         char *dst_a = lds_bytes + stage * A_BYTES;
         char *dst_b = lds_bytes + 2 * A_BYTES + stage * B_BYTES;
+        const char *base_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(ld_m0 + 8 * wave) * K + k0);
+        const char *base_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(ld_n0 + 8 * wave) * K + k0);
+        const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            const int g = wave + WAVES * i;
-            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * g) * K + k0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst_a + 1024 * g), 16, 0, 0);
-        }
+        for (int i = 0; i < A_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_a + i * group_stride + lane_off),
+                                             (lptr_t)(dst_a + 1024 * (wave + WAVES * i)), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) {
-            const int g = wave + WAVES * i;
-            const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * g) * K + k0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + lane_off), (lptr_t)(dst_b + 1024 * g), 16, 0, 0);
+        for (int i = 0; i < B_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(base_b + i * group_stride + lane_off),
+                                             (lptr_t)(dst_b + 1024 * (wave + WAVES * i)), 16, 0, 0);
+        if (++ld_kt == KT) {
+            ld_kt = 0;
+            ++ld_t;
+            if (ld_t < my_tiles) tile_origin(ld_t, ld_m0, ld_n0);
         }
     };
 
-    // Fragment addresses: row (lane % 32) of a 32-row block, chunk (2 ks + lane / 32) ^ swizzle(row).
+    // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps.
     const int frow = lane & 31;
     const int fhalf = lane >> 5;
-    const int sw = (frow >> 1) & 7;  // 32-row blocks start at multiples of 16 rows: the swizzle sees only frow
+    const int sw = (frow >> 1) & 7;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_bytes));  // LDS aperture offset
     uint32_t off_a[KS], off_b[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const uint32_t o = static_cast<uint32_t>(frow * 128 + (((2 * ks + fhalf) ^ sw) << 4));
-        off_a[ks] = o + wm * WTM * 128;
-        off_b[ks] = o + 2 * A_BYTES + wn * WTN * 128;
+        off_a[ks] = lds_base + o + wm * WTM * 128;
+        off_b[ks] = lds_base + o + 2 * A_BYTES + wn * WTN * 128;
     }
 
     float16v acc[TM][TN];
@@ -868,98 +747,117 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent2_kernel(const Pa
     };
     clear_acc();
 
-    auto compute_tile = [&](auto stage_c) {
-        constexpr int S = decltype(stage_c)::value;
-        u32x4 af[2][TM], bf[2][TN];
-        auto read_frags = [&](int ks, int slot) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                af[slot][i] = *reinterpret_cast<const u32x4 *>(lds_bytes + off_a[ks] + (S * A_BYTES + i * 4096));
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                bf[slot][j] = *reinterpret_cast<const u32x4 *>(lds_bytes + off_b[ks] + (S * B_BYTES + j * 4096));
-        };
-        read_frags(0, 0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (ks + 1 < KS) read_frags(ks + 1, (ks + 1) & 1);
-            const int slot = ks & 1;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
-            if constexpr (T::SCHED == 1) {
-                constexpr int READS = TM + TN;
-                if (ks + 1 < KS) {
-#pragma unroll
-                    for (int r = 0; r < READS / 2; ++r) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - READS / 2, 0);
-                } else {
-                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
-                }
+    u32x4 af[2][TM], bf[2][TN];
+
+    // read number R (0 .. READS-1) of K step KSTEP out of stage S into fragment set SLOT
+    auto read_one = [&](auto r_c, auto ks_c, auto slot_c, auto stage_c) {
+        constexpr int R = decltype(r_c)::value, KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value,
+                      S = decltype(stage_c)::value;
+        if constexpr (R < TM) lds_read16<S * A_BYTES + R * 4096>(af[SLOT][R], off_a[KSTEP]);
+        else lds_read16<S * B_BYTES + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[KSTEP]);
+    };
+
+    // MFMAs of one K step out of fragment set SLOT, with the reads reader(R) spread over the first ones
+    auto mfma_step = [&](auto slot_c, auto reader) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        static_for<TM * TN>([&](auto idx_c) {
+            constexpr int IDX = decltype(idx_c)::value;
+            constexpr int I = IDX / TN, J = IDX % TN;
+            mfma_asm<BF16>(acc[I][J], bf[SLOT][J], af[SLOT][I]);
+            if constexpr (IDX < READS / 2) {
+                reader(std::integral_constant<int, 2 * IDX>{});
+                reader(std::integral_constant<int, 2 * IDX + 1>{});
             }
+        });
+    };
+
+    // all reads issued so far have landed; the fake operands keep later MFMAs behind this point
+    auto wait_frags = [&](int slot) {
+        if constexpr (TM == 4 && TN == 2) {
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
+                           "+v"(bf[slot][0]), "+v"(bf[slot][1]));
+        } else if constexpr (TM == 2 && TN == 4) {
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1]),
+                           "+v"(bf[slot][2]), "+v"(bf[slot][3]));
+        } else {
+            static_assert(TM == 4 && TN == 4, "");
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
+                           "+v"(bf[slot][0]), "+v"(bf[slot][1]), "+v"(bf[slot][2]), "+v"(bf[slot][3]));
         }
     };
 
-    // K tiles come in pairs (the launcher takes this kernel for an even number of K tiles only), so
-    // every output tile starts in stage 0 and the stage is a compile-time constant of each half step.
-    auto step_fn = [&](int step, auto stage_c) {
+    int t = 0;
+    auto step_fn = [&](int step, auto last_c, auto stage_c) {
         constexpr int S = decltype(stage_c)::value;
-        const bool tracing = p.trace != nullptr && blockIdx.x == 0 && lane == 0;
-        unsigned long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-        if (tracing) t0 = __builtin_amdgcn_s_memtime();
-        if (step + 1 < total) issue(step + 1, S ^ 1);
-        compute_tile(stage_c);
-        if (tracing) t1 = __builtin_amdgcn_s_memtime();
+        constexpr bool last_of_tile = decltype(last_c)::value;  // last K tile of an output tile
+        using Other = std::integral_constant<int, S ^ 1>;
+        using C0 = std::integral_constant<int, 0>;
+        using C1 = std::integral_constant<int, 1>;
+        using C2 = std::integral_constant<int, 2>;
+        using C3 = std::integral_constant<int, 3>;
+        // K steps 0..2: their MFMAs, with the next step's fragments read early in each
+        mfma_step(C0{}, [&](auto r) { read_one(r, C1{}, C1{}, stage_c); });
+        wait_frags(1);
+        mfma_step(C1{}, [&](auto r) { read_one(r, C2{}, C0{}, stage_c); });
+        wait_frags(0);
+        mfma_step(C0{}, [&](auto r) { read_one(r, C3{}, C1{}, stage_c); });
+        wait_frags(1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (tracing) t2 = __builtin_amdgcn_s_memtime();
         lds_barrier();
-        if (tracing) {
-            t3 = __builtin_amdgcn_s_memtime();
-            unsigned long long *dst = p.trace + (static_cast<size_t>(wave) * 64 + step) * 4;
-            if (step < 64) {
-                dst[0] = t0;
-                dst[1] = t1;
-                dst[2] = t2;
-                dst[3] = t3;
-            }
+        if (!last_of_tile && step + 2 < total) issue_next(S);
+        // K step 3, with step 0 of the next K tile read out of the other stage (after the very last
+        // K tile these reads fetch stale but in-bounds LDS contents that nothing uses)
+        mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Other{}); });
+        wait_frags(0);
+        if constexpr (last_of_tile) {
+            int m0, n0;
+            tile_origin(t, m0, n0);
+            // MFMA results are read by vector ALU instructions next: cover the issue-to-write latency
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+            constexpr int REGION = WTM * WTN * 2 / EPI_PARTS;  // bytes per wave
+            static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
+            char *region = wave < WAVES / 2 ? lds_bytes + S * A_BYTES + wave * REGION
+                                            : lds_bytes + 2 * A_BYTES + S * B_BYTES + (wave - WAVES / 2) * REGION;
+            store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                                                            m0 + wm * WTM, n0 + wn * WTN);
+            clear_acc();
+            lds_barrier();  // every wave is done with its transpose region in stage S
+            if (step + 2 < total) issue_next(S);
+            ++t;
         }
     };
 
-    issue(0, 0);
+    // Prologue: K tile 0 into stage 0, published; K tile 1 on its way into stage 1; fragments of step 0.
+    issue_next(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
+    if (total > 1) issue_next(1);
+    static_for<READS>([&](auto r) {
+        read_one(r, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+    });
+    wait_frags(0);
+
     int step = 0;
-    for (int t = 0; t < my_tiles; ++t) {
-        for (int kt = 0; kt < KT; kt += 2, step += 2) {
-            step_fn(step, std::integral_constant<int, 0>{});
-            step_fn(step + 1, std::integral_constant<int, 1>{});
+    for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
+        for (int kt = 0; kt + 2 < KT; kt += 2, step += 2) {
+            step_fn(step, std::false_type{}, std::integral_constant<int, 0>{});
+            step_fn(step + 1, std::false_type{}, std::integral_constant<int, 1>{});
         }
-        int m0, n0;
-        tile_origin(t, m0, n0);
-        // Stage 1 was consumed last and is free; stage 0 already holds the next tile's first K tile.
-        // The transpose regions of the first half of the waves lie in stage 1's A part, those of the
-        // second half in its B part.
-        constexpr int REGION = WTM * WTN * 2 / EPI_PARTS;  // bytes per wave
-        static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
-        char *region = wave < WAVES / 2 ? lds_bytes + A_BYTES + wave * REGION
-                                        : lds_bytes + 2 * A_BYTES + B_BYTES + (wave - WAVES / 2) * REGION;
-        store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane, m0 + wm * WTM,
-                                                        n0 + wn * WTN);
-        clear_acc();
-        lds_barrier();  // the next step loads into stage 1
+        step_fn(step, std::false_type{}, std::integral_constant<int, 0>{});
+        step_fn(step + 1, std::true_type{}, std::integral_constant<int, 1>{});  // ends with the epilogue
+        step += 2;
     }
 }
 
 template <class T, bool BF16>
-int launch_persistent2(Params p, hipStream_t stream) {
+int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
-    auto kernel = gemm16_persistent2_kernel<T, BF16>;
+    auto kernel = gemm16_pinned_kernel<T, BF16>;
     static bool configured = false;
     if (!configured) {
         KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -967,24 +865,29 @@ int launch_persistent2(Params p, hipStream_t stream) {
         configured = true;
     }
     p.tiles_n = p.N / T::BN;
-    p.nblocks = (p.M / T::BM) * p.tiles_n;
+    const int tiles_m = p.M / T::BM;
+    p.nblocks = tiles_m * p.tiles_n;
     int grid = compute_units() / 8 * 8;
     if (grid > p.nblocks) grid = p.nblocks;
+    // Blocked tile order when the tile grid divides evenly over 8 XCDs x (grid / 8) workgroups.
+    p.band_rows = 0;
+    p.block_cols = 0;
+    const int per_xcd = grid / 8;
+    if (tuning("gemm16.mapping") != 1 && grid % 8 == 0 && tiles_m % 8 == 0) {
+        const int band = tiles_m / 8;
+        if (band <= per_xcd && per_xcd % band == 0 && p.tiles_n % (per_xcd / band) == 0) {
+            p.band_rows = band;
+            p.block_cols = per_xcd / band;
+        }
+    }
     kernel<<<dim3(static_cast<unsigned>(grid)), dim3(T::THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
 
-template <class T, bool BF16, bool B_ROW_MAJOR>
-int launch_persistent2_experimental(const Params &p, hipStream_t stream) {
-    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_persistent2<T, BF16>(p, stream);
-    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
-}
-
 template <class T, bool BF16>
 int launch_persistent(Params p, hipStream_t stream) {
-    // two stages plus 256 bytes per wave of scratch for the cache-line touches
-    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t) + (T::L2_AHEAD > 0 ? T::THREADS * 4 : 0);
+    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the persistent variant needs full tiles");
     auto kernel = gemm16_persistent_kernel<T, BF16>;
@@ -1001,37 +904,6 @@ int launch_persistent(Params p, hipStream_t stream) {
     kernel<<<dim3(static_cast<unsigned>(grid)), dim3(T::THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;
-}
-
-template <class T, bool BF16, bool B_ROW_MAJOR>
-int launch_persistent_experimental(const Params &p, hipStream_t stream) {
-    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_persistent<T, BF16>(p, stream);
-    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
-}
-
-template <class T, bool BF16>
-int launch_dtl(Params p, hipStream_t stream) {
-    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
-    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the direct-to-LDS variant needs full tiles");
-    auto kernel = gemm16_dtl_kernel<T, BF16>;
-    static bool configured = false;
-    if (!configured) {
-        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
-    }
-    p.tiles_n = p.N / T::BN;
-    p.nblocks = (p.M / T::BM) * p.tiles_n;
-    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(T::THREADS), lds_bytes, stream>>>(p);
-    KO_CHECK_LAUNCH();
-    return KO_OK;
-}
-
-template <class T, bool BF16, bool B_ROW_MAJOR>
-int launch_dtl_experimental(const Params &p, hipStream_t stream) {
-    if constexpr (!BF16 && !B_ROW_MAJOR) return launch_dtl<T, BF16>(p, stream);
-    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
 }
 
 template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
@@ -1060,27 +932,38 @@ int launch(Params p, hipStream_t stream) {
     return launch_edge<T, BF16, B_ROW_MAJOR, false>(p, stream);
 }
 
-// Variants that exist for tuning only are built for the binary16, column-major-B case.
-template <class T, bool BF16, bool B_ROW_MAJOR>
-int launch_experimental(const Params &p, hipStream_t stream) {
-    if constexpr (!BF16 && !B_ROW_MAJOR) return launch<T, BF16, B_ROW_MAJOR>(p, stream);
-    else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: this tuning variant is built for f16 with column-major B only");
-}
-
 using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 128x64
 using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
+
+using TileBigTall = Tiling<256, 256, 4, 2, 1, true, 1>; // 8 waves, wave tile 64x128
+
+// The direct-to-LDS kernels need full 256x256x64 tiles and K-contiguous operands.
+template <class T, bool BF16, bool B_ROW_MAJOR, bool PINNED>
+int launch_direct(const Params &p, hipStream_t stream) {
+    if constexpr (B_ROW_MAJOR) {
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the direct-to-LDS variants need column-major B");
+    } else if constexpr (PINNED) {
+        return launch_pinned<T, BF16>(p, stream);
+    } else {
+        return launch_persistent<T, BF16>(p, stream);
+    }
+}
 
 template <bool BF16, bool B_ROW_MAJOR>
 int launch_variant(const Params &p, hipStream_t stream) {
     const int variant = tuning("gemm16.variant");
     if (variant <= 0) {
-        // Enough 256x256 tiles to fill the chip: the big tiling - as the persistent direct-to-LDS kernel
-        // when the tiles are full and both operands are K-contiguous, else as the register pipeline.
+        // Enough 256x256 tiles to fill the chip: the big tiling - as a persistent direct-to-LDS kernel
+        // when the tiles are full and both operands are K-contiguous (the pinned one when K is a
+        // multiple of 128), else as the register pipeline.
         // Fewer: 128x128 tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
         if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         if constexpr (!B_ROW_MAJOR) {
-            if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) return launch_persistent<TileBig, BF16>(p, stream);
+            if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) {
+                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBig, BF16>(p, stream);
+                return launch_persistent<TileBig, BF16>(p, stream);
+            }
         }
         return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
     }
@@ -1089,33 +972,16 @@ int launch_variant(const Params &p, hipStream_t stream) {
         case 6: return launch<Tiling<256, 256, 2, 4, 1, true, 0>, BF16, B_ROW_MAJOR>(p, stream);
         case 9: return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
         case 10: return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
-        case 20: return launch_dtl_experimental<TileBig, BF16, B_ROW_MAJOR>(p, stream);
-        case 23: return launch_dtl_experimental<Tiling<256, 256, 4, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
-        case 30:
-            if constexpr (!B_ROW_MAJOR) return launch_persistent<TileBig, BF16>(p, stream);
-            else return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: the persistent variant needs column-major B");
-        case 31: return launch_persistent_experimental<Tiling<256, 256, 4, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
-        case 36: return launch_persistent_experimental<Tiling<256, 256, 2, 4, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
-        case 41: return launch_persistent2_experimental<Tiling<256, 256, 2, 4, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
-        case 42: return launch_persistent2_experimental<Tiling<256, 256, 4, 2, 1, true, 1, 0, 1>, BF16, B_ROW_MAJOR>(p, stream);
+        case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
+        case 31: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, false>(p, stream);
+        case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 51: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
 
 }  // namespace
 }  // namespace ko
-
-namespace ko {
-namespace {
-unsigned long long *g_trace = nullptr;
-}
-}  // namespace ko
-
-// Tuning aid (not declared in ko.h): device buffer of 8 * 64 * 4 uint64 that the persistent
-// kernels fill with per-step timestamps of workgroup 0, or null to switch tracing off.
-extern "C" __attribute__((visibility("default"))) void ko_internal_gemm16_trace(void *buf) {
-    ko::g_trace = static_cast<unsigned long long *>(buf);
-}
 
 KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
                                 const void *B, int b_layout, float beta, const void *C, void *D,
@@ -1138,7 +1004,7 @@ KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, co
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: C and D must be 8-byte aligned");
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
-             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, g_trace};
+             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);

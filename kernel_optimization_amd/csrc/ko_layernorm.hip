@@ -60,7 +60,10 @@ struct Args {
 };
 
 // ---------------------------------------------------------------- WARP policy
-template <int LPR, int VPL, bool NT>
+// A wavefront takes BATCH consecutive row groups (a row group = 64 / LPR rows, one per lane
+// group); the loads of group b + 1 are issued before group b is reduced and stored, so reads
+// and writes of a wave overlap and gamma/beta are fetched once per BATCH groups.
+template <int LPR, int VPL, bool NT, int BATCH>
 __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
                                                              float *out,
                                                              float *__restrict__ mean_out,
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
     const int nvec = cols >> 2;
     const int64_t waves_per_block = blockDim.x >> 6;
     const int64_t wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * RPW;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * (RPW * BATCH);
 
     // gamma/beta of this lane's columns stay in registers across rows.
     float4v g[VPL], b[VPL];
@@ -91,19 +94,19 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
         }
     }
 
-    for (int64_t row0 = wave * RPW; row0 < rows; row0 += stride) {
-        const int64_t row = row0 + sub;
+    auto load_rows = [&](float4v (&v)[VPL], int64_t row) {
         const bool row_ok = row < rows;
         const float *src = in + row * cols;
-
-        float4v v[VPL];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
             if (row_ok && j < nvec) v[k] = load4<NT>(src + 4 * j);
             else v[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
         }
+    };
 
+    auto finish_rows = [&](float4v (&v)[VPL], int64_t row) {
+        const bool row_ok = row < rows;
         const float x0 = wave::broadcast_group_first<LPR>(v[0][0]);
         wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -134,6 +137,16 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
         if (row_ok && l == 0) {
             if (mean_out) mean_out[row] = x0 + mean;
             if (rstd_out) rstd_out[row] = rstd;
+        }
+    };
+
+    for (int64_t row0 = wave * (RPW * BATCH); row0 < rows; row0 += stride) {
+        float4v v[2][VPL];
+        load_rows(v[0], row0 + sub);
+#pragma unroll
+        for (int bt = 0; bt < BATCH; ++bt) {
+            if (bt + 1 < BATCH) load_rows(v[(bt + 1) & 1], row0 + (bt + 1) * RPW + sub);
+            finish_rows(v[bt & 1], row0 + bt * RPW + sub);
         }
     }
 }
@@ -269,23 +282,35 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float 
 }
 
 // ------------------------------------------------------------------ dispatch
-template <int LPR, int VPL, bool NT>
-int launch_wave(const Args &a) {
+template <int LPR, int VPL, bool NT, int BATCH>
+int launch_wave_batch(const Args &a) {
     constexpr int RPW = 64 / LPR;
-    constexpr int kThreads = 256;
-    const int64_t rows_per_block = RPW * (kThreads / 64);
+    // Single-wavefront workgroups by default (measured slightly faster than 256 threads).
+    int threads = tuning("layernorm.wave_threads");
+    if (threads != 128 && threads != 256) threads = 64;
+    const int64_t rows_per_block = static_cast<int64_t>(RPW) * BATCH * (threads / 64);
     const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
-    // One row batch per wavefront by default (measured faster than a persistent grid-stride
-    // launch: the hardware keeps more loads in flight); a positive knob caps the grid instead.
+    // One batch per wavefront by default; a positive knob caps the grid (grid-stride loop) instead.
     int64_t grid = needed;
     const int per_cu = tuning("layernorm.blocks_per_cu");
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    layernorm_wave_kernel<LPR, VPL, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    layernorm_wave_kernel<LPR, VPL, NT, BATCH><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
+}
+
+template <int LPR, int VPL, bool NT>
+int launch_wave(const Args &a) {
+    // One row group per wavefront by default: on MI355X batching measured slower at every size tried
+    // (the hardware keeps more independent waves in flight than a batch keeps loads).
+    int batch = tuning("layernorm.batch");
+    if (batch != 2 && batch != 4) batch = 1;
+    if (batch == 4) return launch_wave_batch<LPR, VPL, NT, 4>(a);
+    if (batch == 2) return launch_wave_batch<LPR, VPL, NT, 2>(a);
+    return launch_wave_batch<LPR, VPL, NT, 1>(a);
 }
 
 template <int LPR, bool NT>

@@ -9,7 +9,7 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5]
-GEMM16_VARIANTS = [0, 3, 6, 9, 10, 20, 23, 30, 31, 36, 41, 42]
+GEMM16_VARIANTS = [0, 3, 6, 9, 10, 30, 31, 50, 51]
 
 
 @pytest.fixture
@@ -99,14 +99,12 @@ def _to_f64(bits, bf16):
 @pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768), (512, 768, 192)])
 def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
-    if gemm16_variant not in (0, 3, 6, 9, 10, 30) and (bf16 or not b_col_major):
-        pytest.skip("tuning variants are built for f16 with column-major B only")
-    if gemm16_variant == 30 and not b_col_major:
-        pytest.skip("the persistent kernel takes column-major B")
-    if gemm16_variant >= 20 and (m % 256 or n % 256 or k % 64):
-        pytest.skip("the direct-to-LDS variants take full tiles only")
-    if gemm16_variant >= 40 and k % 128:
-        pytest.skip("this persistent variant takes an even number of K tiles")
+    if gemm16_variant >= 30 and not b_col_major:
+        pytest.skip("the direct-to-LDS kernels take column-major B")
+    if gemm16_variant >= 30 and (m % 256 or n % 256 or k % 64):
+        pytest.skip("the direct-to-LDS kernels take full tiles only")
+    if gemm16_variant >= 50 and k % 128:
+        pytest.skip("the pinned kernel takes an even number of K tiles")
     A = _bits16((m, k), 21 + m, bf16)
     B = _bits16((n, k) if b_col_major else (k, n), 23 + n, bf16)
     _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16)
@@ -127,7 +125,7 @@ def test_gemm16_variants_agree_bitwise(ko, m, n, k):
     outs = {}
     try:
         for v in GEMM16_VARIANTS[1:]:
-            if v >= 40 and k % 128:
+            if v >= 50 and k % 128:
                 continue
             ko.set_tuning("gemm16.variant", v)
             dD = ko.DeviceBuffer(m * n * 2)
@@ -147,10 +145,12 @@ def test_gemm16_variants_agree_bitwise(ko, m, n, k):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-def test_gemm16_default_path_big(ko, bf16):
-    """Large enough for the default dispatch to take the persistent direct-to-LDS kernel (512 tiles of
-    256 x 256, 5 K tiles: several tiles per workgroup, odd K-tile count), both 16-bit types."""
-    m, n, k = 8192, 4096, 320
+@pytest.mark.parametrize("k", [320, 384])
+def test_gemm16_default_path_big(ko, bf16, k):
+    """Large enough for the default dispatch to take a persistent direct-to-LDS kernel (512 tiles of
+    256 x 256: several tiles per workgroup), both 16-bit types.  k = 320 is an odd number of K tiles
+    (compiler-scheduled kernel), k = 384 an even one (pinned kernel)."""
+    m, n = 8192, 4096
     A = _bits16((m, k), 31, bf16)
     B = _bits16((n, k), 32, bf16)
     got = ko.gemm16_host(A, B, m, n, k, dtype=ko.BF16 if bf16 else ko.F16)
