@@ -70,7 +70,16 @@ def _vendor():
     V.kov_gemm16.argtypes = [i64, i64, i64, vp, vp, ci, vp, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
                              ctypes.POINTER(ci)]
     V.kov_sgemm.argtypes = [i64, i64, i64, vp, vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ci)]
+    pp = ctypes.POINTER(vp)
+    V.kov_gemm16_sets.argtypes = [i64, i64, i64, pp, pp, ci, pp, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
+                                  ctypes.POINTER(ci)]
+    V.kov_sgemm_sets.argtypes = [i64, i64, i64, pp, pp, pp, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
+                                 ctypes.POINTER(ci)]
     return V
+
+
+def _ptr_array(buffers):
+    return (ctypes.c_void_p * len(buffers))(*[b.ptr for b in buffers])
 
 
 # ------------------------------------------------------------------------------ workloads
@@ -142,8 +151,11 @@ def bench_sgemm(cfg, steps, warmup, vendor):
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
-        tmp = ko.DeviceBuffer(m * n * 4)
-        if vendor.kov_sgemm(m, n, k, As[0].ptr, Bs[0].ptr, tmp.ptr, 16, 50, ctypes.byref(us), ctypes.byref(na)) == 0:
+        # the vendor library rotates through the same operand sets (its own output buffers)
+        Vs = [ko.DeviceBuffer(m * n * 4) for _ in range(nsets)]
+        tmp = Vs[0]
+        if vendor.kov_sgemm_sets(m, n, k, _ptr_array(As), _ptr_array(Bs), _ptr_array(Vs), nsets, 16, 2 * nsets,
+                                 ctypes.byref(us), ctypes.byref(na)) == 0:
             res["hipblaslt_tflops"] = flops / us.value / 1e6
             res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
             ref = tmp.download(np.float32, (m, n))
@@ -170,9 +182,10 @@ def bench_gemm16(cfg, steps, warmup, vendor):
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
-        tmp = ko.DeviceBuffer(m * n * 2)
-        if vendor.kov_gemm16(m, n, k, As[0].ptr, Bs[0].ptr, 1, tmp.ptr, 0, 16, 20, ctypes.byref(us),
-                             ctypes.byref(na)) == 0:
+        Vs = [ko.DeviceBuffer(m * n * 2) for _ in range(nsets)]
+        tmp = Vs[0]
+        if vendor.kov_gemm16_sets(m, n, k, _ptr_array(As), _ptr_array(Bs), 1, _ptr_array(Vs), nsets, 0, 16, 20,
+                                  ctypes.byref(us), ctypes.byref(na)) == 0:
             res["hipblaslt_tflops"] = flops / us.value / 1e6
             res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
             ref = tmp.download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
