@@ -44,6 +44,9 @@ def _traffic(name):
         return None
 
 
+SECONDARY_MIN_WARMUP = 300
+
+
 def _time_steps(launch, steps, warmup):
     """warmup untimed launches, then `steps` launches: wall clock bracketed by device syncs, and a
     HIP event pair on the launch stream around the same launches."""
@@ -253,7 +256,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed launches before the timed ones; the device takes a few hundred short launches "
+                         "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
     ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS) + ["copy_f32"])
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
@@ -284,8 +289,10 @@ def main():
         for other in sorted(inputs.CONFIGS):
             if other == cfg:
                 continue
-            res, k2 = run_workload(other, args.steps, args.warmup, vendor)
+            warm = max(args.warmup, SECONDARY_MIN_WARMUP)
+            res, k2 = run_workload(other, args.steps, warm, vendor)
             del k2
+            res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
 
     line = {
