@@ -87,6 +87,20 @@ def _ptr_array(buffers):
 
 # ------------------------------------------------------------------------------ workloads
 
+def _copy_floor_us(xs, ys, n_f32, steps, warmup):
+    """Times the plain copy kernel over the same buffers (same bytes in, same bytes out, same rotation): what a
+    read+write stream of this size reaches on the device, launch ramp included.  Overwrites ys: call it
+    before the operator that is being measured."""
+    nsets = len(xs)
+    _, dev = _time_steps(lambda i: ko.copy_f32(xs[i % nsets], ys[i % nsets], n_f32), steps, warmup)
+    return dev * 1e6
+
+
+def _add_copy_floor(res, floor_us):
+    res["copy_same_bytes_us"] = floor_us
+    res["vs_copy_same_bytes"] = floor_us / res["kernel_us"]
+
+
 def bench_softmax(cfg, steps, warmup):
     c = inputs.CONFIGS[cfg]
     rows, cols = c["rows"], c["cols"]
@@ -101,12 +115,14 @@ def bench_softmax(cfg, steps, warmup):
     if "n_seq" in c:
         vl, rps = ko.DeviceBuffer(c["n_seq"] * 4), c["rows_per_seq"]
         ko.fill_lengths_i32(vl, c["n_seq"], inputs.tensor_seed(cfg, 1), c["len_lo"], c["len_hi"])
+    floor_us = _copy_floor_us(xs, ys, n, steps, warmup)
     wall, dev = _time_steps(lambda i: ko.softmax(xs[i % nsets], ys[i % nsets], rows, cols, vl, rps), steps, warmup)
     res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
                roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                              frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
+    _add_copy_floor(res, floor_us)
     keep = dict(x=xs[0], y=ys[0], vl=vl, rows=rows, cols=cols, rps=rps)
     return res, keep
 
@@ -126,13 +142,16 @@ def bench_layernorm(cfg, steps, warmup):
         ko.fill_normal_f32(x, n, inputs.tensor_seed(cfg, 0), 0.5, 2.0)
     ko.fill_normal_f32(g, cols, inputs.tensor_seed(cfg, 1), 1.0, 0.1)
     ko.fill_normal_f32(b, cols, inputs.tensor_seed(cfg, 2), 0.0, 0.1)
+    floor_us = _copy_floor_us(xs, ys, n, steps, warmup)
     wall, dev = _time_steps(lambda i: ko.layernorm(xs[i % nsets], ys[i % nsets], rows, cols, ms[i % nsets],
                                                    rs[i % nsets], g, b, c["eps"]), steps, warmup)
-    return dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
-                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-                roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                              frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
-                algorithmic_bytes=work, kernel_us=dev * 1e6), None
+    res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
+               ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
+               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
+               algorithmic_bytes=work, kernel_us=dev * 1e6)
+    _add_copy_floor(res, floor_us)
+    return res, None
 
 
 def bench_sgemm(cfg, steps, warmup, vendor):
@@ -209,6 +228,49 @@ def bench_copy(steps, warmup, nbytes=1 << 30):
                 roofline=dict(bound="hbm", achieved=2 * n * 4 / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                               frac=2 * n * 4 / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
                 algorithmic_bytes=2 * n * 4, kernel_us=dev * 1e6)
+
+
+def bench_rows16(kind, dtype_name, steps, warmup):
+    """The two row operators on 16-bit storage at the shapes of the masked-softmax and LayerNorm configurations
+    (half the bytes per element; fp32 arithmetic).  Inputs: uniform fills of the storage type."""
+    dtype = ko.BF16 if dtype_name == "bf16" else ko.F16
+    if kind == "softmax":
+        c = inputs.CONFIGS[5]
+        rows, cols = c["rows"], c["cols"]
+        work = 2 * rows * cols * 2
+    else:
+        c = inputs.CONFIGS[2]
+        rows, cols = c["rows"], c["cols"]
+        work = 2 * rows * cols * 2 + 2 * cols * 2 + 2 * rows * 4
+    n = rows * cols
+    nsets = max(1, -(-(1 << 30) // work))
+    xs = [ko.DeviceBuffer(n * 2) for _ in range(nsets)]
+    ys = [ko.DeviceBuffer(n * 2) for _ in range(nsets)]
+    for x in xs:
+        ko.fill_uniform_16(x, n, 7, -8.0, 8.0, dtype=dtype)
+    if kind == "softmax":
+        vl = ko.DeviceBuffer(c["n_seq"] * 4)
+        ko.fill_lengths_i32(vl, c["n_seq"], inputs.tensor_seed(5, 1), c["len_lo"], c["len_hi"])
+        launch = lambda i: ko.softmax16(xs[i % nsets], ys[i % nsets], rows, cols, vl, c["rows_per_seq"], dtype)
+        name = "masked_softmax_%s_%dx%d" % (dtype_name, rows, cols)
+    else:
+        g, b = ko.DeviceBuffer(cols * 2), ko.DeviceBuffer(cols * 2)
+        ko.fill_uniform_16(g, cols, 8, 0.8, 1.2, dtype=dtype)
+        ko.fill_uniform_16(b, cols, 9, -0.2, 0.2, dtype=dtype)
+        ms = [ko.DeviceBuffer(rows * 4) for _ in range(nsets)]
+        rs = [ko.DeviceBuffer(rows * 4) for _ in range(nsets)]
+        launch = lambda i: ko.layernorm16(xs[i % nsets], ys[i % nsets], rows, cols, ms[i % nsets], rs[i % nsets], g, b,
+                                          c["eps"], False, dtype)
+        name = "layernorm_%s_%dx%d" % (dtype_name, rows, cols)
+    floor_us = _copy_floor_us(xs, ys, n // 2, steps, warmup)
+    wall, dev = _time_steps(launch, steps, warmup)
+    res = dict(workload=name, metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
+               ms_per_step=wall * 1e3, dtype=dtype_name + " storage, f32 arithmetic", buffer_sets=nsets,
+               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
+               algorithmic_bytes=work, kernel_us=dev * 1e6)
+    _add_copy_floor(res, floor_us)
+    return res
 
 
 def run_workload(cfg, steps, warmup, vendor):
@@ -292,6 +354,11 @@ def main():
             warm = max(args.warmup, SECONDARY_MIN_WARMUP)
             res, k2 = run_workload(other, args.steps, warm, vendor)
             del k2
+            res["steps"], res["warmup"] = args.steps, warm
+            others.append(res)
+        for kind, dt in (("softmax", "f16"), ("layernorm", "bf16")):
+            warm = max(args.warmup, SECONDARY_MIN_WARMUP if kind == "layernorm" else 0)
+            res = bench_rows16(kind, dt, args.steps, warm)
             res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
 

@@ -33,23 +33,35 @@ KO_LAYERNORM_DESCRIPTOR(LayerNormBlockImpl, KO_POLICY_BLOCK,
 KO_LAYERNORM_DESCRIPTOR(LayerNormBlockNoCacheImpl, KO_POLICY_BLOCK_NOCACHE, 32 * 3 * sizeof(_Element));         // :254-300
 #undef KO_LAYERNORM_DESCRIPTOR
 
+// Element = float, half (ko_half) or ko_bfloat16 (storage of in, out, gamma, beta; fp32 arithmetic;
+// mean and rstd are always float).
 template <typename LayerNormKernel>
 void layer_normalization(int grid_dim, int block_dim, int smem_in_bytes, ko_stream_t stream,
                          typename LayerNormKernel::Element *in_data, typename LayerNormKernel::Element *out_data,
                          typename LayerNormKernel::Element epsilon,
                          typename LayerNormKernel::Element *gamma = nullptr,
-                         typename LayerNormKernel::Element *beta = nullptr,
-                         typename LayerNormKernel::Element *mean = nullptr,
-                         typename LayerNormKernel::Element *rstd = nullptr, bool unbiased = false) {
-    static_assert(std::is_same<typename LayerNormKernel::Element, float>::value, "libko provides the fp32 LayerNorm");
+                         typename LayerNormKernel::Element *beta = nullptr, float *mean = nullptr,
+                         float *rstd = nullptr, bool unbiased = false) {
+    using Element = typename LayerNormKernel::Element;
+    static_assert(std::is_same<Element, float>::value || std::is_same<Element, ko_half>::value ||
+                      std::is_same<Element, ko_bfloat16>::value,
+                  "libko provides LayerNorm on float, half and bfloat16 storage");
     (void)grid_dim;
     (void)block_dim;
     (void)smem_in_bytes;
     const bool affine = LayerNormKernel::elementwise_affine;
-    checkKoErrors(ko_layernorm_f32_policy(in_data, out_data, mean, rstd, affine ? gamma : nullptr,
-                                          affine ? beta : nullptr, LayerNormKernel::num_row,
-                                          LayerNormKernel::num_column, epsilon, unbiased ? 1 : 0,
-                                          LayerNormKernel::policy, stream));
+    if constexpr (std::is_same<Element, float>::value) {
+        checkKoErrors(ko_layernorm_f32_policy(in_data, out_data, mean, rstd, affine ? gamma : nullptr,
+                                              affine ? beta : nullptr, LayerNormKernel::num_row,
+                                              LayerNormKernel::num_column, epsilon, unbiased ? 1 : 0,
+                                              LayerNormKernel::policy, stream));
+    } else {
+        checkKoErrors(ko_layernorm_16(in_data, out_data, mean, rstd, affine ? gamma : nullptr, affine ? beta : nullptr,
+                                      LayerNormKernel::num_row, LayerNormKernel::num_column,
+                                      static_cast<float>(epsilon), unbiased ? 1 : 0,
+                                      std::is_same<Element, ko_half>::value ? KO_F16 : KO_BF16,
+                                      LayerNormKernel::policy, stream));
+    }
 }
 
 #endif  // KERNEL_OPTIMIZATION_LAYERNORM_H

@@ -50,15 +50,26 @@ struct SoftMaxBlockNoCacheImpl {
     static_assert(_num_column % _vec_len == 0, "Unaligned vectorized access");
 };
 
+// T = float, half (ko_half) or ko_bfloat16; the 16-bit types are storage types, the arithmetic is fp32
+// (the reference instantiates the same template with its half functors, common/functors.h:71-77).
 template <typename SoftMaxKernel>
 void softmax(int grid_dim, int block_dim, int smem_in_bytes, ko_stream_t stream, typename SoftMaxKernel::T *in_data,
              typename SoftMaxKernel::T *out_data, const int32_t *valid_len = nullptr, int64_t rows_per_seq = 0) {
-    static_assert(std::is_same<typename SoftMaxKernel::T, float>::value, "libko provides the fp32 softmax");
+    using T = typename SoftMaxKernel::T;
+    static_assert(std::is_same<T, float>::value || std::is_same<T, ko_half>::value ||
+                      std::is_same<T, ko_bfloat16>::value,
+                  "libko provides softmax on float, half and bfloat16 storage");
     (void)grid_dim;
     (void)block_dim;
     (void)smem_in_bytes;
-    checkKoErrors(ko_softmax_f32_policy(in_data, out_data, SoftMaxKernel::num_row, SoftMaxKernel::num_column,
-                                        valid_len, rows_per_seq, SoftMaxKernel::policy, stream));
+    if constexpr (std::is_same<T, float>::value) {
+        checkKoErrors(ko_softmax_f32_policy(in_data, out_data, SoftMaxKernel::num_row, SoftMaxKernel::num_column,
+                                            valid_len, rows_per_seq, SoftMaxKernel::policy, stream));
+    } else {
+        checkKoErrors(ko_softmax_16(in_data, out_data, SoftMaxKernel::num_row, SoftMaxKernel::num_column, valid_len,
+                                    rows_per_seq, std::is_same<T, ko_half>::value ? KO_F16 : KO_BF16,
+                                    SoftMaxKernel::policy, stream));
+    }
 }
 
 #endif  // KERNEL_OPTIMIZATION_SOFTMAX_H

@@ -108,6 +108,14 @@ int ko_softmax_f32_policy(const float *in, float *out, int64_t rows, int64_t col
                           const int32_t *valid_len, int64_t rows_per_seq, int policy,
                           ko_stream_t stream);
 
+/* Same operator on 16-bit storage: in, out are binary16 (KO_F16) or bfloat16 (KO_BF16) bit
+ * patterns, the arithmetic is fp32, the result is rounded once to the storage type.  cols must be
+ * a multiple of 8 (one 16-byte vector).  Stands in for the reference's T = half instantiation
+ * of the same template (softmax.h:11, with the half functors of common/functors.h:71-77 and
+ * limits of common/common.h:171-177).  policy: a ko_policy value. */
+int ko_softmax_16(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *valid_len,
+                  int64_t rows_per_seq, int dtype, int policy, ko_stream_t stream);
+
 /* ---- LayerNorm: replaces
  *      layer_normalization<K><<<...>>>(Element *in, Element *out, Element epsilon,
  *                                      Element *gamma = nullptr, Element *beta = nullptr)
@@ -123,6 +131,14 @@ int ko_layernorm_f32(const float *in, float *out, float *mean, float *rstd, cons
 int ko_layernorm_f32_policy(const float *in, float *out, float *mean, float *rstd,
                             const float *gamma, const float *beta, int64_t rows, int64_t cols,
                             float eps, int unbiased, int policy, ko_stream_t stream);
+
+/* Same operator on 16-bit storage: in, out, gamma, beta are binary16 or bfloat16 bit patterns
+ * (all of the one dtype), mean and rstd stay fp32, the arithmetic is fp32.  cols must be a
+ * multiple of 8.  Stands in for Element = half in LayerNormWarpImpl and its siblings
+ * (layernorm.h:145, with Rsqrt<half> of common/functors.h:105-111). */
+int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const void *gamma,
+                    const void *beta, int64_t rows, int64_t cols, float eps, int unbiased, int dtype,
+                    int policy, ko_stream_t stream);
 
 /* ---- SIMT-path SGEMM: replaces
  *      gemm<GemmKernelSimt<...>><<<grid, K::thread_per_block, K::smem_total_size_in_bytes, stream>>>

@@ -65,6 +65,8 @@ SIGNATURES = {
     "ko_softmax_f32_policy": (_int, [_vp, _vp, _i64, _i64, _vp, _i64, _int, _vp]),
     "ko_layernorm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _vp]),
     "ko_layernorm_f32_policy": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _int, _vp]),
+    "ko_softmax_16": (_int, [_vp, _vp, _i64, _i64, _vp, _i64, _int, _int, _vp]),
+    "ko_layernorm_16": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _int, _int, _vp]),
     "ko_sgemm_f32": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _f, _vp, _vp, _vp]),
     "ko_gemm_f16f32acc": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp]),
     "ko_fill_normal_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
@@ -257,6 +259,17 @@ def layernorm(inp, out, rows, cols, mean=None, rstd=None, gamma=None, beta=None,
                                         rows, cols, eps, int(bool(unbiased)), policy, _h(stream)))
 
 
+def softmax16(inp, out, rows, cols, valid_len=None, rows_per_seq=0, dtype=F16, policy=POLICY_AUTO, stream=None):
+    check(lib().ko_softmax_16(_p(inp), _p(out), rows, cols, _p(valid_len), rows_per_seq, dtype, policy,
+                              _h(stream)))
+
+
+def layernorm16(inp, out, rows, cols, mean=None, rstd=None, gamma=None, beta=None, eps=1e-5,
+                unbiased=False, dtype=F16, policy=POLICY_AUTO, stream=None):
+    check(lib().ko_layernorm_16(_p(inp), _p(out), _p(mean), _p(rstd), _p(gamma), _p(beta), rows, cols, eps,
+                                int(bool(unbiased)), dtype, policy, _h(stream)))
+
+
 def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
     check(lib().ko_sgemm_f32(m, n, k, alpha, _p(A), _p(B), beta, _p(C), _p(D), _h(stream)))
 
@@ -298,6 +311,33 @@ def softmax_host(x, valid_len=None, rows_per_seq=0, policy=POLICY_AUTO, in_place
     softmax(dx, dy, rows, cols, dv, rows_per_seq, policy)
     synchronize()
     return dy.download(np.float32, x.shape)
+
+
+def softmax16_host(x_bits, valid_len=None, rows_per_seq=0, dtype=F16, policy=POLICY_AUTO, in_place=False):
+    """x_bits: uint16 bit patterns [rows, cols]; returns uint16 [rows, cols]."""
+    x_bits = np.ascontiguousarray(x_bits).view(np.uint16)
+    rows, cols = x_bits.shape
+    dx = DeviceBuffer.from_numpy(x_bits)
+    dy = dx if in_place else DeviceBuffer(x_bits.nbytes)
+    dv = None if valid_len is None else DeviceBuffer.from_numpy(np.ascontiguousarray(valid_len, np.int32))
+    softmax16(dx, dy, rows, cols, dv, rows_per_seq, dtype, policy)
+    synchronize()
+    return dy.download(np.uint16, x_bits.shape)
+
+
+def layernorm16_host(x_bits, gamma_bits=None, beta_bits=None, eps=1e-5, unbiased=False, dtype=F16,
+                     policy=POLICY_AUTO, in_place=False):
+    """16-bit storage; returns (y uint16 [rows, cols], mean float32 [rows], rstd float32 [rows])."""
+    x_bits = np.ascontiguousarray(x_bits).view(np.uint16)
+    rows, cols = x_bits.shape
+    dx = DeviceBuffer.from_numpy(x_bits)
+    dy = dx if in_place else DeviceBuffer(x_bits.nbytes)
+    dg = None if gamma_bits is None else DeviceBuffer.from_numpy(np.ascontiguousarray(gamma_bits).view(np.uint16))
+    db = None if beta_bits is None else DeviceBuffer.from_numpy(np.ascontiguousarray(beta_bits).view(np.uint16))
+    dm, dr = DeviceBuffer(rows * 4), DeviceBuffer(rows * 4)
+    layernorm16(dx, dy, rows, cols, dm, dr, dg, db, eps, unbiased, dtype, policy)
+    synchronize()
+    return dy.download(np.uint16, x_bits.shape), dm.download(np.float32, (rows,)), dr.download(np.float32, (rows,))
 
 
 def layernorm_host(x, gamma=None, beta=None, eps=1e-5, unbiased=False, policy=POLICY_AUTO,

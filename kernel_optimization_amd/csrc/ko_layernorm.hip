@@ -1,5 +1,7 @@
-// LayerNorm over the last dimension for gfx950: one pass over HBM, fp32,
-// Welford statistics, outputs y and (optionally) per-row mean and rstd.
+// LayerNorm over the last dimension for gfx950: one pass over HBM, fp32
+// arithmetic, fp32 / binary16 / bfloat16 storage (x, y, gamma, beta; mean and
+// rstd are always fp32), Welford statistics, outputs y and (optionally) per-row
+// mean and rstd.
 //
 // Per row (nn_operators/layernorm/layernorm.h): each lane folds its elements
 // into a Welford triplet (count, mean, M2) with the streaming update of
@@ -45,13 +47,14 @@ __device__ __forceinline__ void welford_update(wave::Welford &w, float x, float 
     w.m2 = __builtin_fmaf(d, x - w.mean, w.m2);
 }
 
+template <int IO>
 struct Args {
-    const float *in;
-    float *out;
+    const typename Io<IO>::elem *in;
+    typename Io<IO>::elem *out;
     float *mean;
     float *rstd;
-    const float *gamma;
-    const float *beta;
+    const typename Io<IO>::elem *gamma;
+    const typename Io<IO>::elem *beta;
     int64_t rows;
     int cols;
     float eps;
@@ -63,75 +66,93 @@ struct Args {
 // A wavefront takes BATCH consecutive row groups (a row group = 64 / LPR rows, one per lane
 // group); the loads of group b + 1 are issued before group b is reduced and stored, so reads
 // and writes of a wave overlap and gamma/beta are fetched once per BATCH groups.
-template <int LPR, int VPL, bool NT, int BATCH>
-__global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
-                                                             float *out,
+// FULL: cols == LPR * VPL vectors, every lane folds the same number of elements (no per-vector bounds
+// checks, and the lanes merge with the equal-count form).
+template <int IO, int LPR, int VPL, bool FULL, int BATCH>
+__global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<IO>::elem *in,
+                                                             typename Io<IO>::elem *out,
                                                              float *__restrict__ mean_out,
                                                              float *__restrict__ rstd_out,
-                                                             const float *__restrict__ gamma,
-                                                             const float *__restrict__ beta, int64_t rows,
-                                                             int cols, float eps, float inv_denominator) {
+                                                             const typename Io<IO>::elem *__restrict__ gamma,
+                                                             const typename Io<IO>::elem *__restrict__ beta,
+                                                             int64_t rows, int cols, float eps,
+                                                             float inv_denominator) {
+    constexpr int E = Io<IO>::E;
     constexpr int RPW = 64 / LPR;
-    constexpr Reciprocals<VPL * 4> rcp;
+    constexpr bool NT = true;  // streaming accesses: every byte is touched once
+    constexpr Reciprocals<VPL * E> rcp;
     const int lane = threadIdx.x & 63;
     const int sub = lane / LPR;
     const int l = lane % LPR;
-    const int nvec = cols >> 2;
+    const int nvec = cols / E;
     const int64_t waves_per_block = blockDim.x >> 6;
     const int64_t wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
     const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * (RPW * BATCH);
 
-    // gamma/beta of this lane's columns stay in registers across rows.
-    float4v g[VPL], b[VPL];
-#pragma unroll
-    for (int k = 0; k < VPL; ++k) {
-        const int j = l + k * LPR;
-        g[k] = float4v{1.0f, 1.0f, 1.0f, 1.0f};
-        b[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
-        if (j < nvec) {
-            if (gamma) g[k] = load4<false>(gamma + 4 * j);
-            if (beta) b[k] = load4<false>(beta + 4 * j);
-        }
-    }
-
-    auto load_rows = [&](float4v (&v)[VPL], int64_t row) {
-        const bool row_ok = row < rows;
-        const float *src = in + row * cols;
+    // gamma/beta of this lane's columns stay in registers across rows.  They are fetched behind the first
+    // row's loads: memory returns in order, so loads issued ahead of the row would stand between the row
+    // and the statistics, which do not need them.
+    float g[VPL][E], b[VPL][E];
+    auto load_affine = [&]() {
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            if (row_ok && j < nvec) v[k] = load4<NT>(src + 4 * j);
-            else v[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                g[k][e] = 1.0f;
+                b[k][e] = 0.0f;
+            }
+            if (FULL || j < nvec) {
+                if (gamma) Io<IO>::template load<false>(gamma + E * j, g[k]);
+                if (beta) Io<IO>::template load<false>(beta + E * j, b[k]);
+            }
         }
     };
 
-    auto finish_rows = [&](float4v (&v)[VPL], int64_t row) {
+    auto load_rows = [&](float (&v)[VPL][E], int64_t row) {
+        const bool row_ok = row < rows;
+        const typename Io<IO>::elem *src = in + row * cols;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = l + k * LPR;
+            if (row_ok && (FULL || j < nvec)) {
+                Io<IO>::template load<NT>(src + E * j, v[k]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
+            }
+        }
+    };
+
+    auto finish_rows = [&](float (&v)[VPL][E], int64_t row) {
         const bool row_ok = row < rows;
         const float x0 = wave::broadcast_group_first<LPR>(v[0][0]);
         wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            v[k] = v[k] - x0;
-            if (j < nvec) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) welford_update(w, v[k][e], rcp.v[4 * k + e + 1]);
+            for (int e = 0; e < E; ++e) v[k][e] -= x0;
+            if (FULL || j < nvec) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
             }
         }
-        w = wave::welford_allreduce<LPR>(w);
+        if constexpr (FULL) w = wave::welford_allreduce_equal<LPR>(w);
+        else w = wave::welford_allreduce<LPR>(w);
 
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
 
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            if (row_ok && j < nvec) {
-                float4v y;
+            if (row_ok && (FULL || j < nvec)) {
+                float y[E];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[k][e], b[k][e]);
-                store4<NT>(dst + 4 * j, y);
+                for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[k][e], b[k][e]);
+                Io<IO>::template store<NT>(dst + E * j, y);
             }
         }
         if (row_ok && l == 0) {
@@ -140,9 +161,14 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float *in,
         }
     };
 
+    bool have_affine = false;
     for (int64_t row0 = wave * (RPW * BATCH); row0 < rows; row0 += stride) {
-        float4v v[2][VPL];
+        float v[2][VPL][E];
         load_rows(v[0], row0 + sub);
+        if (!have_affine) {
+            load_affine();
+            have_affine = true;
+        }
 #pragma unroll
         for (int bt = 0; bt < BATCH; ++bt) {
             if (bt + 1 < BATCH) load_rows(v[(bt + 1) & 1], row0 + (bt + 1) * RPW + sub);
@@ -173,55 +199,74 @@ __device__ __forceinline__ wave::Welford block_welford_allreduce(wave::Welford w
     return r;
 }
 
-template <int THREADS, int VPL>
-__global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *in,
-                                                                  float *out,
+// y = (x - mean) * rstd [* gamma] [+ beta] for one vector; gamma/beta are read here (long rows:
+// they do not fit the registers next to the row).
+template <int IO>
+__device__ __forceinline__ void normalize_vec(const float (&x)[Io<IO>::E], float mean, float rstd,
+                                              const typename Io<IO>::elem *gamma,
+                                              const typename Io<IO>::elem *beta, int col, float (&y)[Io<IO>::E]) {
+    constexpr int E = Io<IO>::E;
+    float g[E], b[E];
+    if (gamma) Io<IO>::template load<false>(gamma + col, g);
+    if (beta) Io<IO>::template load<false>(beta + col, b);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        float t = (x[e] - mean) * rstd;
+        if (gamma) t *= g[e];
+        if (beta) t += b[e];
+        y[e] = t;
+    }
+}
+
+template <int IO, int THREADS, int VPL>
+__global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename Io<IO>::elem *in,
+                                                                  typename Io<IO>::elem *out,
                                                                   float *__restrict__ mean_out,
                                                                   float *__restrict__ rstd_out,
-                                                                  const float *__restrict__ gamma,
-                                                                  const float *__restrict__ beta,
+                                                                  const typename Io<IO>::elem *__restrict__ gamma,
+                                                                  const typename Io<IO>::elem *__restrict__ beta,
                                                                   int64_t rows, int cols, float eps,
                                                                   float inv_denominator) {
+    constexpr int E = Io<IO>::E;
     __shared__ float lds[48];
-    constexpr Reciprocals<VPL * 4> rcp;
-    const int nvec = cols >> 2;
+    constexpr Reciprocals<VPL * E> rcp;
+    const int nvec = cols / E;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        const float *src = in + row * cols;
-        float4v v[VPL];
+        const typename Io<IO>::elem *src = in + row * cols;
+        float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
-            if (j < nvec) v[k] = load4<false>(src + 4 * j);
-            else v[k] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+            if (j < nvec) {
+                Io<IO>::template load<false>(src + E * j, v[k]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
+            }
         }
-        const float x0 = src[0];
+        const float x0 = Io<IO>::scalar(src);
         wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
-            v[k] = v[k] - x0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[k][e] -= x0;
             if (j < nvec) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) welford_update(w, v[k][e], rcp.v[4 * k + e + 1]);
+                for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
             }
         }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
             if (j < nvec) {
-                float4v y;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float t = (v[k][e] - mean) * rstd;
-                    if (gamma) t *= gamma[4 * j + e];
-                    if (beta) t += beta[4 * j + e];
-                    y[e] = t;
-                }
-                store4<false>(dst + 4 * j, y);
+                float y[E];
+                normalize_vec<IO>(v[k], mean, rstd, gamma, beta, E * j, y);
+                Io<IO>::template store<false>(dst + E * j, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -232,47 +277,46 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const float *i
 }
 
 // ------------------------------------------------------- BLOCK_NOCACHE policy
-template <int THREADS>
-__global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float *in,
-                                                                    float *out,
+template <int IO, int THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typename Io<IO>::elem *in,
+                                                                    typename Io<IO>::elem *out,
                                                                     float *__restrict__ mean_out,
                                                                     float *__restrict__ rstd_out,
-                                                                    const float *__restrict__ gamma,
-                                                                    const float *__restrict__ beta,
+                                                                    const typename Io<IO>::elem *__restrict__ gamma,
+                                                                    const typename Io<IO>::elem *__restrict__ beta,
                                                                     int64_t rows, int cols, float eps,
                                                                     float inv_denominator) {
+    constexpr int E = Io<IO>::E;
     __shared__ float lds[48];
-    const int nvec = cols >> 2;
+    const int nvec = cols / E;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        const float *src = in + row * cols;
-        const float x0 = src[0];
+        const typename Io<IO>::elem *src = in + row * cols;
+        const float x0 = Io<IO>::scalar(src);
         wave::Welford w{0.0f, 0.0f, 0.0f};
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load4<false>(src + 4 * j) - x0;
+            float x[E];
+            Io<IO>::template load<false>(src + E * j, x);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
+            for (int e = 0; e < E; ++e) {
                 // streaming update with a true division: the count is not a compile-time constant here
+                const float xe = x[e] - x0;
                 w.count += 1.0f;
-                const float d = x[e] - w.mean;
+                const float d = xe - w.mean;
                 w.mean += d / w.count;
-                w.m2 = __builtin_fmaf(d, x[e] - w.mean, w.m2);
+                w.m2 = __builtin_fmaf(d, xe - w.mean, w.m2);
             }
         }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load4<false>(src + 4 * j) - x0;
-            float4v y;
+            float x[E], y[E];
+            Io<IO>::template load<false>(src + E * j, x);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float t = (x[e] - mean) * rstd;
-                if (gamma) t *= gamma[4 * j + e];
-                if (beta) t += beta[4 * j + e];
-                y[e] = t;
-            }
-            store4<false>(dst + 4 * j, y);
+            for (int e = 0; e < E; ++e) x[e] -= x0;
+            normalize_vec<IO>(x, mean, rstd, gamma, beta, E * j, y);
+            Io<IO>::template store<false>(dst + E * j, y);
         }
         if (threadIdx.x == 0) {
             if (mean_out) mean_out[row] = x0 + mean;
@@ -282,8 +326,8 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const float 
 }
 
 // ------------------------------------------------------------------ dispatch
-template <int LPR, int VPL, bool NT, int BATCH>
-int launch_wave_batch(const Args &a) {
+template <int IO, int LPR, int VPL, bool FULL, int BATCH>
+int launch_wave_batch(const Args<IO> &a) {
     constexpr int RPW = 64 / LPR;
     // Single-wavefront workgroups by default (measured slightly faster than 256 threads).
     int threads = tuning("layernorm.wave_threads");
@@ -296,82 +340,91 @@ int launch_wave_batch(const Args &a) {
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    layernorm_wave_kernel<LPR, VPL, NT, BATCH><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+    layernorm_wave_kernel<IO, LPR, VPL, FULL, BATCH><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
 
-template <int LPR, int VPL, bool NT>
-int launch_wave(const Args &a) {
-    // One row group per wavefront by default: on MI355X batching measured slower at every size tried
-    // (the hardware keeps more independent waves in flight than a batch keeps loads).
-    int batch = tuning("layernorm.batch");
-    if (batch != 2 && batch != 4) batch = 1;
-    if (batch == 4) return launch_wave_batch<LPR, VPL, NT, 4>(a);
-    if (batch == 2) return launch_wave_batch<LPR, VPL, NT, 2>(a);
-    return launch_wave_batch<LPR, VPL, NT, 1>(a);
+template <int IO, int LPR, int VPL>
+int launch_wave(const Args<IO> &a) {
+    // One row group per wavefront: batches of 2 and 4 row groups per wave (gamma and beta fetched once per
+    // batch, the next group's loads issued before the current one is reduced) measured 5-8 % slower on
+    // MI355X at [16384, 768] - the hardware keeps more independent waves in flight than a batch keeps loads.
+    if (a.cols == LPR * VPL * Io<IO>::E) return launch_wave_batch<IO, LPR, VPL, true, 1>(a);
+    return launch_wave_batch<IO, LPR, VPL, false, 1>(a);
 }
 
-template <int LPR, bool NT>
-int launch_wave_vpl(const Args &a, int vpl) {
+template <int IO, int LPR>
+int launch_wave_vpl(const Args<IO> &a, int vpl) {
     switch (vpl) {
-        case 1: return launch_wave<LPR, 1, NT>(a);
-        case 2: return launch_wave<LPR, 2, NT>(a);
-        case 3: return launch_wave<LPR, 3, NT>(a);
-        case 4: return launch_wave<LPR, 4, NT>(a);
+        case 1: return launch_wave<IO, LPR, 1>(a);
+        case 2: return launch_wave<IO, LPR, 2>(a);
+        case 3: return launch_wave<IO, LPR, 3>(a);
+        case 4: return launch_wave<IO, LPR, 4>(a);
         case 5:
-        case 6: return launch_wave<LPR, 6, NT>(a);
-        default: return launch_wave<LPR, 8, NT>(a);
+        case 6: return launch_wave<IO, LPR, 6>(a);
+        default: return launch_wave<IO, LPR, 8>(a);
     }
 }
 
-template <bool NT>
-int launch_wave_lpr(const Args &a, int lpr) {
-    const int nvec = a.cols / 4;
+template <int IO>
+int launch_wave_lpr(const Args<IO> &a, int lpr) {
+    const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + lpr - 1) / lpr;
     switch (lpr) {
-        case 8: return launch_wave_vpl<8, NT>(a, vpl);
-        case 16: return launch_wave_vpl<16, NT>(a, vpl);
-        case 32: return launch_wave_vpl<32, NT>(a, vpl);
-        default: return launch_wave_vpl<64, NT>(a, vpl);
+        case 8: return launch_wave_vpl<IO, 8>(a, vpl);
+        case 16: return launch_wave_vpl<IO, 16>(a, vpl);
+        case 32: return launch_wave_vpl<IO, 32>(a, vpl);
+        default: return launch_wave_vpl<IO, 64>(a, vpl);
     }
 }
 
 constexpr int kWaveMaxVpl = 8;
-constexpr int kWaveMaxCols = 64 * kWaveMaxVpl * 4;  // 2048
-constexpr int kBlockMaxCols = 1024 * 8 * 4;         // 32768
+// Longest row per policy, in 16-byte vectors (fp32: 2048 and 32768 columns; 16-bit: twice that).
+constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
+constexpr int kBlockMaxVecs = 1024 * 8;
 
-// Lanes per row for the WARP policy: the narrowest group that gives every lane at most
-// one vector, so that one load instruction of the group covers the row contiguously;
-// rows longer than 64 vectors take the whole wavefront and several vectors per lane.
-int default_lanes_per_row(int cols) {
-    const int nvec = cols / 4;
-    int lpr = 8;
-    while (lpr < 64 && lpr < nvec) lpr <<= 1;
-    return lpr;
+// Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
+// {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
+// and a wavefront's worth of latency), and among equals takes the widest group: one load instruction
+// of the group then covers the longest contiguous piece of the row.
+int default_lanes_per_row(int nvec) {
+    int best = 64, best_waste = 1 << 30;
+    for (int lpr = 8; lpr <= 64; lpr <<= 1) {
+        int vpl = (nvec + lpr - 1) / lpr;
+        if (vpl > 8) continue;
+        if (vpl == 5) vpl = 6;
+        if (vpl == 7) vpl = 8;
+        const int waste = lpr * vpl - nvec;
+        if (waste <= best_waste) {
+            best_waste = waste;
+            best = lpr;
+        }
+    }
+    return best;
 }
 
-int launch_wave_any(const Args &a) {
+template <int IO>
+int launch_wave_any(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     int lpr = tuning("layernorm.lanes_per_row");
-    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(a.cols);
-    while (lpr < 64 && (a.cols / 4 + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
-    // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off.
-    if (tuning("layernorm.nontemporal") == 2) return launch_wave_lpr<false>(a, lpr);
-    return launch_wave_lpr<true>(a, lpr);
+    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec);
+    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    return launch_wave_lpr<IO>(a, lpr);
 }
 
-template <int THREADS>
-int launch_block_threads(const Args &a) {
-    const int nvec = a.cols / 4;
+template <int IO, int THREADS>
+int launch_block_threads(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + THREADS - 1) / THREADS;
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
     if (grid > a.rows) grid = a.rows;
     dim3 g(static_cast<unsigned>(grid)), b(THREADS);
-#define KO_LN_BLOCK(V)                                                                             \
-    layernorm_block_kernel<THREADS, V><<<g, b, 0, a.stream>>>(a.in, a.out, a.mean, a.rstd, a.gamma, \
-                                                              a.beta, a.rows, a.cols, a.eps,        \
-                                                              a.inv_denominator)
+#define KO_LN_BLOCK(V)                                                                                 \
+    layernorm_block_kernel<IO, THREADS, V><<<g, b, 0, a.stream>>>(a.in, a.out, a.mean, a.rstd, a.gamma, \
+                                                                  a.beta, a.rows, a.cols, a.eps,        \
+                                                                  a.inv_denominator)
     if (vpl <= 1) KO_LN_BLOCK(1);
     else if (vpl <= 2) KO_LN_BLOCK(2);
     else if (vpl <= 4) KO_LN_BLOCK(4);
@@ -381,27 +434,72 @@ int launch_block_threads(const Args &a) {
     return KO_OK;
 }
 
-int launch_block(const Args &a) {
-    const int nvec = a.cols / 4;
+template <int IO>
+int launch_block(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     int threads = tuning("layernorm.block_threads");
     if (threads != 256 && threads != 512 && threads != 1024) {
         threads = 256;
         while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;
     }
     while (threads < 1024 && (nvec + threads - 1) / threads > 8) threads <<= 1;
-    if (threads == 256) return launch_block_threads<256>(a);
-    if (threads == 512) return launch_block_threads<512>(a);
-    return launch_block_threads<1024>(a);
+    if (threads == 256) return launch_block_threads<IO, 256>(a);
+    if (threads == 512) return launch_block_threads<IO, 512>(a);
+    return launch_block_threads<IO, 1024>(a);
 }
 
-int launch_nocache(const Args &a) {
+template <int IO>
+int launch_nocache(const Args<IO> &a) {
     constexpr int kThreads = 1024;
     int64_t grid = static_cast<int64_t>(compute_units()) * 4;
     if (grid > a.rows) grid = a.rows;
-    layernorm_nocache_kernel<kThreads><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    layernorm_nocache_kernel<IO, kThreads><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
+}
+
+template <int IO>
+int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma, const void *beta, int64_t rows,
+          int64_t cols, float eps, int unbiased, int policy, ko_stream_t stream) {
+    constexpr int E = Io<IO>::E;
+    typedef typename Io<IO>::elem elem;
+    if (rows < 0 || cols <= 0)
+        return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: rows=%lld cols=%lld", (long long)rows, (long long)cols);
+    if (cols % E != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld is not a multiple of the vector width %d",
+                    (long long)cols, E);
+    if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld too large", (long long)cols);
+    if (rows == 0) return KO_OK;
+    if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: null in/out pointer");
+    uintptr_t align = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
+                      reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta);
+    if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: in/out/gamma/beta must be 16-byte aligned");
+    if (!(eps >= 0.0f)) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: eps must be >= 0");
+    const double denom = unbiased ? static_cast<double>(cols - 1) : static_cast<double>(cols);
+    Args<IO> a{static_cast<const elem *>(in), static_cast<elem *>(out), mean, rstd, static_cast<const elem *>(gamma),
+               static_cast<const elem *>(beta), rows, static_cast<int>(cols), eps, static_cast<float>(1.0 / denom),
+               as_stream(stream)};
+    const int nvec = a.cols / E;
+    if (policy == KO_POLICY_AUTO) {
+        policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
+                 : nvec <= kBlockMaxVecs ? KO_POLICY_BLOCK
+                                         : KO_POLICY_BLOCK_NOCACHE;
+    }
+    switch (policy) {
+        case KO_POLICY_WARP:
+            if (nvec > kWaveMaxVecs)
+                return fail(KO_ERR_UNSUPPORTED_SHAPE,
+                            "layernorm: WARP policy holds at most %d columns per row, got %d", kWaveMaxVecs * E, a.cols);
+            return launch_wave_any<IO>(a);
+        case KO_POLICY_BLOCK:
+            if (nvec > kBlockMaxVecs)
+                return fail(KO_ERR_UNSUPPORTED_SHAPE,
+                            "layernorm: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs * E, a.cols);
+            return launch_block<IO>(a);
+        case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO>(a);
+        default: return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);
+    }
 }
 
 }  // namespace
@@ -411,41 +509,7 @@ KO_EXPORT int ko_layernorm_f32_policy(const float *in, float *out, float *mean, 
                                       const float *gamma, const float *beta, int64_t rows,
                                       int64_t cols, float eps, int unbiased, int policy,
                                       ko_stream_t stream) {
-    using namespace ko;
-    if (rows < 0 || cols <= 0)
-        return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: rows=%lld cols=%lld", (long long)rows, (long long)cols);
-    if (cols % 4 != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld is not a multiple of the vector width 4",
-                    (long long)cols);
-    if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld too large", (long long)cols);
-    if (rows == 0) return KO_OK;
-    if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: null in/out pointer");
-    uintptr_t align = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
-                      reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta);
-    if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: in/out/gamma/beta must be 16-byte aligned");
-    if (!(eps >= 0.0f)) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: eps must be >= 0");
-    const double denom = unbiased ? static_cast<double>(cols - 1) : static_cast<double>(cols);
-    Args a{in, out, mean, rstd, gamma, beta, rows, static_cast<int>(cols), eps,
-           static_cast<float>(1.0 / denom), as_stream(stream)};
-    if (policy == KO_POLICY_AUTO) {
-        policy = a.cols <= kWaveMaxCols ? KO_POLICY_WARP
-                 : a.cols <= kBlockMaxCols ? KO_POLICY_BLOCK
-                                           : KO_POLICY_BLOCK_NOCACHE;
-    }
-    switch (policy) {
-        case KO_POLICY_WARP:
-            if (a.cols > kWaveMaxCols)
-                return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "layernorm: WARP policy holds at most %d columns per row, got %d", kWaveMaxCols, a.cols);
-            return launch_wave_any(a);
-        case KO_POLICY_BLOCK:
-            if (a.cols > kBlockMaxCols)
-                return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "layernorm: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxCols, a.cols);
-            return launch_block(a);
-        case KO_POLICY_BLOCK_NOCACHE: return launch_nocache(a);
-        default: return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);
-    }
+    return ko::entry<ko::IO_F32>(in, out, mean, rstd, gamma, beta, rows, cols, eps, unbiased, policy, stream);
 }
 
 KO_EXPORT int ko_layernorm_f32(const float *in, float *out, float *mean, float *rstd,
@@ -453,4 +517,14 @@ KO_EXPORT int ko_layernorm_f32(const float *in, float *out, float *mean, float *
                                float eps, int unbiased, ko_stream_t stream) {
     return ko_layernorm_f32_policy(in, out, mean, rstd, gamma, beta, rows, cols, eps, unbiased,
                                    KO_POLICY_AUTO, stream);
+}
+
+KO_EXPORT int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const void *gamma,
+                              const void *beta, int64_t rows, int64_t cols, float eps, int unbiased, int dtype,
+                              int policy, ko_stream_t stream) {
+    if (dtype == KO_F16)
+        return ko::entry<ko::IO_F16>(in, out, mean, rstd, gamma, beta, rows, cols, eps, unbiased, policy, stream);
+    if (dtype == KO_BF16)
+        return ko::entry<ko::IO_BF16>(in, out, mean, rstd, gamma, beta, rows, cols, eps, unbiased, policy, stream);
+    return ko::fail(KO_ERR_INVALID_ARGUMENT, "layernorm: dtype=%d is neither KO_F16 nor KO_BF16", dtype);
 }

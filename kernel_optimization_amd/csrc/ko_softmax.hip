@@ -1,5 +1,6 @@
 // Row softmax for gfx950: one pass over HBM (each element read once, written
-// once), fp32, optional per-sequence padding mask.
+// once), fp32 arithmetic, fp32 / binary16 / bfloat16 storage, optional
+// per-sequence padding mask.
 //
 // Three mappings, the counterparts of the reference's three policies
 // (nn_operators/softmax/softmax.h):
@@ -31,38 +32,48 @@ namespace {
 
 constexpr float kMaskValue = -10000.0f;
 
-// Loads vector j (columns 4j..4j+3) of a row whose first `vlen` columns are valid.
-template <bool MASKED, bool NT>
-__device__ __forceinline__ float4v load_row_vec(const float *row, int j, int vlen) {
-    const int c = 4 * j;
+// Loads vector j (columns E*j .. E*j+E-1) of a row whose first `vlen` columns are valid.
+template <int IO, bool MASKED, bool NT>
+__device__ __forceinline__ void load_row_vec(const typename Io<IO>::elem *row, int j, int vlen,
+                                             float (&v)[Io<IO>::E]) {
+    constexpr int E = Io<IO>::E;
+    const int c = E * j;
     if constexpr (!MASKED) {
-        return load4<NT>(row + c);
+        Io<IO>::template load<NT>(row + c, v);
     } else {
-        float4v v = {kMaskValue, kMaskValue, kMaskValue, kMaskValue};
         if (c < vlen) {
-            float4v x = load4<NT>(row + c);
-            v[0] = x[0];
-            if (c + 1 < vlen) v[1] = x[1];
-            if (c + 2 < vlen) v[2] = x[2];
-            if (c + 3 < vlen) v[3] = x[3];
+            Io<IO>::template load<NT>(row + c, v);
+#pragma unroll
+            for (int e = 1; e < E; ++e)
+                if (c + e >= vlen) v[e] = kMaskValue;
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = kMaskValue;
         }
-        return v;
     }
+}
+
+template <int E>
+__device__ __forceinline__ float vec_max(const float (&v)[E], float m) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) m = fmaxf(m, v[e]);
+    return m;
 }
 
 __device__ __forceinline__ int clamp_len(int v, int cols) { return v < 0 ? 0 : (v > cols ? cols : v); }
 
 // ---------------------------------------------------------------- WARP policy
-template <int LPR, int VPL, bool MASKED, bool NT>
-__global__ __launch_bounds__(256) void softmax_wave_kernel(const float *in,
-                                                           float *out, int64_t rows,
+template <int IO, int LPR, int VPL, bool MASKED, bool NT>
+__global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>::elem *in,
+                                                           typename Io<IO>::elem *out, int64_t rows,
                                                            int cols, const int32_t *__restrict__ valid_len,
                                                            int64_t rows_per_seq) {
+    constexpr int E = Io<IO>::E;
     constexpr int RPW = 64 / LPR;  // rows per wavefront
     const int lane = threadIdx.x & 63;
     const int sub = lane / LPR;
     const int l = lane % LPR;
-    const int nvec = cols >> 2;
+    const int nvec = cols / E;
     const int64_t waves_per_block = blockDim.x >> 6;
     const int64_t wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
     const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * RPW;
@@ -70,45 +81,58 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const float *in,
     for (int64_t row0 = wave * RPW; row0 < rows; row0 += stride) {
         const int64_t row = row0 + sub;
         const bool row_ok = row < rows;
-        const float *src = in + row * cols;
+        const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) {
             if (row_ok) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
         }
 
-        float4v v[VPL];
+        float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
             if (row_ok && j < nvec) {
-                v[k] = load_row_vec<MASKED, NT>(src, j, vlen);
+                load_row_vec<IO, MASKED, NT>(src, j, vlen, v[k]);
             } else {
-                v[k] = float4v{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
             }
         }
 
         float m = -FLT_MAX;
 #pragma unroll
-        for (int k = 0; k < VPL; ++k) m = fmaxf(fmaxf(fmaxf(m, v[k][0]), fmaxf(v[k][1], v[k][2])), v[k][3]);
+        for (int k = 0; k < VPL; ++k) m = vec_max<E>(v[k], m);
         m = wave::allreduce<LPR, wave::Max>(m);
 
+        // Vectors wholly inside the padding hold -10000; once the row maximum is more than 128 above
+        // that, their exponentials are exactly zero in fp32 and need not be computed.
+        const bool pad_is_zero = MASKED && m > kMaskValue + 128.0f;
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
+            if (pad_is_zero && E * (l + k * LPR) >= vlen) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[k][e] = exp_nonpositive(v[k][e] - m);
-                s += v[k][e];
+                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    v[k][e] = exp_for_storage<IO>(v[k][e] - m);
+                    s += v[k][e];
+                }
             }
         }
         s = wave::allreduce<LPR, wave::Sum>(s);
         const float inv = 1.0f / s;
 
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            if (row_ok && j < nvec) store4<NT>(dst + 4 * j, v[k] * inv);
+            if (row_ok && j < nvec) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] *= inv;
+                Io<IO>::template store<NT>(dst + E * j, v[k]);
+            }
         }
     }
 }
@@ -130,45 +154,60 @@ __device__ __forceinline__ float block_allreduce(float v, float *lds, float iden
     return r;
 }
 
-template <int THREADS, int VPL, bool MASKED, bool NT>
-__global__ __launch_bounds__(THREADS) void softmax_block_kernel(const float *in,
-                                                                float *out, int64_t rows,
+template <int IO, int THREADS, int VPL, bool MASKED>
+__global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename Io<IO>::elem *in,
+                                                                typename Io<IO>::elem *out, int64_t rows,
                                                                 int cols,
                                                                 const int32_t *__restrict__ valid_len,
                                                                 int64_t rows_per_seq) {
+    constexpr int E = Io<IO>::E;
     __shared__ float lds[16];
-    const int nvec = cols >> 2;
+    const int nvec = cols / E;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        const float *src = in + row * cols;
+        const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
-        float4v v[VPL];
+        float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
-            if (j < nvec) v[k] = load_row_vec<MASKED, NT>(src, j, vlen);
-            else v[k] = float4v{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+            if (j < nvec) {
+                load_row_vec<IO, MASKED, false>(src, j, vlen, v[k]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+            }
         }
         float m = -FLT_MAX;
 #pragma unroll
-        for (int k = 0; k < VPL; ++k) m = fmaxf(fmaxf(fmaxf(m, v[k][0]), fmaxf(v[k][1], v[k][2])), v[k][3]);
+        for (int k = 0; k < VPL; ++k) m = vec_max<E>(v[k], m);
         m = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
+        const bool pad_is_zero = MASKED && m > kMaskValue + 128.0f;  // see the wave kernel
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
+            if (pad_is_zero && E * (static_cast<int>(threadIdx.x) + k * THREADS) >= vlen) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[k][e] = exp_nonpositive(v[k][e] - m);
-                s += v[k][e];
+                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    v[k][e] = exp_for_storage<IO>(v[k][e] - m);
+                    s += v[k][e];
+                }
             }
         }
         s = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
         const float inv = 1.0f / s;
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
-            if (j < nvec) store4<NT>(dst + 4 * j, v[k] * inv);
+            if (j < nvec) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] *= inv;
+                Io<IO>::template store<false>(dst + E * j, v[k]);
+            }
         }
     }
 }
@@ -184,42 +223,46 @@ __device__ __forceinline__ void online_add(float &m, float &s, float x) {
     }
 }
 
-template <int THREADS, bool MASKED>
-__global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const float *in,
-                                                                  float *out,
+template <int IO, int THREADS, bool MASKED>
+__global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename Io<IO>::elem *in,
+                                                                  typename Io<IO>::elem *out,
                                                                   int64_t rows, int cols,
                                                                   const int32_t *__restrict__ valid_len,
                                                                   int64_t rows_per_seq) {
+    constexpr int E = Io<IO>::E;
     __shared__ float lds[16];
-    const int nvec = cols >> 2;
+    const int nvec = cols / E;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        const float *src = in + row * cols;
+        const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
         float m = -FLT_MAX, s = 0.0f;
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load_row_vec<MASKED, false>(src, j, vlen);
+            float x[E];
+            load_row_vec<IO, MASKED, false>(src, j, vlen, x);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) online_add(m, s, x[e]);
+            for (int e = 0; e < E; ++e) online_add(m, s, x[e]);
         }
         const float gm = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
         s *= exp_nonpositive(m - gm);  // threads that saw nothing: s = 0
         const float gs = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
         const float inv = 1.0f / gs;
-        float *dst = out + row * cols;
+        typename Io<IO>::elem *dst = out + row * cols;
         for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float4v x = load_row_vec<MASKED, false>(src, j, vlen);
+            float x[E];
+            load_row_vec<IO, MASKED, false>(src, j, vlen, x);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] = exp_nonpositive(x[e] - gm) * inv;
-            store4<false>(dst + 4 * j, x);
+            for (int e = 0; e < E; ++e) x[e] = exp_for_storage<IO>(x[e] - gm) * inv;
+            Io<IO>::template store<false>(dst + E * j, x);
         }
     }
 }
 
 // ------------------------------------------------------------------ dispatch
+template <int IO>
 struct Args {
-    const float *in;
-    float *out;
+    const typename Io<IO>::elem *in;
+    typename Io<IO>::elem *out;
     int64_t rows;
     int cols;
     const int32_t *valid_len;
@@ -227,8 +270,8 @@ struct Args {
     hipStream_t stream;
 };
 
-template <int LPR, int VPL, bool MASKED, bool NT>
-int launch_wave(const Args &a) {
+template <int IO, int LPR, int VPL, bool MASKED, bool NT>
+int launch_wave(const Args<IO> &a) {
     constexpr int RPW = 64 / LPR;
     // Single-wavefront workgroups by default (measured 1-4 % faster than 256 threads: the dispatcher
     // places waves more freely); the knob selects 128 or 256.
@@ -243,70 +286,88 @@ int launch_wave(const Args &a) {
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    softmax_wave_kernel<LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    softmax_wave_kernel<IO, LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
 
-template <int LPR, bool MASKED, bool NT>
-int launch_wave_vpl(const Args &a, int vpl) {
+template <int IO, int LPR, bool MASKED, bool NT>
+int launch_wave_vpl(const Args<IO> &a, int vpl) {
     switch (vpl) {
-        case 1: return launch_wave<LPR, 1, MASKED, NT>(a);
-        case 2: return launch_wave<LPR, 2, MASKED, NT>(a);
-        case 3: return launch_wave<LPR, 3, MASKED, NT>(a);
-        case 4: return launch_wave<LPR, 4, MASKED, NT>(a);
+        case 1: return launch_wave<IO, LPR, 1, MASKED, NT>(a);
+        case 2: return launch_wave<IO, LPR, 2, MASKED, NT>(a);
+        case 3: return launch_wave<IO, LPR, 3, MASKED, NT>(a);
+        case 4: return launch_wave<IO, LPR, 4, MASKED, NT>(a);
         case 5:
-        case 6: return launch_wave<LPR, 6, MASKED, NT>(a);
-        default: return launch_wave<LPR, 8, MASKED, NT>(a);
+        case 6: return launch_wave<IO, LPR, 6, MASKED, NT>(a);
+        default: return launch_wave<IO, LPR, 8, MASKED, NT>(a);
     }
 }
 
-template <bool MASKED, bool NT>
-int launch_wave_lpr(const Args &a, int lpr) {
-    const int nvec = a.cols / 4;
+template <int IO, bool MASKED, bool NT>
+int launch_wave_lpr(const Args<IO> &a, int lpr) {
+    const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + lpr - 1) / lpr;
     switch (lpr) {
-        case 8: return launch_wave_vpl<8, MASKED, NT>(a, vpl);
-        case 16: return launch_wave_vpl<16, MASKED, NT>(a, vpl);
-        case 32: return launch_wave_vpl<32, MASKED, NT>(a, vpl);
-        default: return launch_wave_vpl<64, MASKED, NT>(a, vpl);
+        case 8: return launch_wave_vpl<IO, 8, MASKED, NT>(a, vpl);
+        case 16: return launch_wave_vpl<IO, 16, MASKED, NT>(a, vpl);
+        case 32: return launch_wave_vpl<IO, 32, MASKED, NT>(a, vpl);
+        default: return launch_wave_vpl<IO, 64, MASKED, NT>(a, vpl);
     }
 }
 
 constexpr int kWaveMaxVpl = 8;
-constexpr int kWaveMaxCols = 64 * kWaveMaxVpl * 4;    // 2048
-constexpr int kBlockMaxCols = 1024 * 8 * 4;           // 32768
+// Longest row per policy, in 16-byte vectors: 512 per wavefront, 8192 per workgroup
+// (fp32: 2048 and 32768 columns; 16-bit: twice that).
+constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
+constexpr int kBlockMaxVecs = 1024 * 8;
 
-// Lanes per row for the WARP policy: the narrowest group that gives every lane at most
-// one vector, so that one load instruction of the group covers the row contiguously;
-// rows longer than 64 vectors take the whole wavefront and several vectors per lane.
-int default_lanes_per_row(int cols) {
-    const int nvec = cols / 4;
-    int lpr = 8;
-    while (lpr < 64 && lpr < nvec) lpr <<= 1;
-    return lpr;
+// Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
+// {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
+// and a wavefront's worth of latency), and among equals takes the widest group: one load instruction
+// of the group then covers the longest contiguous piece of the row.  With a padding mask at least two
+// vectors per lane are preferred: a lane whose only vector lies in the padding idles through the whole
+// row (measured on [786432, 512] binary16, mean valid length 288: 64 x 1 309 us, 32 x 2 230 us).
+int default_lanes_per_row(int nvec, bool masked) {
+    int best = 64, best_waste = 1 << 30;
+    for (int lpr = 8; lpr <= 64; lpr <<= 1) {
+        int vpl = (nvec + lpr - 1) / lpr;
+        if (vpl > 8) continue;
+        if (vpl == 5) vpl = 6;
+        if (vpl == 7) vpl = 8;
+        const int waste = lpr * vpl - nvec;
+        if (waste < best_waste || (waste == best_waste && !(masked && vpl < 2))) {
+            best_waste = waste;
+            best = lpr;
+        }
+    }
+    return best;
 }
 
-template <bool MASKED>
-int launch_wave_any(const Args &a) {
+template <int IO, bool MASKED>
+int launch_wave_any(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     int lpr = tuning("softmax.lanes_per_row");
-    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(a.cols);
-    while (lpr < 64 && (a.cols / 4 + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
-    // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off.
-    if (tuning("softmax.nontemporal") == 2) return launch_wave_lpr<MASKED, false>(a, lpr);
-    return launch_wave_lpr<MASKED, true>(a, lpr);
+    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec, MASKED);
+    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off
+    // (fp32 storage only; the 16-bit kernels are built with streaming accesses).
+    if constexpr (IO == IO_F32) {
+        if (tuning("softmax.nontemporal") == 2) return launch_wave_lpr<IO, MASKED, false>(a, lpr);
+    }
+    return launch_wave_lpr<IO, MASKED, true>(a, lpr);
 }
 
-template <int THREADS, bool MASKED>
-int launch_block_threads(const Args &a) {
-    const int nvec = a.cols / 4;
+template <int IO, int THREADS, bool MASKED>
+int launch_block_threads(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + THREADS - 1) / THREADS;
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
     if (grid > a.rows) grid = a.rows;
     dim3 g(static_cast<unsigned>(grid)), b(THREADS);
 #define KO_SM_BLOCK(V)                                                                         \
-    softmax_block_kernel<THREADS, V, MASKED, false><<<g, b, 0, a.stream>>>(                      \
+    softmax_block_kernel<IO, THREADS, V, MASKED><<<g, b, 0, a.stream>>>(                         \
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq)
     if (vpl <= 1) KO_SM_BLOCK(1);
     else if (vpl <= 2) KO_SM_BLOCK(2);
@@ -317,54 +378,77 @@ int launch_block_threads(const Args &a) {
     return KO_OK;
 }
 
-template <bool MASKED>
-int launch_block(const Args &a) {
-    const int nvec = a.cols / 4;
+template <int IO, bool MASKED>
+int launch_block(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
     int threads = tuning("softmax.block_threads");
     if (threads != 256 && threads != 512 && threads != 1024) {
         threads = 256;
         while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;
     }
     while (threads < 1024 && (nvec + threads - 1) / threads > 8) threads <<= 1;
-    if (threads == 256) return launch_block_threads<256, MASKED>(a);
-    if (threads == 512) return launch_block_threads<512, MASKED>(a);
-    return launch_block_threads<1024, MASKED>(a);
+    if (threads == 256) return launch_block_threads<IO, 256, MASKED>(a);
+    if (threads == 512) return launch_block_threads<IO, 512, MASKED>(a);
+    return launch_block_threads<IO, 1024, MASKED>(a);
 }
 
-template <bool MASKED>
-int launch_nocache(const Args &a) {
+template <int IO, bool MASKED>
+int launch_nocache(const Args<IO> &a) {
     constexpr int kThreads = 1024;
     int64_t grid = static_cast<int64_t>(compute_units()) * 4;
     if (grid > a.rows) grid = a.rows;
-    softmax_nocache_kernel<kThreads, MASKED><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    softmax_nocache_kernel<IO, kThreads, MASKED><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
 
-template <bool MASKED>
-int dispatch(const Args &a, int policy) {
+template <int IO, bool MASKED>
+int dispatch(const Args<IO> &a, int policy) {
+    constexpr int E = Io<IO>::E;
+    const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
-        policy = a.cols <= kWaveMaxCols ? KO_POLICY_WARP
-                 : a.cols <= kBlockMaxCols ? KO_POLICY_BLOCK
-                                           : KO_POLICY_BLOCK_NOCACHE;
+        policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
+                 : nvec <= kBlockMaxVecs ? KO_POLICY_BLOCK
+                                         : KO_POLICY_BLOCK_NOCACHE;
     }
     switch (policy) {
         case KO_POLICY_WARP:
-            if (a.cols > kWaveMaxCols)
+            if (nvec > kWaveMaxVecs)
                 return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "softmax: WARP policy holds at most %d columns per row, got %d", kWaveMaxCols,
+                            "softmax: WARP policy holds at most %d columns per row, got %d", kWaveMaxVecs * E,
                             a.cols);
-            return launch_wave_any<MASKED>(a);
+            return launch_wave_any<IO, MASKED>(a);
         case KO_POLICY_BLOCK:
-            if (a.cols > kBlockMaxCols)
+            if (nvec > kBlockMaxVecs)
                 return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxCols,
+                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs * E,
                             a.cols);
-            return launch_block<MASKED>(a);
-        case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<MASKED>(a);
+            return launch_block<IO, MASKED>(a);
+        case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO, MASKED>(a);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "softmax: unknown policy %d", policy);
     }
+}
+
+template <int IO>
+int entry(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *valid_len, int64_t rows_per_seq,
+          int policy, ko_stream_t stream) {
+    constexpr int E = Io<IO>::E;
+    if (rows < 0 || cols <= 0)
+        return fail(KO_ERR_INVALID_ARGUMENT, "softmax: rows=%lld cols=%lld", (long long)rows, (long long)cols);
+    if (cols % E != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld is not a multiple of the vector width %d",
+                    (long long)cols, E);
+    if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld too large", (long long)cols);
+    if (rows == 0) return KO_OK;
+    if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "softmax: null in/out pointer");
+    if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15)
+        return fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be 16-byte aligned");
+    if (valid_len && rows_per_seq <= 0)
+        return fail(KO_ERR_INVALID_ARGUMENT, "softmax: valid_len given but rows_per_seq=%lld", (long long)rows_per_seq);
+    Args<IO> a{static_cast<const typename Io<IO>::elem *>(in), static_cast<typename Io<IO>::elem *>(out), rows,
+               static_cast<int>(cols), valid_len, rows_per_seq, as_stream(stream)};
+    return valid_len ? dispatch<IO, true>(a, policy) : dispatch<IO, false>(a, policy);
 }
 
 }  // namespace
@@ -373,27 +457,19 @@ int dispatch(const Args &a, int policy) {
 KO_EXPORT int ko_softmax_f32_policy(const float *in, float *out, int64_t rows, int64_t cols,
                                     const int32_t *valid_len, int64_t rows_per_seq, int policy,
                                     ko_stream_t stream) {
-    if (rows < 0 || cols <= 0)
-        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: rows=%lld cols=%lld", (long long)rows,
-                        (long long)cols);
-    if (cols % 4 != 0)
-        return ko::fail(KO_ERR_UNSUPPORTED_SHAPE,
-                        "softmax: cols=%lld is not a multiple of the vector width 4", (long long)cols);
-    if (cols > (1 << 30)) return ko::fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld too large", (long long)cols);
-    if (rows == 0) return KO_OK;
-    if (!in || !out) return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: null in/out pointer");
-    if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15)
-        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be 16-byte aligned");
-    if (valid_len && rows_per_seq <= 0)
-        return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: valid_len given but rows_per_seq=%lld",
-                        (long long)rows_per_seq);
-    ko::Args a{in, out, rows, static_cast<int>(cols), valid_len, rows_per_seq, ko::as_stream(stream)};
-    return valid_len ? ko::dispatch<true>(a, policy) : ko::dispatch<false>(a, policy);
+    return ko::entry<ko::IO_F32>(in, out, rows, cols, valid_len, rows_per_seq, policy, stream);
 }
 
 KO_EXPORT int ko_softmax_f32(const float *in, float *out, int64_t rows, int64_t cols,
                              const int32_t *valid_len, int64_t rows_per_seq, ko_stream_t stream) {
     return ko_softmax_f32_policy(in, out, rows, cols, valid_len, rows_per_seq, KO_POLICY_AUTO, stream);
+}
+
+KO_EXPORT int ko_softmax_16(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *valid_len,
+                            int64_t rows_per_seq, int dtype, int policy, ko_stream_t stream) {
+    if (dtype == KO_F16) return ko::entry<ko::IO_F16>(in, out, rows, cols, valid_len, rows_per_seq, policy, stream);
+    if (dtype == KO_BF16) return ko::entry<ko::IO_BF16>(in, out, rows, cols, valid_len, rows_per_seq, policy, stream);
+    return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: dtype=%d is neither KO_F16 nor KO_BF16", dtype);
 }
 
 // ---- cross-lane primitive check (see ko.h)

@@ -144,10 +144,62 @@ __device__ __forceinline__ Welford welford_allreduce(Welford w) {
     return w;
 }
 
+// The same all-reduce when every lane of the group enters with the same count c (rows whose length is a
+// whole number of vectors per lane): n = 2c at every step, so mean = (ma + mb) / 2 and
+// M2 = (M2a + M2b) + (mb - ma)^2 * c / 2 - Chan's merge with the counts folded into constants, no
+// division, and only two values to exchange.  Symmetric in a and b like the general form.
+__device__ __forceinline__ void welford_merge_equal(float &mean, float &m2, float pmean, float pm2, float half_c) {
+    const float d = pmean - mean;
+    mean = 0.5f * (mean + pmean);
+    m2 = __builtin_fmaf(d * d, half_c, m2 + pm2);
+}
+
+template <int G>
+__device__ __forceinline__ Welford welford_allreduce_equal(Welford w) {
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "");
+    float half_c = 0.5f * w.count;
+    if constexpr (G >= 2) {
+        welford_merge_equal(w.mean, w.m2, dpp<kDppQuadXor1>(w.mean), dpp<kDppQuadXor1>(w.m2), half_c);
+        half_c *= 2.0f;
+    }
+    if constexpr (G >= 4) {
+        welford_merge_equal(w.mean, w.m2, dpp<kDppQuadXor2>(w.mean), dpp<kDppQuadXor2>(w.m2), half_c);
+        half_c *= 2.0f;
+    }
+    if constexpr (G >= 8) {
+        welford_merge_equal(w.mean, w.m2, dpp<kDppRowHalfMirror>(w.mean), dpp<kDppRowHalfMirror>(w.m2), half_c);
+        half_c *= 2.0f;
+    }
+    if constexpr (G >= 16) {
+        welford_merge_equal(w.mean, w.m2, dpp<kDppRowMirror>(w.mean), dpp<kDppRowMirror>(w.m2), half_c);
+        half_c *= 2.0f;
+    }
+    if constexpr (G >= 32) {
+        float am, bm, a2, b2;
+        swap16(w.mean, am, bm);
+        swap16(w.m2, a2, b2);
+        welford_merge_equal(am, a2, bm, b2, half_c);
+        w.mean = am;
+        w.m2 = a2;
+        half_c *= 2.0f;
+    }
+    if constexpr (G >= 64) {
+        float am, bm, a2, b2;
+        swap32(w.mean, am, bm);
+        swap32(w.m2, a2, b2);
+        welford_merge_equal(am, a2, bm, b2, half_c);
+        w.mean = am;
+        w.m2 = a2;
+    }
+    w.count *= static_cast<float>(G);
+    return w;
+}
+
 }  // namespace wave
 
 // 128-bit global accesses, optionally non-temporal (streaming: data is touched once).
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 template <bool NT>
 __device__ __forceinline__ float4v load4(const float *p) {
@@ -162,6 +214,98 @@ __device__ __forceinline__ void store4(float *p, float4v v) {
     if constexpr (NT) __builtin_nontemporal_store(v, q);
     else *q = v;
 }
+
+// Storage types of the row operators.  The arithmetic is always fp32; a 16-byte vector holds
+// E = 4 floats or E = 8 binary16 / bfloat16 values, converted on load and rounded (to nearest
+// even) once on store.  The reference carries half specialisations of its functors for the same
+// purpose (common/functors.h:71-77,105-111, common/common.h:171-177).
+enum { IO_F32 = 0, IO_F16 = 1, IO_BF16 = 2 };
+
+template <int IO>
+struct Io;
+
+template <>
+struct Io<IO_F32> {
+    typedef float elem;
+    static constexpr int E = 4;
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        const float4v x = load4<NT>(p);
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] = x[e];
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
+        store4<NT>(p, float4v{v[0], v[1], v[2], v[3]});
+    }
+    static __device__ __forceinline__ float scalar(const elem *p) { return *p; }
+};
+
+template <bool NT>
+__device__ __forceinline__ uint4v load_bits16(const uint16_t *p) {
+    const uint4v *q = reinterpret_cast<const uint4v *>(p);
+    if constexpr (NT) return __builtin_nontemporal_load(q);
+    return *q;
+}
+
+template <bool NT>
+__device__ __forceinline__ void store_bits16(uint16_t *p, uint4v v) {
+    uint4v *q = reinterpret_cast<uint4v *>(p);
+    if constexpr (NT) __builtin_nontemporal_store(v, q);
+    else *q = v;
+}
+
+template <>
+struct Io<IO_F16> {
+    typedef uint16_t elem;
+    static constexpr int E = 8;
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        const half8 h = __builtin_bit_cast(half8, load_bits16<NT>(p));
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] = static_cast<float>(h[e]);
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < E; ++e) h[e] = static_cast<_Float16>(v[e]);
+        store_bits16<NT>(p, __builtin_bit_cast(uint4v, h));
+    }
+    static __device__ __forceinline__ float scalar(const elem *p) {
+        return static_cast<float>(__builtin_bit_cast(_Float16, *p));
+    }
+};
+
+template <>
+struct Io<IO_BF16> {
+    typedef uint16_t elem;
+    static constexpr int E = 8;
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        const uint4v x = load_bits16<NT>(p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[2 * e] = __builtin_bit_cast(float, x[e] << 16);
+            v[2 * e + 1] = __builtin_bit_cast(float, x[e] & 0xffff0000u);
+        }
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
+        // float -> bfloat16, round to nearest even: v_cvt_pk_bf16_f32, two values per instruction
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        uint4v x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            x[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{v[2 * e], v[2 * e + 1]}, bf16x2));
+        store_bits16<NT>(p, x);
+    }
+    static __device__ __forceinline__ float scalar(const elem *p) {
+        return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
+    }
+};
 
 // exp(d) for d <= 0, about 1 ulp: d*log2(e) is formed as a rounded product plus its
 // exact residual and the low part of log2(e), the integer part is split off and
@@ -178,6 +322,20 @@ __device__ __forceinline__ float exp_nonpositive(float d) {
     float f = (y - n) + r;
     float e = __builtin_amdgcn_exp2f(f);
     return __builtin_ldexpf(e, static_cast<int>(n));
+}
+
+// exp(d) for d <= 0 where the result is rounded to a 16-bit storage type afterwards: one rounded product
+// and the hardware exponential (with the compiler's scaling for results below the normal range).  The
+// product's rounding costs |d| * log2(e) * 2^-24 relative, about 3.5e-6 at d = -40: far inside half an
+// ulp of binary16 (4.9e-4) or bfloat16 (3.9e-3).
+__device__ __forceinline__ float exp_nonpositive_fast(float d) {
+    return __builtin_exp2f(fmaxf(d, -150.0f) * 0x1.715476p+0f);
+}
+
+template <int IO>
+__device__ __forceinline__ float exp_for_storage(float d) {
+    if constexpr (IO == IO_F32) return exp_nonpositive(d);
+    else return exp_nonpositive_fast(d);
 }
 
 }  // namespace ko

@@ -94,6 +94,35 @@ static int gpu_part() {
         REQUIRE(std::fabs(rstd.host_ref<float>()[1] - 1.0 / std::sqrt((768.0 * 768.0 - 1) / 12)) < 1e-8);
     }
     {
+        // 16-bit storage through the same templates: constant rows give exactly 1/C (softmax) and beta (LayerNorm)
+        constexpr int R = 8, C = 128;
+        Tensor in(R * C * 2), out(R * C * 2), beta(C * 2), mean(R * 4);
+        for (int i = 0; i < R * C; ++i) in.host_ref<half>()[i] = half(1.5f);
+        for (int i = 0; i < C; ++i) beta.host_ref<half>()[i] = half(float(i) / 8);
+        in.host_to_device();
+        beta.host_to_device();
+        softmax<SoftMaxWarpImpl<half, 8, R, C>>(320, 128, 0, stream, in.device_ref<half>(), out.device_ref<half>());
+        checkKoErrors(ko_stream_synchronize(stream));
+        out.device_to_host();
+        for (int i = 0; i < R * C; ++i) REQUIRE(float(out.host_ref<half>()[i]) == 1.0f / C);
+        layer_normalization<LayerNormWarpImpl<half, 8, R, C, true>>(320, 128, 0, stream, in.device_ref<half>(),
+                                                                    out.device_ref<half>(), half(1e-5f), nullptr,
+                                                                    beta.device_ref<half>(), mean.device_ref<float>());
+        checkKoErrors(ko_stream_synchronize(stream));
+        out.device_to_host();
+        mean.device_to_host();
+        for (int i = 0; i < R * C; ++i) REQUIRE(float(out.host_ref<half>()[i]) == float(i % C) / 8);
+        REQUIRE(mean.host_ref<float>()[3] == 1.5f);
+        Tensor inb(R * C * 2), outb(R * C * 2);
+        for (int i = 0; i < R * C; ++i) inb.host_ref<ko_bfloat16>()[i] = ko_bfloat16(-2.0f);
+        inb.host_to_device();
+        softmax<SoftMaxBlockImpl<ko_bfloat16, 8, R, C>>(320, 128, 0, stream, inb.device_ref<ko_bfloat16>(),
+                                                        outb.device_ref<ko_bfloat16>());
+        checkKoErrors(ko_stream_synchronize(stream));
+        outb.device_to_host();
+        for (int i = 0; i < R * C; ++i) REQUIRE(float(outb.host_ref<ko_bfloat16>()[i]) == 1.0f / C);
+    }
+    {
         constexpr int N = 128;
         Tensor A(N * N * 4), B(N * N * 4), C(N * N * 4), D(N * N * 4);
         for (int i = 0; i < N * N; ++i) {

@@ -51,6 +51,9 @@ def lib():
                                        ctypes.c_double, _f32p, _f32p, _f64p]
         L.oracle_gemm_16.argtypes = [_i64, _i64, _i64, ctypes.c_double, _u16p, _u16p, ctypes.c_int,
                                      ctypes.c_double, _u16p, _u16p, ctypes.c_int, _f64p, _f64p]
+        L.oracle_softmax_16.argtypes = [_u16p, _u16p, _f64p, _i64, _i64, _i32p, _i64, ctypes.c_int]
+        L.oracle_layernorm_16.argtypes = [_u16p, _u16p, _f64p, _f32p, _f32p, _u16p, _u16p, _i64, _i64,
+                                          ctypes.c_double, ctypes.c_int, ctypes.c_int]
         for name in ("oracle_f16_to_f64", "oracle_bf16_to_f64"):
             getattr(L, name).argtypes = [_u16p, _f64p, _i64]
         for name in ("oracle_f64_to_f16", "oracle_f64_to_bf16"):
@@ -119,6 +122,37 @@ def layernorm_welford(x, gamma=None, beta=None, eps=1e-5, unbiased=False, lanes=
     if rc:
         raise ValueError("oracle_layernorm_welford_f32: bad arguments")
     return y, mean, rstd
+
+
+def softmax16(x_bits, valid_len=None, rows_per_seq=0, bf16=False):
+    """Row softmax on 16-bit storage (uint16 bit patterns [rows, cols]).  Returns (y_bits, y_float64)."""
+    x_bits = _c(x_bits, np.uint16)
+    rows, cols = x_bits.shape
+    out = np.empty_like(x_bits)
+    out64 = np.empty(x_bits.shape, np.float64)
+    vl = _c(valid_len, np.int32)
+    rc = lib().oracle_softmax_16(_ptr(x_bits, _u16p), _ptr(out, _u16p), _ptr(out64, _f64p), rows, cols,
+                                 _ptr(vl, _i32p), int(rows_per_seq), int(bool(bf16)))
+    if rc:
+        raise ValueError("oracle_softmax_16: bad arguments")
+    return out, out64
+
+
+def layernorm16(x_bits, gamma_bits=None, beta_bits=None, eps=1e-5, unbiased=False, bf16=False):
+    """LayerNorm on 16-bit storage.  Returns (y_bits, y_float64, mean float32, rstd float32)."""
+    x_bits = _c(x_bits, np.uint16)
+    rows, cols = x_bits.shape
+    out = np.empty_like(x_bits)
+    out64 = np.empty(x_bits.shape, np.float64)
+    mean = np.empty(rows, np.float32)
+    rstd = np.empty(rows, np.float32)
+    g, b = _c(gamma_bits, np.uint16), _c(beta_bits, np.uint16)
+    rc = lib().oracle_layernorm_16(_ptr(x_bits, _u16p), _ptr(out, _u16p), _ptr(out64, _f64p), _ptr(mean, _f32p),
+                                   _ptr(rstd, _f32p), _ptr(g, _u16p), _ptr(b, _u16p), rows, cols, float(eps),
+                                   int(bool(unbiased)), int(bool(bf16)))
+    if rc:
+        raise ValueError("oracle_layernorm_16: bad arguments")
+    return out, out64, mean, rstd
 
 
 def sgemm(A, B, C=None, alpha=1.0, beta=0.0, want_absprod=False):

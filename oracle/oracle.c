@@ -238,6 +238,80 @@ ORACLE_API int oracle_layernorm_f32(const float *in, float *out, float *mean_out
     return 0;
 }
 
+/*
+ * The same two operators on 16-bit storage (binary16 or bfloat16 bit patterns; gamma and beta
+ * in the same type): inputs are widened exactly, the arithmetic is the double arithmetic above,
+ * and the result is rounded once to the storage type.  out64 (optional) receives the unrounded
+ * values.  The reference carries half specialisations of its functors for this case
+ * (common/functors.h:71-77,105-111).
+ */
+static double bits16_to_double(uint16_t b, int bf16) { return bf16 ? bf16_bits_to_double(b) : f16_bits_to_double(b); }
+static uint16_t double_to_bits16(double d, int bf16) { return bf16 ? double_to_bf16_bits(d) : double_to_f16_bits(d); }
+
+ORACLE_API int oracle_softmax_16(const uint16_t *in, uint16_t *out, double *out64, int64_t rows, int64_t cols,
+                                 const int32_t *valid_len, int64_t rows_per_seq, int bf16) {
+    if (rows < 0 || cols <= 0) return 1;
+    if (valid_len && rows_per_seq <= 0) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const uint16_t *x = in + r * cols;
+        int64_t vl = cols;
+        if (valid_len) {
+            vl = valid_len[r / rows_per_seq];
+            if (vl < 0) vl = 0;
+            if (vl > cols) vl = cols;
+        }
+        double mx = -(double)FLT_MAX;
+        for (int64_t j = 0; j < cols; ++j) {
+            double v = j < vl ? bits16_to_double(x[j], bf16) : ORACLE_MASK_VALUE;
+            if (v > mx) mx = v;
+        }
+        double sum = 0.0;
+        for (int64_t j = 0; j < cols; ++j) {
+            double v = j < vl ? bits16_to_double(x[j], bf16) : ORACLE_MASK_VALUE;
+            sum += exp(v - mx);
+        }
+        for (int64_t j = 0; j < cols; ++j) {
+            double v = j < vl ? bits16_to_double(x[j], bf16) : ORACLE_MASK_VALUE;
+            double y = exp(v - mx) / sum;
+            if (out64) out64[r * cols + j] = y;
+            if (out) out[r * cols + j] = double_to_bits16(y, bf16);
+        }
+    }
+    return 0;
+}
+
+ORACLE_API int oracle_layernorm_16(const uint16_t *in, uint16_t *out, double *out64, float *mean_out,
+                                   float *rstd_out, const uint16_t *gamma, const uint16_t *beta, int64_t rows,
+                                   int64_t cols, double eps, int unbiased, int bf16) {
+    if (rows < 0 || cols <= 0) return 1;
+    if (unbiased && cols < 2) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const uint16_t *x = in + r * cols;
+        double s = 0.0;
+        for (int64_t j = 0; j < cols; ++j) s += bits16_to_double(x[j], bf16);
+        double mean = s / (double)cols;
+        double m2 = 0.0;
+        for (int64_t j = 0; j < cols; ++j) {
+            double d = bits16_to_double(x[j], bf16) - mean;
+            m2 += d * d;
+        }
+        double var = m2 / (double)(unbiased ? cols - 1 : cols);
+        double rstd = 1.0 / sqrt(var + eps);
+        for (int64_t j = 0; j < cols; ++j) {
+            double v = (bits16_to_double(x[j], bf16) - mean) * rstd;
+            if (gamma) v *= bits16_to_double(gamma[j], bf16);
+            if (beta) v += bits16_to_double(beta[j], bf16);
+            if (out64) out64[r * cols + j] = v;
+            if (out) out[r * cols + j] = double_to_bits16(v, bf16);
+        }
+        if (mean_out) mean_out[r] = (float)mean;
+        if (rstd_out) rstd_out[r] = (float)rstd;
+    }
+    return 0;
+}
+
 /* Welford triplets in float, as the reference keeps them (count is a float). */
 static void welford_update_f32(float *count, float *mean, float *m2, float v) {
     /* nn_operators/layernorm/layernorm.h:13-23 */

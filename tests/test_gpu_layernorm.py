@@ -26,18 +26,18 @@ def test_layernorm_matches_oracle(ko, rows, cols, unbiased):
 
 
 @pytest.mark.parametrize("lpr", [8, 16, 32, 64])
-@pytest.mark.parametrize("cols", [128, 768])
+@pytest.mark.parametrize("cols", [128, 768, 1024, 200])
 def test_layernorm_every_lane_mapping(ko, lpr, cols):
+    """Every group width, on row lengths that fill the lanes evenly (equal-count merge: 128 with 8/16/32 lanes,
+    768 and 1024 with 64) and on ones that do not (general merge with ragged per-lane counts)."""
     x, g, b = _case(517, cols, 31 + lpr)
     ref = oracle.layernorm(x, g, b)
     ko.set_tuning("layernorm.lanes_per_row", lpr)
     try:
-        for nt in (1, 2):  # streaming accesses on / off
-            ko.set_tuning("layernorm.nontemporal", nt)
-            assert_layernorm_close(ko.layernorm_host(x, g, b), ref)
+        for unbiased in (False, True):
+            assert_layernorm_close(ko.layernorm_host(x, g, b, unbiased=unbiased), oracle.layernorm(x, g, b, unbiased=unbiased))
     finally:
         ko.set_tuning("layernorm.lanes_per_row", 0)
-        ko.set_tuning("layernorm.nontemporal", 0)
 
 
 @pytest.mark.parametrize("policy,rows,cols", [

@@ -68,3 +68,35 @@ def assert_gemm16_close(got_f64, ref_f64, absprod, k, bf16=False):
     worst = (d / bound).max()
     assert worst <= 1.0, "gemm16 err exceeds bound by factor %.3f" % worst
     return d.max(), worst
+
+
+# 16-bit storage (binary16 / bfloat16 in and out, fp32 arithmetic): the fp32 gates above plus one
+# rounding to the storage type - half an ulp, i.e. 2^-11 |ref| (binary16; 2^-25 absolute in its
+# subnormal range) or 2^-8 |ref| (bfloat16).
+def _round16_bound(ref, bf16):
+    return (2.0 ** -8 if bf16 else 2.0 ** -11) * np.abs(ref) + (0.0 if bf16 else 2.0 ** -25)
+
+
+def assert_softmax16_close(got64, ref64, bf16=False):
+    got, ref = np.asarray(got64, np.float64), np.asarray(ref64, np.float64)
+    assert got.shape == ref.shape and np.all(np.isfinite(got))
+    d = np.abs(got - ref)
+    bound = _round16_bound(ref, bf16) + np.minimum(1e-6, 1e-5 * np.abs(ref)) + 1e-45
+    worst = (d / bound).max()
+    assert worst <= 1.0, "softmax16 err exceeds rounding + fp32 gate by factor %.3f" % worst
+    return worst
+
+
+def assert_layernorm16_close(got, ref, bf16=False):
+    (y, mean, rstd), (ry64, rmean, rrstd) = got, ref
+    y, ry = np.asarray(y, np.float64), np.asarray(ry64, np.float64)
+    assert np.all(np.isfinite(y))
+    bound = _round16_bound(ry, bf16) + 1e-5 * np.maximum(np.abs(ry), 1.0)
+    worst = (np.abs(y - ry) / bound).max()
+    assert worst <= 1.0, "layernorm16 y err exceeds rounding + fp32 gate by factor %.3f" % worst
+    mean, rmean = np.asarray(mean, np.float64), np.asarray(rmean, np.float64)
+    rstd, rrstd = np.asarray(rstd, np.float64), np.asarray(rrstd, np.float64)
+    scale = np.maximum(np.abs(rmean), 1.0 / rrstd)
+    assert (np.abs(mean - rmean) / scale).max() <= 1e-5
+    assert (np.abs(rstd - rrstd) / rrstd).max() <= 1e-5
+    return worst
