@@ -76,6 +76,8 @@ def _vendor():
     pp = ctypes.POINTER(vp)
     V.kov_gemm16_sets.argtypes = [i64, i64, i64, pp, pp, ci, pp, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
                                   ctypes.POINTER(ci)]
+    V.kov_gemm16_bias_gelu_sets.argtypes = [i64, i64, i64, pp, pp, vp, ci, pp, ci, ci, ci, ci,
+                                            ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ci)]
     V.kov_sgemm_sets.argtypes = [i64, i64, i64, pp, pp, pp, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
                                  ctypes.POINTER(ci)]
     return V
@@ -214,6 +216,41 @@ def bench_gemm16(cfg, steps, warmup, vendor):
             got = Ds[0].download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
             res["max_abs_diff_vs_hipblaslt"] = float(np.abs(got - ref).max())
     return res, None
+
+
+def bench_gemm16_bias_gelu(steps, warmup, vendor):
+    """The feed-forward up-projection whole: D = gelu(A B + bias) (tanh form) at the shape of configuration 4,
+    next to the vendor library's fused GELU_BIAS epilogue on the same buffers."""
+    c = inputs.CONFIGS[4]
+    m, n, k = c["m"], c["n"], c["k"]
+    flops = inputs.algorithmic_work(4)
+    nsets = 4
+    As = [ko.DeviceBuffer(m * k * 2) for _ in range(nsets)]
+    Bs = [ko.DeviceBuffer(k * n * 2) for _ in range(nsets)]
+    Ds = [ko.DeviceBuffer(m * n * 2) for _ in range(nsets)]
+    bias = ko.DeviceBuffer(n * 2)
+    ko.fill_uniform_16(bias, n, inputs.tensor_seed(4, 2))
+    for a, b in zip(As, Bs):
+        ko.fill_uniform_16(a, m * k, inputs.tensor_seed(4, 0))
+        ko.fill_uniform_16(b, k * n, inputs.tensor_seed(4, 1))
+    wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets], bias=bias,
+                                                act=ko.ACT_GELU_TANH), steps, warmup)
+    res = dict(workload="gemm_f16_bias_gelu_%dx%dx%d" % (m, n, k), metric="tflops", unit="TFLOP/s",
+               value=flops / wall / 1e12, ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
+               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=None),
+               flops=flops, kernel_us=dev * 1e6)
+    if vendor is not None:
+        us, na = ctypes.c_float(), ctypes.c_int()
+        Vs = [ko.DeviceBuffer(m * n * 2) for _ in range(nsets)]
+        if vendor.kov_gemm16_bias_gelu_sets(m, n, k, _ptr_array(As), _ptr_array(Bs), bias.ptr, 1, _ptr_array(Vs), nsets,
+                                            0, 16, 20, ctypes.byref(us), ctypes.byref(na)) == 0:
+            res["hipblaslt_tflops"] = flops / us.value / 1e6
+            res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
+            ref = Vs[0].download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
+            got = Ds[0].download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
+            res["max_abs_diff_vs_hipblaslt"] = float(np.abs(got - ref).max())
+    return res
 
 
 def bench_copy(steps, warmup, nbytes=1 << 30):
@@ -356,6 +393,9 @@ def main():
             del k2
             res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
+        res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         for kind, dt in (("softmax", "f16"), ("layernorm", "bf16")):
             warm = max(args.warmup, SECONDARY_MIN_WARMUP if kind == "layernorm" else 0)
             res = bench_rows16(kind, dt, args.steps, warm)

@@ -50,6 +50,10 @@ typedef enum ko_policy {
 } ko_policy;
 
 typedef enum ko_dtype16 { KO_F16 = 0, KO_BF16 = 1 } ko_dtype16;
+
+/* Epilogue activations of the 16-bit GEMM: GELU(x) = x/2 (1 + erf(x / sqrt 2)), or its tanh form
+ * x/2 (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))). */
+typedef enum ko_activation { KO_ACT_NONE = 0, KO_ACT_GELU_ERF = 1, KO_ACT_GELU_TANH = 2 } ko_activation;
 typedef enum ko_layout { KO_ROW_MAJOR = 0, KO_COL_MAJOR = 1 } ko_layout;
 
 typedef struct ko_device_info_t {
@@ -158,10 +162,21 @@ int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, c
  * the reference's layout, tensor_core_gemm.h:178) or column-major (KO_COL_MAJOR:
  * memory [n][k]); C, D [m,n] row-major.  Elements are binary16 or bfloat16
  * (in_dtype); products accumulate in fp32 on the matrix cores; D is rounded once
- * to the 16-bit type.  C may be NULL.  k must be a multiple of 8. */
+ * to the 16-bit type.  C may be NULL.  k must be a multiple of 8; A, B, C, D 16-byte aligned. */
 int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A, const void *B,
                       int b_layout, float beta, const void *C, void *D, int in_dtype,
                       ko_stream_t stream);
+
+/* Same with the rest of a feed-forward up-projection fused into the epilogue:
+ *      D = activation(alpha * A B + beta * C + bias),   bias: [n] in the 16-bit type or NULL,
+ * evaluated in fp32 and rounded once.  The reference's epilogue is D = acc + C
+ * (simt_gemm.h:325-354; the tensor-core one is unfinished, tensor_core_gemm.h:366-397) and its
+ * functor header carries MultiplyAdd for such fusions (common/functors.h); the 16384 x 3072 x 768
+ * configuration is that projection's shape.  activation: a ko_activation value. */
+int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
+                               const void *B, int b_layout, float beta, const void *C,
+                               const void *bias, int activation, void *D, int in_dtype,
+                               ko_stream_t stream);
 
 /* ---- seeded device fills: replace the host RNG loops of the benchmark drivers
  *      (softmax/main.cu:31-36, layernorm/main.cu:30-35, gemm/main.cu:46-66) with a

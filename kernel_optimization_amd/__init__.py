@@ -21,6 +21,7 @@ KO_ERR_NO_DEVICE = 5
 
 POLICY_AUTO, POLICY_WARP, POLICY_BLOCK, POLICY_BLOCK_NOCACHE = 0, 1, 2, 3
 F16, BF16 = 0, 1
+ACT_NONE, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
 ROW_MAJOR, COL_MAJOR = 0, 1
 
 _vp = ctypes.c_void_p
@@ -69,6 +70,7 @@ SIGNATURES = {
     "ko_layernorm_16": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _int, _int, _vp]),
     "ko_sgemm_f32": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _f, _vp, _vp, _vp]),
     "ko_gemm_f16f32acc": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp]),
+    "ko_gemm_f16f32acc_bias_act": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp, _int, _vp]),
     "ko_fill_normal_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
     "ko_fill_uniform_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
     "ko_fill_uniform_16": (_int, [_vp, _i64, _u64, _d, _d, _i64, _int, _vp]),
@@ -275,9 +277,13 @@ def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
 
 
 def gemm16(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, b_layout=COL_MAJOR, dtype=F16,
-           stream=None):
-    check(lib().ko_gemm_f16f32acc(m, n, k, alpha, _p(A), _p(B), b_layout, beta, _p(C), _p(D),
-                                  dtype, _h(stream)))
+           stream=None, bias=None, act=ACT_NONE):
+    if bias is None and act == ACT_NONE:
+        check(lib().ko_gemm_f16f32acc(m, n, k, alpha, _p(A), _p(B), b_layout, beta, _p(C), _p(D),
+                                      dtype, _h(stream)))
+    else:
+        check(lib().ko_gemm_f16f32acc_bias_act(m, n, k, alpha, _p(A), _p(B), b_layout, beta, _p(C), _p(bias), act,
+                                               _p(D), dtype, _h(stream)))
 
 
 def fill_normal_f32(out, n, seed, mean=0.0, std=1.0, first=0, stream=None):
@@ -373,14 +379,15 @@ def sgemm_host(A, B, C=None, alpha=1.0, beta=0.0):
 
 
 def gemm16_host(A_bits, B_bits, m, n, k, C_bits=None, alpha=1.0, beta=0.0, b_layout=COL_MAJOR,
-                dtype=F16):
+                dtype=F16, bias_bits=None, act=ACT_NONE):
     """Operands as uint16 bit patterns (binary16 or bfloat16); returns uint16 [m, n]."""
     A_bits = np.ascontiguousarray(A_bits).view(np.uint16)
     B_bits = np.ascontiguousarray(B_bits).view(np.uint16)
     assert A_bits.size == m * k and B_bits.size == n * k
     dA, dB = DeviceBuffer.from_numpy(A_bits), DeviceBuffer.from_numpy(B_bits)
     dC = None if C_bits is None else DeviceBuffer.from_numpy(np.ascontiguousarray(C_bits).view(np.uint16))
+    dbias = None if bias_bits is None else DeviceBuffer.from_numpy(np.ascontiguousarray(bias_bits).view(np.uint16))
     dD = DeviceBuffer(max(m * n * 2, 8))
-    gemm16(m, n, k, dA, dB, dD, dC, alpha, beta, b_layout, dtype)
+    gemm16(m, n, k, dA, dB, dD, dC, alpha, beta, b_layout, dtype, bias=dbias, act=act)
     synchronize()
     return dD.download(np.uint16, (m, n))

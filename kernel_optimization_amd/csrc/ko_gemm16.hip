@@ -105,7 +105,45 @@ struct Params {
     int nblocks;
     int band_rows;              // persistent kernels: > 0 selects the blocked tile order (see tile_of)
     int block_cols;
+    const uint16_t *bias;       // [N] or null: added to every row before the activation
+    int act;                    // KO_ACT_*
 };
+
+// x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
+// x * rcp(1 + 2^(x (c1 + c2 x^2))), c1 = -2 sqrt(2/pi) log2(e), c2 = 0.044715 c1: two multiplies, one FMA,
+// one add and the hardware 2^x and reciprocal (about 1 ulp each; the result is rounded to 16 bits next).
+// Large negative x: 2^(+big) = inf, rcp = 0, result -0; large positive x: 2^(-big) = 0, result x.
+__device__ __forceinline__ float gelu_tanh(float x) {
+    constexpr float c1 = -2.0f * 0.79788456080286535588f * 1.44269504088896340736f;
+    constexpr float c2 = 0.044715f * c1;
+    const float t = x * __builtin_fmaf(c2 * x, x, c1);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
+}
+
+// Epilogue of one group of four consecutive columns n .. n+3 of row m (all inside the matrix):
+// v = act(alpha * acc + beta * C + bias).  C and bias are read as 8-byte groups.
+template <bool BF16>
+__device__ __forceinline__ void finish4(const Params &p, float (&v)[4], int64_t off, int n, bool use_c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= p.alpha;
+    if (use_c) {
+        const u32x2 c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += p.beta * to_float<BF16>(static_cast<uint16_t>(c2[e >> 1] >> ((e & 1) * 16)));
+    }
+    if (p.bias) {
+        const u32x2 b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += to_float<BF16>(static_cast<uint16_t>(b2[e >> 1] >> ((e & 1) * 16)));
+    }
+    if (p.act == KO_ACT_GELU_ERF) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = 0.5f * v[e] * (1.0f + erff(v[e] * 0.70710678118654752440f));
+    } else if (p.act == KO_ACT_GELU_TANH) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+    }
+}
 
 // Persistent kernels: tile number t (0, 1, ...) of workgroup b when the grid has `grid` workgroups.
 // Workgroup b runs on XCD b % 8 and is the (b / 8)-th of the workgroups there.  With band_rows > 0
@@ -138,11 +176,12 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
     constexpr int TM = WTM / 32, TN = WTN / 32;
     const int M = p.M, N = p.N;
     const int frow = lane & 31, fhalf = lane >> 5;
-    const float alpha = p.alpha, beta = p.beta;
-    const bool use_c = p.C != nullptr && beta != 0.0f;
+    const float alpha = p.alpha;
+    const bool use_c = p.C != nullptr && p.beta != 0.0f;
+    const bool plain = !use_c && p.bias == nullptr && p.act == KO_ACT_NONE;  // D = alpha * acc
 
-    if (!EDGE && !use_c) {
-        // Full tiles, no C: each wave transposes its own tile through LDS (free now: the last
+    if (!EDGE) {
+        // Full tiles: each wave transposes its own tile through LDS (free now: the last
         // barrier of the K loop is behind every wave) and writes whole 16-byte chunks, a
         // contiguous WTN*2-byte run per row.  8-byte units of a row are XOR-swizzled with the
         // row index: the accumulator writes (32 consecutive rows, one unit) and the row reads
@@ -171,11 +210,18 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int unit = j * 8 + 2 * q + fhalf;
+                        float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                        if (plain) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] *= alpha;
+                        } else {  // C, bias and the activation enter before the one rounding to 16 bits
+                            const int gm = row0 + i * 32 + frow;
+                            const int gn = col0 + j * 32 + 8 * q + 4 * fhalf;
+                            finish4<BF16>(p, v, static_cast<int64_t>(gm) * N + gn, gn, use_c);
+                        }
                         u32x2 o;
-                        o[0] = from_float<BF16>(alpha * acc[i][j][4 * q]) |
-                               (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 1])) << 16);
-                        o[1] = from_float<BF16>(alpha * acc[i][j][4 * q + 2]) |
-                               (static_cast<uint32_t>(from_float<BF16>(alpha * acc[i][j][4 * q + 3])) << 16);
+                        o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
+                        o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
                         region8[row * (2 * ROW_CHUNKS) + (unit ^ (erow(row) & SWZ))] = o;
                     }
                 }
@@ -206,16 +252,9 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int n = col0 + j * 32 + 8 * q + 4 * fhalf;
                 if (EDGE && n >= N) continue;
                 const int64_t off = static_cast<int64_t>(m) * N + n;
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][4 * q + e];
+                float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                 if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
-                    if (use_c) {
-                        const u32x2 c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            v[e] += beta * to_float<BF16>(static_cast<uint16_t>(c2[e >> 1] >> ((e & 1) * 16)));
-                    }
+                    finish4<BF16>(p, v, off, n, use_c);
                     u32x2 o;
                     o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
                     o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
@@ -224,8 +263,11 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         if (n + e < N) {
-                            float t = v[e];
-                            if (use_c) t += beta * to_float<BF16>(p.C[off + e]);
+                            float t = alpha * v[e];
+                            if (use_c) t += p.beta * to_float<BF16>(p.C[off + e]);
+                            if (p.bias) t += to_float<BF16>(p.bias[n + e]);
+                            if (p.act == KO_ACT_GELU_ERF) t = 0.5f * t * (1.0f + erff(t * 0.70710678118654752440f));
+                            else if (p.act == KO_ACT_GELU_TANH) t = gelu_tanh(t);
                             p.D[off + e] = from_float<BF16>(t);
                         }
                     }
@@ -983,30 +1025,40 @@ int launch_variant(const Params &p, hipStream_t stream) {
 }  // namespace
 }  // namespace ko
 
-KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
-                                const void *B, int b_layout, float beta, const void *C, void *D,
-                                int in_dtype, ko_stream_t stream) {
+KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
+                                         const void *B, int b_layout, float beta, const void *C, const void *bias,
+                                         int activation, void *D, int in_dtype, ko_stream_t stream) {
     using namespace ko;
     if (m < 0 || n < 0 || k < 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
     if (in_dtype != KO_F16 && in_dtype != KO_BF16) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: in_dtype=%d", in_dtype);
     if (b_layout != KO_ROW_MAJOR && b_layout != KO_COL_MAJOR)
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: b_layout=%d", b_layout);
+    if (activation != KO_ACT_NONE && activation != KO_ACT_GELU_ERF && activation != KO_ACT_GELU_TANH)
+        return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: activation=%d", activation);
     if (m == 0 || n == 0) return KO_OK;
     if (k == 0 || k % 8 != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: k=%lld must be a positive multiple of 8", (long long)k);
     if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: dimension too large");
     if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: null A/B/D pointer");
-    uintptr_t align = reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B);
-    if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: A and B must be 16-byte aligned");
-    if ((reinterpret_cast<uintptr_t>(D) | reinterpret_cast<uintptr_t>(C)) & 7)
-        return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: C and D must be 8-byte aligned");
+    uintptr_t align = reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
+                      reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D);
+    if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: A, B, C and D must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(bias) & 7) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: bias must be 8-byte aligned");
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
-             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0};
+             static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0,
+             static_cast<const uint16_t *>(bias), activation};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);
     return b_layout == KO_COL_MAJOR ? launch_variant<true, false>(p, s) : launch_variant<true, true>(p, s);
+}
+
+KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
+                                const void *B, int b_layout, float beta, const void *C, void *D,
+                                int in_dtype, ko_stream_t stream) {
+    return ko_gemm_f16f32acc_bias_act(m, n, k, alpha, A, B, b_layout, beta, C, nullptr, KO_ACT_NONE, D, in_dtype,
+                                      stream);
 }

@@ -51,6 +51,9 @@ def lib():
                                        ctypes.c_double, _f32p, _f32p, _f64p]
         L.oracle_gemm_16.argtypes = [_i64, _i64, _i64, ctypes.c_double, _u16p, _u16p, ctypes.c_int,
                                      ctypes.c_double, _u16p, _u16p, ctypes.c_int, _f64p, _f64p]
+        L.oracle_gemm_16_bias_act.argtypes = [_i64, _i64, _i64, ctypes.c_double, _u16p, _u16p, ctypes.c_int,
+                                              ctypes.c_double, _u16p, _u16p, ctypes.c_int, _u16p, ctypes.c_int,
+                                              _f64p, _f64p]
         L.oracle_softmax_16.argtypes = [_u16p, _u16p, _f64p, _i64, _i64, _i32p, _i64, ctypes.c_int]
         L.oracle_layernorm_16.argtypes = [_u16p, _u16p, _f64p, _f32p, _f32p, _u16p, _u16p, _i64, _i64,
                                           ctypes.c_double, ctypes.c_int, ctypes.c_int]
@@ -170,8 +173,11 @@ def sgemm(A, B, C=None, alpha=1.0, beta=0.0, want_absprod=False):
     return (D, ap) if want_absprod else D
 
 
+ACT_NONE, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
+
+
 def gemm16(A_bits, B_bits, m, n, k, b_col_major=True, C_bits=None, alpha=1.0, beta=0.0,
-           bf16=False):
+           bf16=False, bias_bits=None, act=ACT_NONE):
     """16-bit-input GEMM.  A_bits [m,k], B_bits [n,k] (col-major B) or [k,n]; uint16 bit patterns.
 
     Returns (D_bits uint16 [m,n], d64 float64 [m,n], absprod float64 [m,n])."""
@@ -180,11 +186,14 @@ def gemm16(A_bits, B_bits, m, n, k, b_col_major=True, C_bits=None, alpha=1.0, be
     D = np.empty((m, n), np.uint16)
     d64 = np.empty((m, n), np.float64)
     ap = np.empty((m, n), np.float64)
-    rc = lib().oracle_gemm_16(m, n, k, float(alpha), _ptr(A_bits, _u16p), _ptr(B_bits, _u16p),
-                              int(bool(b_col_major)), float(beta), _ptr(C_bits, _u16p),
-                              _ptr(D, _u16p), int(bool(bf16)), _ptr(d64, _f64p), _ptr(ap, _f64p))
+    bias_bits = _c(bias_bits, np.uint16)
+    assert bias_bits is None or bias_bits.size == n
+    rc = lib().oracle_gemm_16_bias_act(m, n, k, float(alpha), _ptr(A_bits, _u16p), _ptr(B_bits, _u16p),
+                                       int(bool(b_col_major)), float(beta), _ptr(C_bits, _u16p),
+                                       _ptr(bias_bits, _u16p), int(act), _ptr(D, _u16p), int(bool(bf16)),
+                                       _ptr(d64, _f64p), _ptr(ap, _f64p))
     if rc:
-        raise ValueError("oracle_gemm_16: bad arguments")
+        raise ValueError("oracle_gemm_16_bias_act: bad arguments")
     return D, d64, ap
 
 

@@ -439,10 +439,21 @@ ORACLE_API int oracle_sgemm_f32(int64_t m, int64_t n, int64_t k, double alpha, c
  * rounding; one final rounding to the 16-bit type.  d64 (may be NULL)
  * receives the unrounded double result, absprod as above.
  */
-ORACLE_API int oracle_gemm_16(int64_t m, int64_t n, int64_t k, double alpha, const uint16_t *A,
-                              const uint16_t *B, int b_col_major, double beta, const uint16_t *C,
-                              uint16_t *D, int is_bf16, double *d64, double *absprod) {
-    if (m < 0 || n < 0 || k < 0) return 1;
+/* Epilogue activations: 0 none; 1 GELU(x) = x/2 (1 + erf(x / sqrt 2)); 2 its tanh form
+ * x/2 (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))). */
+static double apply_activation(double x, int act) {
+    if (act == 1) return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440));
+    if (act == 2) return 0.5 * x * (1.0 + tanh(0.79788456080286535588 * (x + 0.044715 * x * x * x)));
+    return x;
+}
+
+/* D = act(alpha A B + beta C + bias[n]): the epilogue of the feed-forward up-projection that the
+ * 16384 x 3072 x 768 configuration stands for.  bias (may be NULL) is a 16-bit vector of length n. */
+ORACLE_API int oracle_gemm_16_bias_act(int64_t m, int64_t n, int64_t k, double alpha, const uint16_t *A,
+                                       const uint16_t *B, int b_col_major, double beta, const uint16_t *C,
+                                       const uint16_t *bias, int act, uint16_t *D, int is_bf16, double *d64,
+                                       double *absprod) {
+    if (m < 0 || n < 0 || k < 0 || act < 0 || act > 2) return 1;
     /* widen B once into [N][K] doubles so the inner loop is contiguous */
     double *Bt = (double *)__builtin_malloc(sizeof(double) * (size_t)(n * k > 0 ? n * k : 1));
     if (!Bt) return 2;
@@ -471,6 +482,8 @@ ORACLE_API int oracle_gemm_16(int64_t m, int64_t n, int64_t k, double alpha, con
                 uint16_t cb = C[i * n + j];
                 v += beta * (is_bf16 ? bf16_bits_to_double(cb) : f16_bits_to_double(cb));
             }
+            if (bias) v += is_bf16 ? bf16_bits_to_double(bias[j]) : f16_bits_to_double(bias[j]);
+            v = apply_activation(v, act);
             if (D) D[i * n + j] = is_bf16 ? double_to_bf16_bits(v) : double_to_f16_bits(v);
             if (d64) d64[i * n + j] = v;
             if (absprod) absprod[i * n + j] = aacc;
@@ -480,4 +493,10 @@ ORACLE_API int oracle_gemm_16(int64_t m, int64_t n, int64_t k, double alpha, con
     }
     __builtin_free(Bt);
     return 0;
+}
+
+ORACLE_API int oracle_gemm_16(int64_t m, int64_t n, int64_t k, double alpha, const uint16_t *A,
+                              const uint16_t *B, int b_col_major, double beta, const uint16_t *C,
+                              uint16_t *D, int is_bf16, double *d64, double *absprod) {
+    return oracle_gemm_16_bias_act(m, n, k, alpha, A, B, b_col_major, beta, C, NULL, 0, D, is_bf16, d64, absprod);
 }

@@ -237,3 +237,65 @@ def test_gemm16_errors(ko):
     with pytest.raises(ko.KoError) as e:
         ko.gemm16(16, 16, 16, buf, None, buf)
     assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+
+
+# ------------------------------------------------------------------------------------ fused epilogue
+
+def assert_gemm16_act_close(got_f64, ref_f64, absprod, k, bf16=False):
+    """act(alpha A B + beta C + bias): the activations used here have slope <= 1.13, and their fp32
+    evaluation (erff / exp) adds a few units in the last place of the result."""
+    got, ref = np.asarray(got_f64, np.float64), np.asarray(ref_f64, np.float64)
+    assert np.all(np.isfinite(got))
+    ulp = 2.0 ** -8 if bf16 else 2.0 ** -11
+    bound = ulp * np.abs(ref) + 1.13 * (k * 2.0 ** -24 * absprod + 2.0 ** -22) + 4 * 2.0 ** -24 * np.abs(ref) + 2.0 ** -24
+    worst = (np.abs(got - ref) / bound).max()
+    assert worst <= 1.0, "gemm16 epilogue err exceeds bound by factor %.3f" % worst
+
+
+@pytest.mark.parametrize("act", [0, 1, 2])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (70, 45, 40)])
+def test_gemm16_bias_activation(ko, act, bf16, b_col_major, m, n, k):
+    A = _bits16((m, k), 41 + m, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 43 + n, bf16)
+    C = _bits16((m, n), 45, bf16)
+    bias = _bits16((n,), 47, bf16)
+    for c_bits, beta, use_bias in ((None, 0.0, True), (C, 0.5, True), (C, 1.0, False)):
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16, C_bits=c_bits, beta=beta,
+                                     bias_bits=bias if use_bias else None, act=act)
+        ap = ap + 2.0  # |beta C| + |bias| <= 2: their roundings enter like one more product each
+        got = ko.gemm16_host(A, B, m, n, k, C_bits=c_bits, beta=beta, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR,
+                             dtype=ko.BF16 if bf16 else ko.F16, bias_bits=bias if use_bias else None, act=act)
+        assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+
+
+@pytest.mark.parametrize("variant", [0, 9, 30, 50])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm16_bias_gelu_big(ko, variant, bf16):
+    """The up-projection shape in small (512 tiles of 256 x 256, K = 384): bias + GELU and beta * C through the
+    coalesced epilogue of every kernel family; sampled rows against the oracle."""
+    m, n, k = 8192, 4096, 384
+    A = _bits16((m, k), 51, bf16)
+    B = _bits16((n, k), 52, bf16)
+    bias = _bits16((n,), 53, bf16)
+    C = _bits16((m, n), 54, bf16)
+    idx = np.sort(np.random.default_rng(6).choice(m, 48, replace=False))
+    ko.set_tuning("gemm16.variant", variant)
+    try:
+        for act, c_bits, beta in ((1, None, 0.0), (2, C, -0.5), (0, C, 1.0)):
+            got = ko.gemm16_host(A, B, m, n, k, C_bits=c_bits, beta=beta, dtype=ko.BF16 if bf16 else ko.F16,
+                                 bias_bits=bias, act=act)
+            _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, bf16=bf16, C_bits=None if c_bits is None else c_bits[idx],
+                                         beta=beta, bias_bits=bias, act=act)
+            assert_gemm16_act_close(_to_f64(got[idx], bf16), ref64, ap + 2.0, k, bf16=bf16)
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+
+
+def test_gemm16_bias_act_errors(ko):
+    d = ko.DeviceBuffer(1 << 16)
+    L = ko.lib()
+    assert L.ko_gemm_f16f32acc_bias_act(16, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, None, 7, d.ptr, ko.F16, None) == ko.KO_ERR_INVALID_ARGUMENT
+    assert L.ko_gemm_f16f32acc_bias_act(16, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, d.ptr + 2, 1, d.ptr, ko.F16, None) == ko.KO_ERR_INVALID_ARGUMENT
+    assert L.ko_gemm_f16f32acc_bias_act(0, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, None, 1, d.ptr, ko.F16, None) == ko.KO_OK
