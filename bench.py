@@ -267,6 +267,39 @@ def bench_copy(steps, warmup, nbytes=1 << 30):
                 algorithmic_bytes=2 * n * 4, kernel_us=dev * 1e6)
 
 
+def bench_long_rows(op, rows, cols, policy, steps, warmup):
+    """Row lengths past what one wavefront holds: the row-per-workgroup (BLOCK) and re-read (BLOCK_NOCACHE) policies,
+    and the reference's commented-out [49152, 1024] run (nn_operators/softmax/main.cu:78-79)."""
+    n = rows * cols
+    if op == "softmax":
+        work = 2 * n * 4
+    else:
+        work = 2 * n * 4 + 2 * cols * 4 + 2 * rows * 4
+    nsets = max(1, -(-(1 << 30) // work))
+    xs = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    ys = [ko.DeviceBuffer(n * 4) for _ in range(nsets)]
+    for x in xs:
+        ko.fill_normal_f32(x, n, 11, 0.0, 4.0)
+    floor_us = _copy_floor_us(xs, ys, n, steps, warmup)
+    if op == "softmax":
+        launch = lambda i: ko.softmax(xs[i % nsets], ys[i % nsets], rows, cols, None, 0, policy)
+    else:
+        g, b = ko.DeviceBuffer(cols * 4), ko.DeviceBuffer(cols * 4)
+        ko.fill_normal_f32(g, cols, 12, 1.0, 0.1)
+        ko.fill_normal_f32(b, cols, 13, 0.0, 0.1)
+        m, r = ko.DeviceBuffer(rows * 4), ko.DeviceBuffer(rows * 4)
+        launch = lambda i: ko.layernorm(xs[i % nsets], ys[i % nsets], rows, cols, m, r, g, b, 1e-5, False, policy)
+    wall, dev = _time_steps(launch, steps, warmup)
+    names = {ko.POLICY_AUTO: "auto", ko.POLICY_WARP: "warp", ko.POLICY_BLOCK: "block", ko.POLICY_BLOCK_NOCACHE: "nocache"}
+    res = dict(workload="%s_f32_%dx%d_%s" % (op, rows, cols, names[policy]), metric="hbm_gbytes_per_s", unit="GB/s",
+               value=work / wall / 1e9, ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
+               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
+               algorithmic_bytes=work, kernel_us=dev * 1e6)
+    _add_copy_floor(res, floor_us)
+    return res
+
+
 def bench_rows16(kind, dtype_name, steps, warmup):
     """The two row operators on 16-bit storage at the shapes of the masked-softmax and LayerNorm configurations
     (half the bytes per element; fp32 arithmetic).  Inputs: uniform fills of the storage type."""
@@ -392,6 +425,13 @@ def main():
             res, k2 = run_workload(other, args.steps, warm, vendor)
             del k2
             res["steps"], res["warmup"] = args.steps, warm
+            others.append(res)
+        for op, rows, cols, policy in (("softmax", 49152, 1024, ko.POLICY_WARP), ("softmax", 8192, 16384, ko.POLICY_BLOCK),
+                                       ("softmax", 1024, 131072, ko.POLICY_BLOCK_NOCACHE),
+                                       ("layernorm", 8192, 16384, ko.POLICY_BLOCK),
+                                       ("layernorm", 1024, 131072, ko.POLICY_BLOCK_NOCACHE)):
+            res = bench_long_rows(op, rows, cols, policy, args.steps, args.warmup)
+            res["steps"], res["warmup"] = args.steps, args.warmup
             others.append(res)
         res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)

@@ -193,10 +193,11 @@ __device__ __forceinline__ wave::Welford block_welford_allreduce(wave::Welford w
         lds[32 + wv] = w.m2;
     }
     __syncthreads();
-    wave::Welford r{lds[0], lds[16], lds[32]};
-#pragma unroll
-    for (int i = 1; i < WAVES; ++i) r = wave::welford_merge(r, wave::Welford{lds[i], lds[16 + i], lds[32 + i]});
-    return r;
+    // every lane picks up one wave's triplet and the WAVES of them are merged as a tree by the same
+    // symmetric exchanges (log2(WAVES) merges instead of WAVES - 1 in a row); all lanes of all waves
+    // end with the same bits
+    const int i = threadIdx.x & (WAVES - 1);
+    return wave::welford_allreduce<WAVES>(wave::Welford{lds[i], lds[16 + i], lds[32 + i]});
 }
 
 // y = (x - mean) * rstd [* gamma] [+ beta] for one vector; gamma/beta are read here (long rows:
@@ -231,6 +232,23 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
     __shared__ float lds[48];
     constexpr Reciprocals<VPL * E> rcp;
     const int nvec = cols / E;
+    // gamma/beta of this thread's columns stay in registers across the rows the workgroup walks, when
+    // row, gamma and beta fit the register budget of the workgroup size (128 per lane at 1024 threads)
+    constexpr bool HOIST = VPL * E * 3 + 48 <= (THREADS == 1024 ? 128 : 256);
+    float g[HOIST ? VPL : 1][E], b[HOIST ? VPL : 1][E];
+#pragma unroll
+    for (int k = 0; k < (HOIST ? VPL : 0); ++k) {
+        const int j = threadIdx.x + k * THREADS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            g[k][e] = 1.0f;
+            b[k][e] = 0.0f;
+        }
+        if (j < nvec) {
+            if (gamma) Io<IO>::template load<false>(gamma + E * j, g[k]);
+            if (beta) Io<IO>::template load<false>(beta + E * j, b[k]);
+        }
+    }
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const typename Io<IO>::elem *src = in + row * cols;
         float v[VPL][E];
@@ -265,7 +283,12 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
             const int j = threadIdx.x + k * THREADS;
             if (j < nvec) {
                 float y[E];
-                normalize_vec<IO>(v[k], mean, rstd, gamma, beta, E * j, y);
+                if constexpr (HOIST) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[k][e], b[k][e]);
+                } else {
+                    normalize_vec<IO>(v[k], mean, rstd, gamma, beta, E * j, y);
+                }
                 Io<IO>::template store<false>(dst + E * j, y);
             }
         }
@@ -293,30 +316,49 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
         const typename Io<IO>::elem *src = in + row * cols;
         const float x0 = Io<IO>::scalar(src);
         wave::Welford w{0.0f, 0.0f, 0.0f};
-        for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float x[E];
-            Io<IO>::template load<false>(src + E * j, x);
+        // UNROLL vectors per thread and trip: their loads are issued together, so that a workgroup keeps
+        // enough bytes in flight to cover the memory latency (one vector per trip leaves the pipe half empty)
+        constexpr int UNROLL = 4;
+        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+            float x[UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) {
-                // streaming update with a true division: the count is not a compile-time constant here
-                const float xe = x[e] - x0;
-                w.count += 1.0f;
-                const float d = xe - w.mean;
-                w.mean += d / w.count;
-                w.m2 = __builtin_fmaf(d, xe - w.mean, w.m2);
+            for (int u = 0; u < UNROLL; ++u)
+                if (j0 + u * THREADS < nvec) Io<IO>::template load<false>(src + E * (j0 + u * THREADS), x[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (j0 + u * THREADS >= nvec) break;
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    // streaming update; the count is not a compile-time constant here, and 1/count comes from
+                    // the hardware reciprocal (1 ulp): M2 is accumulated against the mean actually formed, so
+                    // the triplet stays consistent and the deviation is far inside the 1e-5 gate
+                    const float xe = x[u][e] - x0;
+                    w.count += 1.0f;
+                    const float d = xe - w.mean;
+                    w.mean = __builtin_fmaf(d, __builtin_amdgcn_rcpf(w.count), w.mean);
+                    w.m2 = __builtin_fmaf(d, xe - w.mean, w.m2);
+                }
             }
         }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
         typename Io<IO>::elem *dst = out + row * cols;
-        for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float x[E], y[E];
-            Io<IO>::template load<false>(src + E * j, x);
+        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+            float x[UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) x[e] -= x0;
-            normalize_vec<IO>(x, mean, rstd, gamma, beta, E * j, y);
-            Io<IO>::template store<false>(dst + E * j, y);
+            for (int u = 0; u < UNROLL; ++u)
+                if (j0 + u * THREADS < nvec) Io<IO>::template load<false>(src + E * (j0 + u * THREADS), x[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int j = j0 + u * THREADS;
+                if (j >= nvec) break;
+                float y[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e) x[u][e] -= x0;
+                normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
+                Io<IO>::template store<false>(dst + E * j, y);
+            }
         }
         if (threadIdx.x == 0) {
             if (mean_out) mean_out[row] = x0 + mean;
@@ -380,10 +422,13 @@ int launch_wave_lpr(const Args<IO> &a, int lpr) {
     }
 }
 
+// Longest row per policy, in 16-byte vectors: 512 per wavefront (2048 fp32 or 4096 16-bit columns); per
+// workgroup 8192 vectors of fp32 (32768 columns) or 4096 vectors of 16-bit values (32768 columns: eight
+// vectors of eight values per thread do not fit the 128 registers of a 1024-thread workgroup).
 constexpr int kWaveMaxVpl = 8;
-// Longest row per policy, in 16-byte vectors (fp32: 2048 and 32768 columns; 16-bit: twice that).
 constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
-constexpr int kBlockMaxVecs = 1024 * 8;
+template <int IO>
+constexpr int kBlockMaxVecs = 1024 * (Io<IO>::E == 8 ? 4 : 8);
 
 // Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
 // {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
@@ -427,8 +472,8 @@ int launch_block_threads(const Args<IO> &a) {
                                                                   a.inv_denominator)
     if (vpl <= 1) KO_LN_BLOCK(1);
     else if (vpl <= 2) KO_LN_BLOCK(2);
-    else if (vpl <= 4) KO_LN_BLOCK(4);
-    else KO_LN_BLOCK(8);
+    else if (vpl <= 4 || Io<IO>::E == 8) KO_LN_BLOCK(4);
+    else KO_LN_BLOCK((Io<IO>::E == 8 ? 4 : 8));
 #undef KO_LN_BLOCK
     KO_CHECK_LAUNCH();
     return KO_OK;
@@ -483,7 +528,7 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
-                 : nvec <= kBlockMaxVecs ? KO_POLICY_BLOCK
+                 : nvec <= kBlockMaxVecs<IO> ? KO_POLICY_BLOCK
                                          : KO_POLICY_BLOCK_NOCACHE;
     }
     switch (policy) {
@@ -493,9 +538,9 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
                             "layernorm: WARP policy holds at most %d columns per row, got %d", kWaveMaxVecs * E, a.cols);
             return launch_wave_any<IO>(a);
         case KO_POLICY_BLOCK:
-            if (nvec > kBlockMaxVecs)
+            if (nvec > kBlockMaxVecs<IO>)
                 return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "layernorm: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs * E, a.cols);
+                            "layernorm: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs<IO> * E, a.cols);
             return launch_block<IO>(a);
         case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO>(a);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);

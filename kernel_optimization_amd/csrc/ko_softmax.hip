@@ -237,23 +237,39 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
         float m = -FLT_MAX, s = 0.0f;
-        for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float x[E];
-            load_row_vec<IO, MASKED, false>(src, j, vlen, x);
+        // UNROLL vectors per thread and trip: their loads are issued together, so that a workgroup keeps
+        // enough bytes in flight to cover the memory latency
+        constexpr int UNROLL = 4;
+        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+            float x[UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) online_add(m, s, x[e]);
+            for (int u = 0; u < UNROLL; ++u)
+                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, false>(src, j0 + u * THREADS, vlen, x[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (j0 + u * THREADS >= nvec) break;
+#pragma unroll
+                for (int e = 0; e < E; ++e) online_add(m, s, x[u][e]);
+            }
         }
         const float gm = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
         s *= exp_nonpositive(m - gm);  // threads that saw nothing: s = 0
         const float gs = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
         const float inv = 1.0f / gs;
         typename Io<IO>::elem *dst = out + row * cols;
-        for (int j = threadIdx.x; j < nvec; j += THREADS) {
-            float x[E];
-            load_row_vec<IO, MASKED, false>(src, j, vlen, x);
+        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+            float x[UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) x[e] = exp_for_storage<IO>(x[e] - gm) * inv;
-            Io<IO>::template store<false>(dst + E * j, x);
+            for (int u = 0; u < UNROLL; ++u)
+                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, false>(src, j0 + u * THREADS, vlen, x[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int j = j0 + u * THREADS;
+                if (j >= nvec) break;
+#pragma unroll
+                for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
+                Io<IO>::template store<false>(dst + E * j, x[u]);
+            }
         }
     }
 }

@@ -100,8 +100,8 @@ def test_layernorm16_matches_oracle(ko, rows, cols, unbiased, bf16):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("policy,rows,cols", [(2, 37, 128), (2, 19, 1024), (2, 5, 16384), (2, 3, 65536),
-                                              (3, 37, 128), (3, 4, 40000), (0, 3, 8192), (0, 2, 131072)])
+@pytest.mark.parametrize("policy,rows,cols", [(2, 37, 128), (2, 19, 1024), (2, 5, 16384), (2, 3, 32768),
+                                              (3, 37, 128), (3, 4, 40000), (0, 3, 8192), (0, 2, 65536), (0, 2, 131072)])
 def test_layernorm16_block_policies(ko, policy, rows, cols, bf16):
     xb = _bits(inputs.normal_f32((rows, cols), 110 + cols, 0.5, 2.0), bf16)
     gb = _bits(inputs.normal_f32((cols,), 111, 1.0, 0.1), bf16)
@@ -122,6 +122,8 @@ def test_layernorm16_plain_in_place_and_errors(ko, bf16):
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 12, 1e-5, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 16, 1e-5, 0, 9, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 0, 16, 1e-5, 0, dt, 0, None) == ko.KO_OK
+    # the row-per-workgroup policy holds 32768 16-bit columns
+    assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 1, 65536, 1e-5, 0, dt, 2, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
 
 
 @pytest.mark.parametrize("bf16", [False, True])
