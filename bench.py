@@ -450,7 +450,7 @@ def main():
         "config": {"workload": head["workload"], "buffer_sets": head["buffer_sets"],
                    "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
         "roofline": head["roofline"], "cpu_baseline": cpu, "parity": parity,
-        "kernel_us": head["kernel_us"],
+        "kernel_us": head["kernel_us"], "copy_same_bytes_us": head.get("copy_same_bytes_us"),
         "copy_ceiling": None if copy is None else {"GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"],
                                                    "workload": copy["workload"]},
         "workloads": others,
