@@ -73,6 +73,20 @@ __device__ __forceinline__ uint16_t from_float(float v) {
     }
 }
 
+// Two floats -> two 16-bit values in one register (low half first), each rounded to nearest even by the
+// hardware conversions (v_cvt_pk_bf16_f32 / v_cvt_f16_f32).
+template <bool BF16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef float float2v __attribute__((ext_vector_type(2)));
+    if constexpr (BF16) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{lo, hi}, bf16x2));
+    } else {
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{lo, hi}, half2v));
+    }
+}
+
 // Workgroup -> output tile.  Workgroups are handed to the 8 XCDs round-robin by
 // their index, and each XCD has its own L2; the remap gives every XCD one
 // contiguous band of tiles (tile_n fastest), so the tiles resident on an XCD at any
@@ -220,8 +234,8 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                             finish4<BF16>(p, v, static_cast<int64_t>(gm) * N + gn, gn, use_c);
                         }
                         u32x2 o;
-                        o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
-                        o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
+                        o[0] = pack2<BF16>(v[0], v[1]);
+                        o[1] = pack2<BF16>(v[2], v[3]);
                         region8[row * (2 * ROW_CHUNKS) + (unit ^ (erow(row) & SWZ))] = o;
                     }
                 }
@@ -256,8 +270,8 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
                     finish4<BF16>(p, v, off, n, use_c);
                     u32x2 o;
-                    o[0] = from_float<BF16>(v[0]) | (static_cast<uint32_t>(from_float<BF16>(v[1])) << 16);
-                    o[1] = from_float<BF16>(v[2]) | (static_cast<uint32_t>(from_float<BF16>(v[3])) << 16);
+                    o[0] = pack2<BF16>(v[0], v[1]);
+                    o[1] = pack2<BF16>(v[2], v[3]);
                     *reinterpret_cast<u32x2 *>(p.D + off) = o;
                 } else {
 #pragma unroll
@@ -739,29 +753,39 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         n0 = tile_n * BN;
     };
 
-    // The loads walk the K tiles of this workgroup's output tiles in order; the cursor holds the
-    // next one to fetch, so no division is needed per step.
-    int ld_kt = 0, ld_t = 0, ld_m0, ld_n0;
-    tile_origin(0, ld_m0, ld_n0);
+    // The loads walk the K tiles of this workgroup's output tiles in order.  The cursor is a pair of
+    // wave-uniform pointers (row 8 * wave of the A and of the B panel, at the K tile to fetch next), moved
+    // on by 128 bytes per K tile and recomputed when an output tile is finished, so that a load costs a
+    // scalar 64-bit add, the lane offset and the LDS address in M0 - no multiplication per load.
+    int ld_kt = 0, ld_t = 0;
+    const char *cur_a, *cur_b;
+    auto set_cursor = [&]() {
+        int m0, n0;
+        tile_origin(ld_t, m0, n0);
+        cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
+        cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
+    };
+    set_cursor();
+    const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
     auto issue_next = [&](int stage) {
-        const int k0 = ld_kt * kBK;
         char *dst_a = lds_bytes + stage * A_BYTES;
         char *dst_b = lds_bytes + 2 * A_BYTES + stage * B_BYTES;
-        const char *base_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(ld_m0 + 8 * wave) * K + k0);
-        const char *base_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(ld_n0 + 8 * wave) * K + k0);
-        const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(base_a + i * group_stride + lane_off),
+            __builtin_amdgcn_global_load_lds((gptr_t)(cur_a + i * group_stride + lane_off),
                                              (lptr_t)(dst_a + 1024 * (wave + WAVES * i)), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(base_b + i * group_stride + lane_off),
+            __builtin_amdgcn_global_load_lds((gptr_t)(cur_b + i * group_stride + lane_off),
                                              (lptr_t)(dst_b + 1024 * (wave + WAVES * i)), 16, 0, 0);
-        if (++ld_kt == KT) {
+        if (ld_kt + 1 < KT) {
+            ++ld_kt;
+            cur_a += kBK * 2;
+            cur_b += kBK * 2;
+        } else if (ld_t + 1 < my_tiles) {
             ld_kt = 0;
             ++ld_t;
-            if (ld_t < my_tiles) tile_origin(ld_t, ld_m0, ld_n0);
+            set_cursor();
         }
     };
 
