@@ -374,6 +374,14 @@ def cpu_baseline_softmax(keep, cfg):
         ref = oracle.softmax(x, vl, keep["rps"])
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
+    # one thread, on the first sixteenth of the rows (whole sequences): the scalar port's own speed
+    nthreads = oracle.max_threads()
+    rows1 = max(keep["rps"] or 1, (rows // 16) // (keep["rps"] or 1) * (keep["rps"] or 1))
+    oracle.set_threads(1)
+    t0 = time.perf_counter()
+    oracle.softmax(x[:rows1], vl, keep["rps"])
+    single = time.perf_counter() - t0
+    oracle.set_threads(nthreads)
     d = np.abs(y.astype(np.float64) - ref)
     sel = ref >= np.finfo(np.float32).tiny
     parity = dict(rows_checked=rows, max_abs_err=float(d.max()), max_rel_err=float((d[sel] / ref[sel]).max()),
@@ -381,7 +389,9 @@ def cpu_baseline_softmax(keep, cfg):
     return dict(value=2 * rows * cols * 4 / best / 1e9, unit="GB/s", cores=oracle.max_threads(), kind="port",
                 sample="all %d rows x %d cols of the same device-resident input, %d threads, best of 3; "
                        "host cpus visible: %d" % (rows, cols, oracle.max_threads(), os.cpu_count() or 0),
-                seconds=best), parity
+                seconds=best,
+                single_thread=dict(value=2 * rows1 * cols * 4 / single / 1e9, unit="GB/s", cores=1,
+                                   sample="first %d rows, 1 thread, one run" % rows1, seconds=single)), parity
 
 
 def main():

@@ -493,15 +493,23 @@ int launch_block(const Args<IO> &a) {
     return launch_block_threads<IO, 1024>(a);
 }
 
-template <int IO>
-int launch_nocache(const Args<IO> &a) {
-    constexpr int kThreads = 1024;
-    int64_t grid = static_cast<int64_t>(compute_units()) * 4;
+template <int IO, int THREADS>
+int launch_nocache_threads(const Args<IO> &a) {
+    int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
     if (grid > a.rows) grid = a.rows;
-    layernorm_nocache_kernel<IO, kThreads><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    layernorm_nocache_kernel<IO, THREADS><<<dim3(static_cast<unsigned>(grid)), dim3(THREADS), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
+}
+
+// Workgroup size by row length: a thread should have several trips of four vectors to make.
+template <int IO>
+int launch_nocache(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
+    if (nvec <= 2048) return launch_nocache_threads<IO, 256>(a);
+    if (nvec <= 8192) return launch_nocache_threads<IO, 512>(a);
+    return launch_nocache_threads<IO, 1024>(a);
 }
 
 template <int IO>
