@@ -63,12 +63,10 @@ struct Args {
 };
 
 // ---------------------------------------------------------------- WARP policy
-// A wavefront takes BATCH consecutive row groups (a row group = 64 / LPR rows, one per lane
-// group); the loads of group b + 1 are issued before group b is reduced and stored, so reads
-// and writes of a wave overlap and gamma/beta are fetched once per BATCH groups.
+// A wavefront takes one row group (64 / LPR rows, one per lane group) per trip.
 // FULL: cols == LPR * VPL vectors, every lane folds the same number of elements (no per-vector bounds
 // checks, and the lanes merge with the equal-count form).
-template <int IO, int LPR, int VPL, bool FULL, int BATCH>
+template <int IO, int LPR, int VPL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<IO>::elem *in,
                                                              typename Io<IO>::elem *out,
                                                              float *__restrict__ mean_out,
@@ -87,7 +85,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     const int nvec = cols / E;
     const int64_t waves_per_block = blockDim.x >> 6;
     const int64_t wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * (RPW * BATCH);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * waves_per_block * RPW;
 
     // gamma/beta of this lane's columns stay in registers across rows.  They are fetched behind the first
     // row's loads: memory returns in order, so loads issued ahead of the row would stand between the row
@@ -162,24 +160,20 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     };
 
     bool have_affine = false;
-    for (int64_t row0 = wave * (RPW * BATCH); row0 < rows; row0 += stride) {
-        float v[2][VPL][E];
-        load_rows(v[0], row0 + sub);
+    for (int64_t row0 = wave * RPW; row0 < rows; row0 += stride) {
+        float v[VPL][E];
+        load_rows(v, row0 + sub);
         if (!have_affine) {
             load_affine();
             have_affine = true;
         }
-#pragma unroll
-        for (int bt = 0; bt < BATCH; ++bt) {
-            if (bt + 1 < BATCH) load_rows(v[(bt + 1) & 1], row0 + (bt + 1) * RPW + sub);
-            finish_rows(v[bt & 1], row0 + bt * RPW + sub);
-        }
+        finish_rows(v, row0 + sub);
     }
 }
 
 // --------------------------------------------------------------- BLOCK policy
-// Workgroup-wide Welford all-reduce: per-wave triplets through LDS, folded by
-// every thread in the same order.
+// Workgroup-wide Welford all-reduce: per-wave triplets through LDS, then merged as a tree by
+// every wave in the same way.
 template <int THREADS>
 __device__ __forceinline__ wave::Welford block_welford_allreduce(wave::Welford w, float *lds) {
     constexpr int WAVES = THREADS / 64;
@@ -368,21 +362,21 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
 }
 
 // ------------------------------------------------------------------ dispatch
-template <int IO, int LPR, int VPL, bool FULL, int BATCH>
-int launch_wave_batch(const Args<IO> &a) {
+template <int IO, int LPR, int VPL, bool FULL>
+int launch_wave_full(const Args<IO> &a) {
     constexpr int RPW = 64 / LPR;
     // Single-wavefront workgroups by default (measured slightly faster than 256 threads).
     int threads = tuning("layernorm.wave_threads");
     if (threads != 128 && threads != 256) threads = 64;
-    const int64_t rows_per_block = static_cast<int64_t>(RPW) * BATCH * (threads / 64);
+    const int64_t rows_per_block = static_cast<int64_t>(RPW) * (threads / 64);
     const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
-    // One batch per wavefront by default; a positive knob caps the grid (grid-stride loop) instead.
+    // One row group per wavefront by default; a positive knob caps the grid (grid-stride loop) instead.
     int64_t grid = needed;
     const int per_cu = tuning("layernorm.blocks_per_cu");
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    layernorm_wave_kernel<IO, LPR, VPL, FULL, BATCH><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+    layernorm_wave_kernel<IO, LPR, VPL, FULL><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
@@ -393,8 +387,8 @@ int launch_wave(const Args<IO> &a) {
     // One row group per wavefront: batches of 2 and 4 row groups per wave (gamma and beta fetched once per
     // batch, the next group's loads issued before the current one is reduced) measured 5-8 % slower on
     // MI355X at [16384, 768] - the hardware keeps more independent waves in flight than a batch keeps loads.
-    if (a.cols == LPR * VPL * Io<IO>::E) return launch_wave_batch<IO, LPR, VPL, true, 1>(a);
-    return launch_wave_batch<IO, LPR, VPL, false, 1>(a);
+    if (a.cols == LPR * VPL * Io<IO>::E) return launch_wave_full<IO, LPR, VPL, true>(a);
+    return launch_wave_full<IO, LPR, VPL, false>(a);
 }
 
 template <int IO, int LPR>
