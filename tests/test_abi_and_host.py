@@ -96,6 +96,7 @@ def test_input_generators():
     assert vl.min() >= 64 and vl.max() <= 512 and vl.max() > 500 and vl.min() < 76
     assert inputs.algorithmic_work(1) == 201326592 and inputs.algorithmic_work(2) == 100800512
     assert inputs.algorithmic_work(5) == 3221225472 and inputs.algorithmic_work(4) == 77309411328
+    assert inputs.algorithmic_work(3) == 2147483648
 
 
 @pytest.mark.gpu
@@ -137,3 +138,13 @@ def test_device_fill_matches_host_generator(ko):
     dev = buf.download(np.float32, (n,))
     assert np.all(np.abs(dev - host) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))  # libm vs device log/cos: <= 1 ulp
     assert (dev != host).mean() < 0.01
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus value ends with a message, before anything touches a device."""
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout)
+
