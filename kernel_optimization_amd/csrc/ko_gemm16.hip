@@ -184,7 +184,9 @@ __device__ __forceinline__ void tile_of(const Params &p, int b, int grid, int t,
 // four consecutive columns per (i, j, q).  `region` is this wave's own piece of LDS, free for reuse.
 // The LDS transpose runs in PARTS passes over WTM / PARTS rows each, so that a wave needs
 // only WTM * WTN * 2 / PARTS bytes of LDS.
-template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1>
+// WAIT_VM: wait for this wave's outstanding vector memory operations right before the first global store
+// (the caller has loads in flight that it wants confirmed while they are still the only ones outstanding).
+template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1, bool WAIT_VM = false>
 __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
                                            int lane, int row0, int col0) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -241,6 +243,9 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 }
             }
             wave_lds_fence();
+            if constexpr (WAIT_VM) {
+                if (part == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
 #pragma unroll
             for (int it = 0; it < PROWS / ROWS_PER_ITER; ++it) {
                 const int row = it * ROWS_PER_ITER + lane / ROW_CHUNKS;
@@ -298,8 +303,10 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 // function XOR-ed into the chunk index of the LDS stages: 0 = row % 8 (conflict free for 8
 // consecutive rows when two rows share a bank line of 32 banks), 1 = (row / 2) % 8 (conflict
 // free for 16 consecutive rows on 64 banks, where two 128-byte rows make one bank line).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_,
+          bool SPARE_EPILOGUE_ = false>
 struct Tiling {
+    static constexpr bool SPARE_EPILOGUE = SPARE_EPILOGUE_;  // pinned kernel: see SPARE there
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, REG_STAGES = REG_STAGES_;
     static constexpr bool FRAG_DB = FRAG_DB_;
     static constexpr int SWIZZLE = SWIZZLE_;
@@ -855,6 +862,16 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         }
     };
 
+    // SPARE: the epilogue transposes through the 32 KB of LDS that the two stages leave free (four passes of
+    // 32 rows per wave) instead of through the stage just consumed.  The loads of the K tile after next then
+    // go out at their usual place, ahead of the epilogue; each wave confirms them (vmcnt(0)) before its first
+    // store, while they are still its only outstanding memory operations, and the next K tile's barrier skips
+    // the vmcnt wait.  Stores count in vmcnt too on this architecture: waiting there would mean waiting for
+    // the whole chip's 32 MB burst of output to drain before the next K tile could be published.
+    constexpr int SPARE_BYTES = 160 * 1024 - 2 * (A_BYTES + B_BYTES);
+    constexpr bool SPARE = T::SPARE_EPILOGUE && TM % 4 == 0 && WTM * WTN * 2 / 4 * WAVES <= SPARE_BYTES;
+    bool stores_in_flight = false;  // SPARE: set by the epilogue, cleared at the next barrier
+
     int t = 0;
     auto step_fn = [&](int step, auto last_c, auto stage_c) {
         constexpr int S = decltype(stage_c)::value;
@@ -871,9 +888,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         wait_frags(0);
         mfma_step(C0{}, [&](auto r) { read_one(r, C3{}, C1{}, stage_c); });
         wait_frags(1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if constexpr (SPARE) {
+            // right after an epilogue the loads this barrier publishes were confirmed before the stores went out
+            if (!stores_in_flight) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            stores_in_flight = false;
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
         lds_barrier();
-        if (!last_of_tile && step + 2 < total) issue_next(S);
+        if ((SPARE || !last_of_tile) && step + 2 < total) issue_next(S);
         // K step 3, with step 0 of the next K tile read out of the other stage (after the very last
         // K tile these reads fetch stale but in-bounds LDS contents that nothing uses)
         mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Other{}); });
@@ -883,15 +906,24 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             tile_origin(t, m0, n0);
             // MFMA results are read by vector ALU instructions next: cover the issue-to-write latency
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-            constexpr int REGION = WTM * WTN * 2 / EPI_PARTS;  // bytes per wave
-            static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
-            char *region = wave < WAVES / 2 ? lds_bytes + S * A_BYTES + wave * REGION
-                                            : lds_bytes + 2 * A_BYTES + S * B_BYTES + (wave - WAVES / 2) * REGION;
-            store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
-                                                            m0 + wm * WTM, n0 + wn * WTN);
-            clear_acc();
-            lds_barrier();  // every wave is done with its transpose region in stage S
-            if (step + 2 < total) issue_next(S);
+            if constexpr (SPARE) {
+                constexpr int REGION = WTM * WTN * 2 / 4;  // bytes per wave and pass
+                char *region = lds_bytes + 2 * (A_BYTES + B_BYTES) + wave * REGION;
+                store_tile<WTM, WTN, 1, BF16, false, 4, true>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                                                              m0 + wm * WTM, n0 + wn * WTN);
+                clear_acc();
+                stores_in_flight = true;
+            } else {
+                constexpr int REGION = WTM * WTN * 2 / EPI_PARTS;  // bytes per wave
+                static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
+                char *region = wave < WAVES / 2 ? lds_bytes + S * A_BYTES + wave * REGION
+                                                : lds_bytes + 2 * A_BYTES + S * B_BYTES + (wave - WAVES / 2) * REGION;
+                store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                                                                m0 + wm * WTM, n0 + wn * WTN);
+                clear_acc();
+                lds_barrier();  // every wave is done with its transpose region in stage S
+                if (step + 2 < total) issue_next(S);
+            }
             ++t;
         }
     };
@@ -920,7 +952,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
 
 template <class T, bool BF16>
 int launch_pinned(Params p, hipStream_t stream) {
-    constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
+    constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
     auto kernel = gemm16_pinned_kernel<T, BF16>;
@@ -1001,6 +1033,7 @@ int launch(Params p, hipStream_t stream) {
 using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 128x64
 using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
 
+using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigTall = Tiling<256, 256, 4, 2, 1, true, 1>; // 8 waves, wave tile 64x128
 
 // The direct-to-LDS kernels need full 256x256x64 tiles and K-contiguous operands.
@@ -1027,7 +1060,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         if constexpr (!B_ROW_MAJOR) {
             if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) {
-                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBig, BF16>(p, stream);
+                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBigSpare, BF16>(p, stream);
                 return launch_persistent<TileBig, BF16>(p, stream);
             }
         }
@@ -1042,6 +1075,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         case 31: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 51: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
