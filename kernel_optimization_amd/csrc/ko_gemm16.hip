@@ -304,9 +304,10 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 // consecutive rows when two rows share a bank line of 32 banks), 1 = (row / 2) % 8 (conflict
 // free for 16 consecutive rows on 64 banks, where two 128-byte rows make one bank line).
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int REG_STAGES_, bool FRAG_DB_, int SWIZZLE_,
-          bool SPARE_EPILOGUE_ = false>
+          bool SPARE_EPILOGUE_ = false, bool SPREAD_LOADS_ = false>
 struct Tiling {
     static constexpr bool SPARE_EPILOGUE = SPARE_EPILOGUE_;  // pinned kernel: see SPARE there
+    static constexpr bool SPREAD_LOADS = SPREAD_LOADS_;      // pinned kernel with SPARE: loads one by one in K step 3
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, REG_STAGES = REG_STAGES_;
     static constexpr bool FRAG_DB = FRAG_DB_;
     static constexpr int SWIZZLE = SWIZZLE_;
@@ -774,6 +775,31 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     };
     set_cursor();
     const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
+    auto advance_cursor = [&]() {
+        if (ld_kt + 1 < KT) {
+            ++ld_kt;
+            cur_a += kBK * 2;
+            cur_b += kBK * 2;
+        } else if (ld_t + 1 < my_tiles) {
+            ld_kt = 0;
+            ++ld_t;
+            set_cursor();
+        }
+    };
+    // load number I of the cursor's K tile (the A loads first, then the B loads); the last one moves the cursor
+    auto issue_one = [&](int stage, auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        if constexpr (I < A_LOADS) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(cur_a + I * group_stride + lane_off),
+                                             (lptr_t)(lds_bytes + stage * A_BYTES + 1024 * (wave + WAVES * I)), 16, 0, 0);
+        } else {
+            constexpr int J = I - A_LOADS;
+            __builtin_amdgcn_global_load_lds(
+                (gptr_t)(cur_b + J * group_stride + lane_off),
+                (lptr_t)(lds_bytes + 2 * A_BYTES + stage * B_BYTES + 1024 * (wave + WAVES * J)), 16, 0, 0);
+            if constexpr (J == B_LOADS - 1) advance_cursor();
+        }
+    };
     auto issue_next = [&](int stage) {
         char *dst_a = lds_bytes + stage * A_BYTES;
         char *dst_b = lds_bytes + 2 * A_BYTES + stage * B_BYTES;
@@ -831,7 +857,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     };
 
     // MFMAs of one K step out of fragment set SLOT, with the reads reader(R) spread over the first ones
-    auto mfma_step = [&](auto slot_c, auto reader) {
+    // and after(IDX) called behind every MFMA
+    auto mfma_step = [&](auto slot_c, auto reader, auto after) {
         constexpr int SLOT = decltype(slot_c)::value;
         static_for<TM * TN>([&](auto idx_c) {
             constexpr int IDX = decltype(idx_c)::value;
@@ -841,8 +868,10 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
                 reader(std::integral_constant<int, 2 * IDX>{});
                 reader(std::integral_constant<int, 2 * IDX + 1>{});
             }
+            after(idx_c);
         });
     };
+    auto nothing = [](auto) {};
 
     // all reads issued so far have landed; the fake operands keep later MFMAs behind this point
     auto wait_frags = [&](int slot) {
@@ -882,11 +911,11 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         using C2 = std::integral_constant<int, 2>;
         using C3 = std::integral_constant<int, 3>;
         // K steps 0..2: their MFMAs, with the next step's fragments read early in each
-        mfma_step(C0{}, [&](auto r) { read_one(r, C1{}, C1{}, stage_c); });
+        mfma_step(C0{}, [&](auto r) { read_one(r, C1{}, C1{}, stage_c); }, nothing);
         wait_frags(1);
-        mfma_step(C1{}, [&](auto r) { read_one(r, C2{}, C0{}, stage_c); });
+        mfma_step(C1{}, [&](auto r) { read_one(r, C2{}, C0{}, stage_c); }, nothing);
         wait_frags(0);
-        mfma_step(C0{}, [&](auto r) { read_one(r, C3{}, C1{}, stage_c); });
+        mfma_step(C0{}, [&](auto r) { read_one(r, C3{}, C1{}, stage_c); }, nothing);
         wait_frags(1);
         if constexpr (SPARE) {
             // right after an epilogue the loads this barrier publishes were confirmed before the stores went out
@@ -896,10 +925,20 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         lds_barrier();
-        if ((SPARE || !last_of_tile) && step + 2 < total) issue_next(S);
         // K step 3, with step 0 of the next K tile read out of the other stage (after the very last
         // K tile these reads fetch stale but in-bounds LDS contents that nothing uses)
-        mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Other{}); });
+        if constexpr (SPARE && T::SPREAD_LOADS) {
+            // one load of the K tile after next behind each MFMA, unconditionally: past the end of the work
+            // the cursor stands still and the loads fetch the last K tile again into a stage nobody reads
+            // (the epilogue waits for them before its first store, so none is in flight at the end)
+            static_assert(TM * TN >= A_LOADS + B_LOADS, "");
+            mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Other{}); }, [&](auto i_c) {
+                if constexpr (decltype(i_c)::value < A_LOADS + B_LOADS) issue_one(S, i_c);
+            });
+        } else {
+            if ((SPARE || !last_of_tile) && step + 2 < total) issue_next(S);
+            mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Other{}); }, nothing);
+        }
         wait_frags(0);
         if constexpr (last_of_tile) {
             int m0, n0;
@@ -1034,6 +1073,7 @@ using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 12
 using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
 
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
+using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
 using TileBigTall = Tiling<256, 256, 4, 2, 1, true, 1>; // 8 waves, wave tile 64x128
 
 // The direct-to-LDS kernels need full 256x256x64 tiles and K-contiguous operands.
@@ -1060,7 +1100,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         if constexpr (!B_ROW_MAJOR) {
             if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) {
-                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBigSpare, BF16>(p, stream);
+                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBigSpread, BF16>(p, stream);
                 return launch_persistent<TileBig, BF16>(p, stream);
             }
         }
@@ -1076,6 +1116,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 51: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 53: return launch_direct<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
