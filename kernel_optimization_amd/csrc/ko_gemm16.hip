@@ -135,18 +135,17 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 }
 
 // Epilogue of one group of four consecutive columns n .. n+3 of row m (all inside the matrix):
-// v = act(alpha * acc + beta * C + bias).  C and bias are read as 8-byte groups.
+// v = act(alpha * acc + beta * C + bias).  c2 and b2 hold the group's four C and bias values (8 bytes
+// each, loaded by the caller - several groups at a time, so that the loads overlap).
 template <bool BF16>
-__device__ __forceinline__ void finish4(const Params &p, float (&v)[4], int64_t off, int n, bool use_c) {
+__device__ __forceinline__ void finish4(const Params &p, float (&v)[4], u32x2 c2, u32x2 b2, bool use_c) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] *= p.alpha;
     if (use_c) {
-        const u32x2 c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] += p.beta * to_float<BF16>(static_cast<uint16_t>(c2[e >> 1] >> ((e & 1) * 16)));
     }
     if (p.bias) {
-        const u32x2 b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] += to_float<BF16>(static_cast<uint16_t>(b2[e >> 1] >> ((e & 1) * 16)));
     }
@@ -214,6 +213,15 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
         u32x2 *region8 = reinterpret_cast<u32x2 *>(region);
         const u32x4 *region16 = reinterpret_cast<const u32x4 *>(region8);
         const int c = lane % ROW_CHUNKS;
+        // the bias of this lane's column groups, once per tile
+        u32x2 bias_q[TN][4];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                bias_q[j][q] = u32x2{0, 0};
+                if (p.bias) bias_q[j][q] = *reinterpret_cast<const u32x2 *>(p.bias + col0 + j * 32 + 8 * q + 4 * fhalf);
+            }
 #pragma unroll
         for (int part = 0; part < PARTS; ++part) {
             if (part > 0) wave_lds_fence();  // the previous pass has read its rows
@@ -221,6 +229,15 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
             for (int ii = 0; ii < PTM; ++ii) {
                 const int i = part * PTM + ii;
                 const int row = ii * 32 + frow;
+                // C of this 32-row block: all loads first, so that their latencies overlap
+                u32x2 c_q[TN][4];
+                if (use_c) {
+                    const uint16_t *crow = p.C + static_cast<int64_t>(row0 + i * 32 + frow) * N + col0 + 4 * fhalf;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) c_q[j][q] = *reinterpret_cast<const u32x2 *>(crow + j * 32 + 8 * q);
+                }
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -231,9 +248,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] *= alpha;
                         } else {  // C, bias and the activation enter before the one rounding to 16 bits
-                            const int gm = row0 + i * 32 + frow;
-                            const int gn = col0 + j * 32 + 8 * q + 4 * fhalf;
-                            finish4<BF16>(p, v, static_cast<int64_t>(gm) * N + gn, gn, use_c);
+                            finish4<BF16>(p, v, use_c ? c_q[j][q] : u32x2{0, 0}, bias_q[j][q], use_c);
                         }
                         u32x2 o;
                         o[0] = pack2<BF16>(v[0], v[1]);
@@ -273,7 +288,10 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int64_t off = static_cast<int64_t>(m) * N + n;
                 float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                 if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
-                    finish4<BF16>(p, v, off, n, use_c);
+                    u32x2 c2 = {0, 0}, b2 = {0, 0};
+                    if (use_c) c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+                    if (p.bias) b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
+                    finish4<BF16>(p, v, c2, b2, use_c);
                     u32x2 o;
                     o[0] = pack2<BF16>(v[0], v[1]);
                     o[1] = pack2<BF16>(v[2], v[3]);
@@ -1074,7 +1092,6 @@ using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64
 
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
-using TileBigTall = Tiling<256, 256, 4, 2, 1, true, 1>; // 8 waves, wave tile 64x128
 
 // The direct-to-LDS kernels need full 256x256x64 tiles and K-contiguous operands.
 template <class T, bool BF16, bool B_ROW_MAJOR, bool PINNED>
@@ -1112,9 +1129,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         case 9: return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
         case 10: return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
-        case 31: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
-        case 51: return launch_direct<TileBigTall, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
         case 53: return launch_direct<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
