@@ -1,50 +1,51 @@
-// Tensor over the C ABI (reference: common/tensor.cu:8-42).  Plain C++: no HIP headers.
+// Out-of-line part of Tensor: allocation and the four copies, all through the C ABI (no HIP headers).
+// The reference's counterpart is common/tensor.cu:8-42.
 #include "kernel_optimization/common/tensor.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <limits>
+#include <utility>
+
 #include "kernel_optimization/common/common.h"
 
-#include <cstdint>
+namespace ko_detail {
 
-Tensor::Tensor(size_t _size_in_bytes) : host_ptr(nullptr), device_ptr(nullptr), size_in_bytes(_size_in_bytes) {
-    this->host_ptr = new uint8_t[this->size_in_bytes ? this->size_in_bytes : 1];
-    checkKoErrors(ko_malloc(&this->device_ptr, this->size_in_bytes));
-}
+DeviceBlock::DeviceBlock(size_t bytes) { checkKoErrors(ko_malloc(&ptr_, bytes)); }
 
-Tensor::Tensor(Tensor &&rhs) : host_ptr(rhs.host_ptr), device_ptr(rhs.device_ptr), size_in_bytes(rhs.size_in_bytes) {
-    rhs.host_ptr = nullptr;
-    rhs.device_ptr = nullptr;
-    rhs.size_in_bytes = 0;
-}
-
-Tensor &Tensor::operator=(Tensor &&rhs) {
-    if (this != &rhs) {
-        this->release();
-        this->host_ptr = rhs.host_ptr;
-        this->device_ptr = rhs.device_ptr;
-        this->size_in_bytes = rhs.size_in_bytes;
-        rhs.host_ptr = nullptr;
-        rhs.device_ptr = nullptr;
-        rhs.size_in_bytes = 0;
-    }
+DeviceBlock &DeviceBlock::operator=(DeviceBlock &&other) noexcept {
+    std::swap(ptr_, other.ptr_);  // the old allocation leaves with `other`
     return *this;
 }
 
-void Tensor::release() {
-    if (this->host_ptr) delete[] reinterpret_cast<uint8_t *>(this->host_ptr);
-    if (this->device_ptr) checkKoErrors(ko_free(this->device_ptr));
-    this->host_ptr = nullptr;
-    this->device_ptr = nullptr;
+DeviceBlock::~DeviceBlock() {
+    if (ptr_ != nullptr) checkKoErrors(ko_free(ptr_));
 }
 
-Tensor::~Tensor() { this->release(); }
+size_t checked_byte_count(const std::vector<size_t> &shape, size_t bytes_per_element) {
+    size_t total = bytes_per_element;
+    for (size_t extent : shape) {
+        if (extent != 0 && total > std::numeric_limits<size_t>::max() / extent) {
+            std::fprintf(stderr, "Tensor: shape does not fit size_t\n");
+            std::exit(EXIT_FAILURE);
+        }
+        total *= extent;
+    }
+    return total;
+}
 
-void Tensor::host_to_device() { checkKoErrors(ko_memcpy_h2d(this->device_ptr, this->host_ptr, this->size_in_bytes)); }
+}  // namespace ko_detail
+
+Tensor::Tensor(size_t bytes) : host_(new unsigned char[bytes > 0 ? bytes : 1]), device_(bytes), bytes_(bytes) {}
+
+void Tensor::host_to_device() { checkKoErrors(ko_memcpy_h2d(device_.get(), host_.get(), bytes_)); }
+
+void Tensor::device_to_host() { checkKoErrors(ko_memcpy_d2h(host_.get(), device_.get(), bytes_)); }
 
 void Tensor::host_to_device_async(ko_stream_t &stream) {
-    checkKoErrors(ko_memcpy_h2d_async(this->device_ptr, this->host_ptr, this->size_in_bytes, stream));
+    checkKoErrors(ko_memcpy_h2d_async(device_.get(), host_.get(), bytes_, stream));
 }
 
-void Tensor::device_to_host() { checkKoErrors(ko_memcpy_d2h(this->host_ptr, this->device_ptr, this->size_in_bytes)); }
-
 void Tensor::device_to_host_async(ko_stream_t &stream) {
-    checkKoErrors(ko_memcpy_d2h_async(this->host_ptr, this->device_ptr, this->size_in_bytes, stream));
+    checkKoErrors(ko_memcpy_d2h_async(host_.get(), device_.get(), bytes_, stream));
 }
