@@ -24,6 +24,8 @@
 // row in the registers of a workgroup, per-wave triplets through LDS;
 // BLOCK_NOCACHE (LayerNormBlockNoCacheImpl :254-300) = two reads of the row.
 #include "ko_internal.h"
+#include <type_traits>
+
 #include "wave64.h"
 
 namespace ko {
@@ -194,6 +196,13 @@ __device__ __forceinline__ wave::Welford block_welford_allreduce(wave::Welford w
     return wave::welford_allreduce<WAVES>(wave::Welford{lds[i], lds[16 + i], lds[32 + i]});
 }
 
+// base + bytes, for addresses formed from a uniform pointer and a 32-bit per-lane offset
+template <class T>
+__device__ __forceinline__ T *at_bytes(T *base, uint32_t bytes) {
+    typedef typename std::conditional<std::is_const<T>::value, const char, char>::type Byte;
+    return reinterpret_cast<T *>(reinterpret_cast<Byte *>(base) + bytes);
+}
+
 // y = (x - mean) * rstd [* gamma] [+ beta] for one vector; gamma/beta are read here (long rows:
 // they do not fit the registers next to the row).
 template <int IO>
@@ -213,6 +222,8 @@ __device__ __forceinline__ void normalize_vec(const float (&x)[Io<IO>::E], float
     }
 }
 
+// One workgroup per row, the row held in registers between its single read and its single write; both are
+// nontemporal (every byte is touched once; measured faster than cached accesses on rows of 16 KB and more).
 template <int IO, int THREADS, int VPL>
 __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename Io<IO>::elem *in,
                                                                   typename Io<IO>::elem *out,
@@ -243,14 +254,20 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
             if (beta) Io<IO>::template load<false>(beta + E * j, b[k]);
         }
     }
+    // Byte offset of this thread's first vector in a row (vector k lies k * THREADS * 16 bytes further).  The
+    // row loop passes it through an empty asm: addresses are then formed per use from a uniform base and this
+    // one register, instead of 2 * VPL pointers to gamma and beta being kept across rows (which spilled).
+    uint32_t first = threadIdx.x * 16u;
+    constexpr uint32_t kStep = THREADS * 16u;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
         float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
             if (j < nvec) {
-                Io<IO>::template load<false>(src + E * j, v[k]);
+                Io<IO>::template load<true>(at_bytes(src, first + k * kStep), v[k]);
             } else {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
@@ -281,9 +298,18 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
 #pragma unroll
                     for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[k][e], b[k][e]);
                 } else {
-                    normalize_vec<IO>(v[k], mean, rstd, gamma, beta, E * j, y);
+                    float gk[E], bk[E];
+                    if (gamma) Io<IO>::template load<false>(at_bytes(gamma, first + k * kStep), gk);
+                    if (beta) Io<IO>::template load<false>(at_bytes(beta, first + k * kStep), bk);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        float t = (v[k][e] - mean) * rstd;
+                        if (gamma) t *= gk[e];
+                        if (beta) t += bk[e];
+                        y[e] = t;
+                    }
                 }
-                Io<IO>::template store<false>(dst + E * j, y);
+                Io<IO>::template store<true>(at_bytes(dst, first + k * kStep), y);
             }
         }
         if (threadIdx.x == 0) {
@@ -338,11 +364,15 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
         typename Io<IO>::elem *dst = out + row * cols;
-        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+        // Second pass from the row's end backwards (what the first pass read last is the likeliest to be in a
+        // cache still), with nontemporal accesses: nothing is touched again.
+        const int trips = (nvec + THREADS * UNROLL - 1) / (THREADS * UNROLL);
+        for (int t = trips - 1; t >= 0; --t) {
+            const int j0 = threadIdx.x + t * (THREADS * UNROLL);
             float x[UNROLL][E];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) Io<IO>::template load<false>(src + E * (j0 + u * THREADS), x[u]);
+                if (j0 + u * THREADS < nvec) Io<IO>::template load<true>(src + E * (j0 + u * THREADS), x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const int j = j0 + u * THREADS;
@@ -351,7 +381,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] -= x0;
                 normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                Io<IO>::template store<false>(dst + E * j, y);
+                Io<IO>::template store<true>(dst + E * j, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -417,12 +447,11 @@ int launch_wave_lpr(const Args<IO> &a, int lpr) {
 }
 
 // Longest row per policy, in 16-byte vectors: 512 per wavefront (2048 fp32 or 4096 16-bit columns); per
-// workgroup 8192 vectors of fp32 (32768 columns) or 4096 vectors of 16-bit values (32768 columns: eight
-// vectors of eight values per thread do not fit the 128 registers of a 1024-thread workgroup).
+// workgroup 80 values per thread of 1024 threads (81920 columns).
 constexpr int kWaveMaxVpl = 8;
 constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
 template <int IO>
-constexpr int kBlockMaxVecs = 1024 * (Io<IO>::E == 8 ? 4 : 8);
+constexpr int kBlockMaxVecs = 1024 * (80 / Io<IO>::E);
 
 // Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
 // {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
@@ -466,8 +495,18 @@ int launch_block_threads(const Args<IO> &a) {
                                                                   a.inv_denominator)
     if (vpl <= 1) KO_LN_BLOCK(1);
     else if (vpl <= 2) KO_LN_BLOCK(2);
-    else if (vpl <= 4 || Io<IO>::E == 8) KO_LN_BLOCK(4);
-    else KO_LN_BLOCK((Io<IO>::E == 8 ? 4 : 8));
+    else if (vpl <= 4) KO_LN_BLOCK(4);
+    else if (vpl <= 8) KO_LN_BLOCK(8);
+    else if constexpr (THREADS == 1024) {
+        // a single resident workgroup of 1024 threads has 128 registers per thread: up to 80 hold the row
+        if constexpr (Io<IO>::E == 4) {
+            if (vpl <= 12) KO_LN_BLOCK(12);
+            else if (vpl <= 16) KO_LN_BLOCK(16);
+            else KO_LN_BLOCK(20);
+        } else {
+            KO_LN_BLOCK(10);
+        }
+    }
 #undef KO_LN_BLOCK
     KO_CHECK_LAUNCH();
     return KO_OK;

@@ -23,6 +23,8 @@
 // Mask: columns j >= valid_len[row / rows_per_seq] take the value -10000.  Vectors
 // that lie wholly in the padded part are not loaded.
 #include "ko_internal.h"
+#include <type_traits>
+
 #include "wave64.h"
 
 #include <cfloat>
@@ -51,6 +53,13 @@ __device__ __forceinline__ void load_row_vec(const typename Io<IO>::elem *row, i
             for (int e = 0; e < E; ++e) v[e] = kMaskValue;
         }
     }
+}
+
+// base + bytes, for addresses formed from a uniform pointer and a 32-bit per-lane offset
+template <class T>
+__device__ __forceinline__ T *at_bytes(T *base, uint32_t bytes) {
+    typedef typename std::conditional<std::is_const<T>::value, const char, char>::type Byte;
+    return reinterpret_cast<T *>(reinterpret_cast<Byte *>(base) + bytes);
 }
 
 template <int E>
@@ -154,6 +163,25 @@ __device__ __forceinline__ float block_allreduce(float v, float *lds, float iden
     return r;
 }
 
+// One barrier per reduction: `slot` holds this reduction's partials and is not written again before every
+// wave has passed the workgroup's next barrier (the caller alternates between two slots).
+template <int THREADS, class Op>
+__device__ __forceinline__ float block_allreduce_slot(float v, float *slot, float identity) {
+    constexpr int WAVES = THREADS / 64;
+    v = wave::allreduce<64, Op>(v);
+    if constexpr (WAVES == 1) return v;
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = identity;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) r = Op()(r, slot[w]);
+    return r;
+}
+
+// One workgroup per row, the row held in registers between its single read and its single write.  Loads and
+// stores bypass the caches' retention (nontemporal): every byte is touched once, and on rows of 16 to 128 KB
+// that measured 9 % faster than cached accesses.  Issuing the next row's loads ahead of the reductions
+// measured no different: two or more resident workgroups already cover each other's reductions.
 template <int IO, int THREADS, int VPL, bool MASKED>
 __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename Io<IO>::elem *in,
                                                                 typename Io<IO>::elem *out, int64_t rows,
@@ -161,9 +189,15 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                                                                 const int32_t *__restrict__ valid_len,
                                                                 int64_t rows_per_seq) {
     constexpr int E = Io<IO>::E;
-    __shared__ float lds[16];
+    __shared__ float lds[2][16];
     const int nvec = cols / E;
+    // Byte offset of this thread's first vector in a row (vector k lies k * THREADS * 16 bytes further); passed
+    // through an empty asm per row so that addresses are formed per use from the uniform row pointer and this
+    // one register rather than kept as VPL pointer pairs.
+    uint32_t first = threadIdx.x * 16u;
+    constexpr uint32_t kStep = THREADS * 16u;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
@@ -172,7 +206,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
             if (j < nvec) {
-                load_row_vec<IO, MASKED, false>(src, j, vlen, v[k]);
+                load_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), 0, vlen - E * j, v[k]);
             } else {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
@@ -181,7 +215,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
         float m = -FLT_MAX;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) m = vec_max<E>(v[k], m);
-        m = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
+        m = block_allreduce_slot<THREADS, wave::Max>(m, lds[0], -FLT_MAX);
         const bool pad_is_zero = MASKED && m > kMaskValue + 128.0f;  // see the wave kernel
         float s = 0.0f;
 #pragma unroll
@@ -197,7 +231,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                 }
             }
         }
-        s = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
+        s = block_allreduce_slot<THREADS, wave::Sum>(s, lds[1], 0.0f);
         const float inv = 1.0f / s;
         typename Io<IO>::elem *dst = out + row * cols;
 #pragma unroll
@@ -206,7 +240,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
             if (j < nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
-                Io<IO>::template store<false>(dst + E * j, v[k]);
+                Io<IO>::template store<true>(at_bytes(dst, first + k * kStep), v[k]);
             }
         }
     }
@@ -257,18 +291,23 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
         const float gs = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
         const float inv = 1.0f / gs;
         typename Io<IO>::elem *dst = out + row * cols;
-        for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+        // Second pass from the row's end backwards: what the first pass read last is the likeliest to be in a
+        // cache still (measured 5 % faster at 65536 columns, no different at 131072).  Nontemporal accesses from
+        // here on: nothing is touched again (19 % faster than cached ones at 131072 columns).
+        const int trips = (nvec + THREADS * UNROLL - 1) / (THREADS * UNROLL);
+        for (int t = 0; t < trips; ++t) {
+            const int j0 = threadIdx.x + (trips - 1 - t) * (THREADS * UNROLL);
             float x[UNROLL][E];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, false>(src, j0 + u * THREADS, vlen, x[u]);
+                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, true>(src, j0 + u * THREADS, vlen, x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const int j = j0 + u * THREADS;
                 if (j >= nvec) break;
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
-                Io<IO>::template store<false>(dst + E * j, x[u]);
+                Io<IO>::template store<true>(dst + E * j, x[u]);
             }
         }
     }
@@ -337,7 +376,12 @@ constexpr int kWaveMaxVpl = 8;
 // Longest row per policy, in 16-byte vectors: 512 per wavefront, 8192 per workgroup
 // (fp32: 2048 and 32768 columns; 16-bit: twice that).
 constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
-constexpr int kBlockMaxVecs = 1024 * 8;
+// BLOCK policy: at most 96 values per thread of a 1024-thread workgroup (98304 columns).  With a mask the
+// kernels past 64 values per thread spill registers, and AUTO leaves those rows to the re-reading policy.
+template <int IO>
+constexpr int kBlockMaxVecs = 1024 * (96 / Io<IO>::E);
+template <int IO>
+constexpr int kBlockMaxVecsMasked = 1024 * (64 / Io<IO>::E);
 
 // Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
 // {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
@@ -385,10 +429,21 @@ int launch_block_threads(const Args<IO> &a) {
 #define KO_SM_BLOCK(V)                                                                         \
     softmax_block_kernel<IO, THREADS, V, MASKED><<<g, b, 0, a.stream>>>(                         \
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq)
+    constexpr int E = Io<IO>::E;
     if (vpl <= 1) KO_SM_BLOCK(1);
     else if (vpl <= 2) KO_SM_BLOCK(2);
     else if (vpl <= 4) KO_SM_BLOCK(4);
-    else KO_SM_BLOCK(8);
+    else if (vpl <= 8) KO_SM_BLOCK(8);
+    else if constexpr (THREADS == 1024) {
+        // a single resident workgroup of 1024 threads has 128 registers per thread: up to 96 hold the row
+        if constexpr (E == 4) {
+            if (vpl <= 12) KO_SM_BLOCK(12);
+            else if (vpl <= 16) KO_SM_BLOCK(16);
+            else if (vpl <= 20) KO_SM_BLOCK(20);
+            else KO_SM_BLOCK(24);
+        } else if (vpl <= 10) KO_SM_BLOCK(10);
+        else KO_SM_BLOCK(12);
+    }
 #undef KO_SM_BLOCK
     KO_CHECK_LAUNCH();
     return KO_OK;
@@ -433,7 +488,7 @@ int dispatch(const Args<IO> &a, int policy) {
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
-                 : nvec <= kBlockMaxVecs ? KO_POLICY_BLOCK
+                 : nvec <= (MASKED ? kBlockMaxVecsMasked<IO> : kBlockMaxVecs<IO>) ? KO_POLICY_BLOCK
                                          : KO_POLICY_BLOCK_NOCACHE;
     }
     switch (policy) {
@@ -444,9 +499,9 @@ int dispatch(const Args<IO> &a, int policy) {
                             a.cols);
             return launch_wave_any<IO, MASKED>(a);
         case KO_POLICY_BLOCK:
-            if (nvec > kBlockMaxVecs)
+            if (nvec > kBlockMaxVecs<IO>)
                 return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs * E,
+                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs<IO> * E,
                             a.cols);
             return launch_block<IO, MASKED>(a);
         case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO, MASKED>(a);

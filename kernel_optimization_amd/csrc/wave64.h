@@ -228,11 +228,18 @@ template <>
 struct Io<IO_F32> {
     typedef float elem;
     static constexpr int E = 4;
+    typedef float4v raw;  // one 16-byte vector as loaded, before conversion
     template <bool NT>
-    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
-        const float4v x = load4<NT>(p);
+    static __device__ __forceinline__ raw load_raw(const elem *p) {
+        return load4<NT>(p);
+    }
+    static __device__ __forceinline__ void unpack(raw x, float (&v)[E]) {
 #pragma unroll
         for (int e = 0; e < E; ++e) v[e] = x[e];
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        unpack(load_raw<NT>(p), v);
     }
     template <bool NT>
     static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
@@ -260,11 +267,19 @@ struct Io<IO_F16> {
     typedef uint16_t elem;
     static constexpr int E = 8;
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    typedef uint4v raw;
     template <bool NT>
-    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
-        const half8 h = __builtin_bit_cast(half8, load_bits16<NT>(p));
+    static __device__ __forceinline__ raw load_raw(const elem *p) {
+        return load_bits16<NT>(p);
+    }
+    static __device__ __forceinline__ void unpack(raw x, float (&v)[E]) {
+        const half8 h = __builtin_bit_cast(half8, x);
 #pragma unroll
         for (int e = 0; e < E; ++e) v[e] = static_cast<float>(h[e]);
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        unpack(load_raw<NT>(p), v);
     }
     template <bool NT>
     static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
@@ -282,14 +297,21 @@ template <>
 struct Io<IO_BF16> {
     typedef uint16_t elem;
     static constexpr int E = 8;
+    typedef uint4v raw;
     template <bool NT>
-    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
-        const uint4v x = load_bits16<NT>(p);
+    static __device__ __forceinline__ raw load_raw(const elem *p) {
+        return load_bits16<NT>(p);
+    }
+    static __device__ __forceinline__ void unpack(raw x, float (&v)[E]) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             v[2 * e] = __builtin_bit_cast(float, x[e] << 16);
             v[2 * e + 1] = __builtin_bit_cast(float, x[e] & 0xffff0000u);
         }
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        unpack(load_raw<NT>(p), v);
     }
     template <bool NT>
     static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {

@@ -47,8 +47,9 @@ def test_softmax_every_lane_mapping(ko, lpr, cols):
 
 @pytest.mark.parametrize("policy,rows,cols", [
     (2, 37, 128), (2, 19, 1024), (2, 9, 4096), (2, 5, 8192), (2, 3, 32768), (2, 11, 5000),
-    (3, 37, 128), (3, 19, 1024), (3, 4, 40000), (3, 2, 131072),
-    (0, 3, 4096), (0, 2, 65536)])
+    (2, 3, 40960), (2, 2, 49152), (2, 3, 65536), (2, 2, 81920), (2, 3, 98304), (2, 2, 70004), (2, 5000, 2052),
+    (3, 5000, 2052), (3, 37, 128), (3, 19, 1024), (3, 4, 40000), (3, 2, 131072),
+    (0, 3, 4096), (0, 2, 65536), (0, 2, 98304), (0, 2, 98308)])
 def test_softmax_block_policies(ko, policy, rows, cols):
     """Row-per-workgroup (BLOCK) and re-read (BLOCK_NOCACHE) policies, and AUTO on long rows."""
     x = inputs.normal_f32((rows, cols), 4321 + cols, 0.0, 4.0)
@@ -74,6 +75,18 @@ def test_masked_softmax_matches_oracle(ko, policy):
             assert np.all(blk[:, L:] == 0.0)
         if L == 0:
             np.testing.assert_array_equal(blk, np.full_like(blk, 1.0 / cols))
+
+
+@pytest.mark.parametrize("policy,cols", [(2, 16384), (2, 65536), (2, 98304), (3, 98304), (0, 65536), (0, 98304)])
+def test_masked_softmax_long_rows(ko, policy, cols):
+    """Masks on rows that one workgroup holds in registers (up to 96 values per thread) or reads twice."""
+    vl = np.array([0, 1, 5, cols // 3 + 1, cols - 4, cols - 1, cols, cols + 7], np.int32)
+    rows_per_seq = 2
+    rows = rows_per_seq * len(vl) - 1
+    x = inputs.normal_f32((rows, cols), 58 + cols, 0.0, 4.0)
+    got = ko.softmax_host(x, valid_len=vl, rows_per_seq=rows_per_seq, policy=policy)
+    assert_softmax_close(got, oracle.softmax(x, valid_len=vl, rows_per_seq=rows_per_seq))
+    assert np.all(got[4:6, 5:] == 0.0) and np.all(got[2:4, 1:] == 0.0)
 
 
 def test_softmax_properties(ko):
@@ -119,6 +132,10 @@ def test_softmax_errors(ko):
         ko.softmax(buf, buf, 1, 4096, policy=1)  # WARP policy holds at most 2048 columns
     assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert "WARP" in str(e.value)
+    big = ko.DeviceBuffer(131072 * 4)
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(big, big, 1, 131072, policy=2)  # BLOCK policy holds at most 98304 columns
+    assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE and "BLOCK" in str(e.value)
 
 
 def test_softmax_full_size_cfg1_properties(ko):
