@@ -338,6 +338,27 @@ __device__ __forceinline__ int swz(int row) {
     else return row & 7;
 }
 
+// B fragment of a 32x32x16 MFMA out of a row-major [k][BN] LDS tile (16-byte chunks swizzled with k & 3, see the
+// store): columns n0 .. n0+31, rows k0 .. k0+7 for this lane's half of the K step.  ds_read_b64_tr_b16 works on
+// groups of 16 lanes: lane i of a group supplies the address of four consecutive 16-bit values (here: row
+// k + i / 4, columns 4 * (i % 4) .. + 3 of the group's 16 columns) and receives, of the 16 x 4 values the group
+// read, column i of rows 0..3 - i.e. the four k values of its own column n0 + i.  Two reads give the eight
+// consecutive k that the MFMA wants per lane.
+template <int BN>
+__device__ __forceinline__ u32x4 read_b_transposed(const u32x4 *sb, int k0, int n0, int lane) {
+    typedef short short4v __attribute__((ext_vector_type(4)));
+    typedef short short8v __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) short4v *lds_ptr;
+    constexpr int NCH = BN / 8;
+    const int i = lane & 15, g = (lane >> 4) & 1;
+    const int kq = i >> 2;  // row within the four rows of one read (k0 is a multiple of 4: (k0 + kq) & 3 == kq)
+    const int chunk = ((n0 + g * 16 + 4 * (i & 3)) >> 3) ^ (kq << 2);
+    const char *base = reinterpret_cast<const char *>(sb) + ((k0 + kq) * NCH + chunk) * 16 + (i & 1) * 8;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base));
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * NCH * 16));
+    return __builtin_bit_cast(u32x4, static_cast<short8v>(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7)));
+}
+
 template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
 __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N, REG_STAGES = T::REG_STAGES;
@@ -457,19 +478,14 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
                 sb[row * kChunks + (c ^ swz<SWIZZLE>(row))] = rb[S][i];
             }
         } else {
-            uint16_t *sb16 = reinterpret_cast<uint16_t *>(sb);
+            // Row-major B stays row-major in LDS ([k][n], 16-byte chunks of 8 consecutive n); the chunk index is
+            // swizzled with k & 3 so that the four k rows one transposing read touches lie in different banks.
 #pragma unroll
             for (int i = 0; i < B_ITERS; ++i) {
                 const int idx = tid + i * THREADS;
                 constexpr int NCH = BN / 8;
                 const int kr = idx / NCH, c = idx % NCH;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int n = c * 8 + e;
-                    const uint16_t h = static_cast<uint16_t>(rb[S][i][e >> 1] >> ((e & 1) * 16));
-                    const int chunk = (kr >> 3) ^ swz<SWIZZLE>(n);
-                    sb16[(n * kChunks + chunk) * 8 + (kr & 7)] = h;
-                }
+                sb[kr * NCH + (c ^ ((kr & 3) << 2))] = rb[S][i];
             }
         }
     };
@@ -499,8 +515,12 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int row = wn * WTN + j * 32 + frow;
-                bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
+                if constexpr (!B_ROW_MAJOR) {
+                    const int row = wn * WTN + j * 32 + frow;
+                    bf[slot][j] = sb[row * kChunks + (chunk ^ swz<SWIZZLE>(row))];
+                } else {
+                    bf[slot][j] = read_b_transposed<BN>(sb, ks * 16 + fhalf * 8, wn * WTN + j * 32, lane);
+                }
             }
         };
         if constexpr (FRAG_DB) read_frags(0, 0);
