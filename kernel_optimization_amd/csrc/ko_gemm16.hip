@@ -739,6 +739,11 @@ __device__ __forceinline__ void lds_read16(u32x4 &dst, uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(IMM));
 }
 
+template <int IMM>
+__device__ __forceinline__ void lds_read_tr(u32x2 &dst, uint32_t addr) {
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(IMM));
+}
+
 // f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order
 template <class F, int... I>
 __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
@@ -755,7 +760,7 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
     else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
-template <class T, bool BF16>
+template <class T, bool BF16, bool B_ROW>
 __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -789,6 +794,17 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     const uint32_t lane_off =
         static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<1>(8 * wave + row_in)) << 3)) * 2u;
 
+    // Row-major B ([K][N]): the K tile of B is 64 rows of BN values and stays row-major in LDS.  A load
+    // instruction of a wave covers two rows (k = 2 * (wave + WAVES * J) + r, r = lane / 32); the 16-byte chunk a
+    // lane fetches is permuted with k & 3 (= 2 * (wave & 1) + r) so that the four rows of a transposing fragment
+    // read lie in different banks (see read_b_transposed).
+    static_assert(!B_ROW || (BN == 256 && WTN == 64), "");
+    uint32_t lane_off_b = lane_off;
+    if constexpr (B_ROW) {
+        const int r = lane >> 5;
+        lane_off_b = static_cast<uint32_t>(r * p.N + 8 * ((lane & 31) ^ ((2 * (wave & 1) + r) << 2))) * 2u;
+    }
+
     typedef const __attribute__((address_space(1))) void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
 
@@ -809,15 +825,18 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         int m0, n0;
         tile_origin(ld_t, m0, n0);
         cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
-        cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
+        if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(2 * wave) * p.N + n0);
+        else cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
     };
     set_cursor();
     const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
+    const int64_t group_stride_b = B_ROW ? static_cast<int64_t>(2 * WAVES) * p.N * 2 : group_stride;
+    const int64_t ktile_step_b = B_ROW ? static_cast<int64_t>(kBK) * p.N * 2 : kBK * 2;  // bytes from a K tile to the next
     auto advance_cursor = [&]() {
         if (ld_kt + 1 < KT) {
             ++ld_kt;
             cur_a += kBK * 2;
-            cur_b += kBK * 2;
+            cur_b += ktile_step_b;
         } else if (ld_t + 1 < my_tiles) {
             ld_kt = 0;
             ++ld_t;
@@ -833,7 +852,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         } else {
             constexpr int J = I - A_LOADS;
             __builtin_amdgcn_global_load_lds(
-                (gptr_t)(cur_b + J * group_stride + lane_off),
+                (gptr_t)(cur_b + J * group_stride_b + lane_off_b),
                 (lptr_t)(lds_bytes + 2 * A_BYTES + stage * B_BYTES + 1024 * (wave + WAVES * J)), 16, 0, 0);
             if constexpr (J == B_LOADS - 1) advance_cursor();
         }
@@ -847,12 +866,12 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
                                              (lptr_t)(dst_a + 1024 * (wave + WAVES * i)), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(cur_b + i * group_stride + lane_off),
+            __builtin_amdgcn_global_load_lds((gptr_t)(cur_b + i * group_stride_b + lane_off_b),
                                              (lptr_t)(dst_b + 1024 * (wave + WAVES * i)), 16, 0, 0);
         if (ld_kt + 1 < KT) {
             ++ld_kt;
             cur_a += kBK * 2;
-            cur_b += kBK * 2;
+            cur_b += ktile_step_b;
         } else if (ld_t + 1 < my_tiles) {
             ld_kt = 0;
             ++ld_t;
@@ -885,13 +904,33 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     clear_acc();
 
     u32x4 af[2][TM], bf[2][TN];
+    // row-major B: the halves of a B fragment as the two reads deliver them; bf is put together from them behind
+    // the wait (the compiler may need copies for that, and before the wait the registers hold nothing yet)
+    u32x2 b_lo[2][B_ROW ? TN : 1], b_hi[2][B_ROW ? TN : 1];
+    uint32_t off_br[B_ROW ? TN : 1];
+    if constexpr (B_ROW) {
+        const int i = lane & 15, g = (lane >> 4) & 1, kq = i >> 2;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int chunk = ((wn * WTN + j * 32 + g * 16 + 4 * (i & 3)) >> 3) ^ (kq << 2);
+            off_br[j] = lds_base + 2 * A_BYTES + (fhalf * 8 + kq) * (BN * 2) + chunk * 16 + (i & 1) * 8;
+        }
+    }
 
     // read number R (0 .. READS-1) of K step KSTEP out of stage S into fragment set SLOT
     auto read_one = [&](auto r_c, auto ks_c, auto slot_c, auto stage_c) {
         constexpr int R = decltype(r_c)::value, KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value,
                       S = decltype(stage_c)::value;
-        if constexpr (R < TM) lds_read16<S * A_BYTES + R * 4096>(af[SLOT][R], off_a[KSTEP]);
-        else lds_read16<S * B_BYTES + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[KSTEP]);
+        if constexpr (R < TM) {
+            lds_read16<S * A_BYTES + R * 4096>(af[SLOT][R], off_a[KSTEP]);
+        } else if constexpr (!B_ROW) {
+            lds_read16<S * B_BYTES + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[KSTEP]);
+        } else {
+            // two transposing reads: k .. k+3 and k+4 .. k+7 of this lane's column (rows of BN * 2 bytes)
+            constexpr int IMM = S * B_BYTES + KSTEP * 16 * BN * 2;
+            lds_read_tr<IMM>(b_lo[SLOT][R - TM], off_br[R - TM]);
+            lds_read_tr<IMM + 4 * BN * 2>(b_hi[SLOT][R - TM], off_br[R - TM]);
+        }
     };
 
     // MFMAs of one K step out of fragment set SLOT, with the reads reader(R) spread over the first ones
@@ -913,7 +952,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
 
     // all reads issued so far have landed; the fake operands keep later MFMAs behind this point
     auto wait_frags = [&](int slot) {
-        if constexpr (TM == 4 && TN == 2) {
+        if constexpr (B_ROW) {
+            static_assert(!B_ROW || (TM == 4 && TN == 2), "");
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
+                           "+v"(b_lo[slot][0]), "+v"(b_hi[slot][0]), "+v"(b_lo[slot][TN - 1]), "+v"(b_hi[slot][TN - 1]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bf[slot][j] = u32x4{b_lo[slot][j][0], b_lo[slot][j][1], b_hi[slot][j][0], b_hi[slot][j][1]};
+        } else if constexpr (TM == 4 && TN == 2) {
             asm volatile("s_waitcnt lgkmcnt(0)"
                          : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
                            "+v"(bf[slot][0]), "+v"(bf[slot][1]));
@@ -1027,12 +1074,12 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     }
 }
 
-template <class T, bool BF16>
+template <class T, bool BF16, bool B_ROW = false>
 int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
-    auto kernel = gemm16_pinned_kernel<T, BF16>;
+    auto kernel = gemm16_pinned_kernel<T, BF16, B_ROW>;
     static bool configured = false;
     if (!configured) {
         KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1113,13 +1160,14 @@ using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
 
-// The direct-to-LDS kernels need full 256x256x64 tiles and K-contiguous operands.
+// The direct-to-LDS kernels need full 256x256x64 tiles; the pinned one takes B in either layout, the
+// compiler-scheduled one K-contiguous (column-major) B only.
 template <class T, bool BF16, bool B_ROW_MAJOR, bool PINNED>
 int launch_direct(const Params &p, hipStream_t stream) {
-    if constexpr (B_ROW_MAJOR) {
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the direct-to-LDS variants need column-major B");
-    } else if constexpr (PINNED) {
-        return launch_pinned<T, BF16>(p, stream);
+    if constexpr (PINNED) {
+        return launch_pinned<T, BF16, B_ROW_MAJOR>(p, stream);
+    } else if constexpr (B_ROW_MAJOR) {
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this direct-to-LDS variant needs column-major B");
     } else {
         return launch_persistent<T, BF16>(p, stream);
     }
@@ -1135,11 +1183,10 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // Fewer: 128x128 tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
         if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+        if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % (2 * kBK) == 0)
+            return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
         if constexpr (!B_ROW_MAJOR) {
-            if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) {
-                if (p.K % (2 * kBK) == 0) return launch_pinned<TileBigSpread, BF16>(p, stream);
-                return launch_persistent<TileBig, BF16>(p, stream);
-            }
+            if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) return launch_persistent<TileBig, BF16>(p, stream);
         }
         return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
     }

@@ -99,8 +99,8 @@ def _to_f64(bits, bf16):
 @pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768), (512, 768, 192)])
 def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
-    if gemm16_variant >= 30 and not b_col_major:
-        pytest.skip("the direct-to-LDS kernels take column-major B")
+    if gemm16_variant == 30 and not b_col_major:
+        pytest.skip("the compiler-scheduled direct-to-LDS kernel takes column-major B")
     if gemm16_variant >= 30 and (m % 256 or n % 256 or k % 64):
         pytest.skip("the direct-to-LDS kernels take full tiles only")
     if gemm16_variant >= 50 and k % 128:
@@ -111,6 +111,28 @@ def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
     got = ko.gemm16_host(A, B, m, n, k, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR,
                          dtype=ko.BF16 if bf16 else ko.F16)
     assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("m,n,k", [(512, 768, 128), (2048, 1024, 256), (16384, 3072, 768), (4096, 4096, 200)])
+def test_gemm16_row_major_b_gives_the_same_bits(ko, m, n, k, bf16):
+    """B handed over as [K][N] (the reference's layout, tensor_core_gemm.h) or as its transpose [N][K]: the same
+    products are accumulated in the same order by the same instruction, so D must agree bit for bit - through the
+    register pipeline (small and ragged-K shapes) and through the pinned direct-to-LDS kernel (the big ones)."""
+    dt = ko.BF16 if bf16 else ko.F16
+    dA, dBc, dBr = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(n * k * 2)
+    ko.fill_uniform_16(dA, m * k, 81, dtype=dt)
+    ko.fill_uniform_16(dBc, n * k, 82, dtype=dt)
+    ko.synchronize()
+    b_col = dBc.download(np.uint16, (n, k))
+    dBr.upload(np.ascontiguousarray(b_col.T))
+    outs = []
+    for buf, layout in ((dBc, ko.COL_MAJOR), (dBr, ko.ROW_MAJOR)):
+        dD = ko.DeviceBuffer(m * n * 2)
+        ko.gemm16(m, n, k, dA, buf, dD, b_layout=layout, dtype=dt)
+        ko.synchronize()
+        outs.append(dD.download(np.uint16, (m, n)))
+    np.testing.assert_array_equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("m,n,k", [(8192, 4096, 192), (2048, 1024, 64), (16384, 3072, 768)])
