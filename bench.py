@@ -187,7 +187,9 @@ def bench_sgemm(cfg, steps, warmup, vendor):
     return res, None
 
 
-def bench_gemm16(cfg, steps, warmup, vendor):
+def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False):
+    """Configuration 4 (B column-major, both operands K-contiguous) or, with b_row_major, the same product with B
+    handed over as [K][N], the layout of the reference's own tensor-core kernel (tensor_core_gemm.h:178)."""
     c = inputs.CONFIGS[cfg]
     m, n, k = c["m"], c["n"], c["k"]
     flops = inputs.algorithmic_work(cfg)
@@ -198,8 +200,11 @@ def bench_gemm16(cfg, steps, warmup, vendor):
     for a, b in zip(As, Bs):
         ko.fill_uniform_16(a, m * k, inputs.tensor_seed(cfg, 0))
         ko.fill_uniform_16(b, k * n, inputs.tensor_seed(cfg, 1))
-    wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
-    res = dict(workload=c["name"], metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
+    layout = ko.ROW_MAJOR if b_row_major else ko.COL_MAJOR
+    wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets], b_layout=layout),
+                            steps, warmup)
+    name = c["name"].replace("gemm_f16_", "gemm_f16_rowmajorB_") if b_row_major else c["name"]
+    res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
                roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
                              frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=None),
@@ -208,8 +213,8 @@ def bench_gemm16(cfg, steps, warmup, vendor):
         us, na = ctypes.c_float(), ctypes.c_int()
         Vs = [ko.DeviceBuffer(m * n * 2) for _ in range(nsets)]
         tmp = Vs[0]
-        if vendor.kov_gemm16_sets(m, n, k, _ptr_array(As), _ptr_array(Bs), 1, _ptr_array(Vs), nsets, 0, 16, 20,
-                                  ctypes.byref(us), ctypes.byref(na)) == 0:
+        if vendor.kov_gemm16_sets(m, n, k, _ptr_array(As), _ptr_array(Bs), 0 if b_row_major else 1, _ptr_array(Vs), nsets,
+                                  0, 16, 20, ctypes.byref(us), ctypes.byref(na)) == 0:
             res["hipblaslt_tflops"] = flops / us.value / 1e6
             res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
             ref = tmp.download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
@@ -445,6 +450,9 @@ def main():
             res = bench_long_rows(op, rows, cols, policy, args.steps, args.warmup)
             res["steps"], res["warmup"] = args.steps, args.warmup
             others.append(res)
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, b_row_major=True)
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
