@@ -41,7 +41,10 @@ typedef enum ko_status {
  *         (SoftMaxBlockImpl softmax.h:62-113, LayerNormBlockImpl layernorm.h:204-252)
  * BLOCK_NOCACHE = row per workgroup, row re-read from global memory
  *         (SoftMaxBlockNoCacheImpl softmax.h:116-166, LayerNormBlockNoCacheImpl layernorm.h:254-300)
- * AUTO  = chosen from the row length. */
+ * AUTO  = chosen from the row length: the first of the three that holds the row.
+ * Longest rows: WARP 2048 fp32 / 4096 16-bit columns; BLOCK 98304 columns for softmax, 81920 for
+ * LayerNorm; BLOCK_NOCACHE any length.  A policy asked for explicitly on a longer row returns
+ * KO_ERR_UNSUPPORTED_SHAPE. */
 typedef enum ko_policy {
     KO_POLICY_AUTO = 0,
     KO_POLICY_WARP = 1,
