@@ -335,7 +335,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_kernel(
                 const int64_t off = static_cast<int64_t>(m) * N + n;
                 float v = alpha * acc[i][j][r];
                 if (use_c) v += beta * p.C[off];
-                p.D[off] = v;
+                __builtin_nontemporal_store(v, &p.D[off]);
             }
         }
     }
