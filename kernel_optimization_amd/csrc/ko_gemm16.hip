@@ -353,7 +353,7 @@ __device__ __forceinline__ u32x4 read_b_transposed(const u32x4 *sb, int k0, int 
     constexpr int NCH = BN / 8;
     const int i = lane & 15, g = (lane >> 4) & 1;
     const int kq = i >> 2;  // row within the four rows of one read (k0 is a multiple of 4: (k0 + kq) & 3 == kq)
-    const int chunk = ((n0 + g * 16 + 4 * (i & 3)) >> 3) ^ (kq << 2);
+    const int chunk = ((n0 + g * 16 + 4 * (i & 3)) >> 3) ^ ((kq << 2) & (NCH - 1));
     const char *base = reinterpret_cast<const char *>(sb) + ((k0 + kq) * NCH + chunk) * 16 + (i & 1) * 8;
     const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base));
     const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * NCH * 16));
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
                 const int idx = tid + i * THREADS;
                 constexpr int NCH = BN / 8;
                 const int kr = idx / NCH, c = idx % NCH;
-                sb[kr * NCH + (c ^ ((kr & 3) << 2))] = rb[S][i];
+                sb[kr * NCH + (c ^ (((kr & 3) << 2) & (NCH - 1)))] = rb[S][i];  // the swizzle stays inside the row
             }
         }
     };
@@ -1157,6 +1157,8 @@ int launch(Params p, hipStream_t stream) {
 
 using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 128x64
 using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
+using TileSmallN = Tiling<128, 64, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x32
+using TileTiny = Tiling<64, 64, 2, 2, 2, true, 1>;      // 4 waves, wave tile 32x32
 
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
@@ -1181,11 +1183,23 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // Enough 256x256 tiles to fill the chip: the big tiling - as a persistent direct-to-LDS kernel
         // when the tiles are full and both operands are K-contiguous (the pinned one when K is a
         // multiple of 128), else as the register pipeline.
-        // Fewer: 128x128 tiles so that the grid still covers the compute units.
+        // Fewer: smaller tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
-        if (big_tiles < compute_units()) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
-        if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % (2 * kBK) == 0)
+        // The pinned kernel is so much faster per tile that it wins from half a chip's worth of full tiles on
+        // (192 tiles on 256 CUs: 16384 x 768 x 3072 takes 69 us against 103 us with 128 x 128 tiles; at 96 tiles
+        // the two are level).
+        if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K % (2 * kBK) == 0)
             return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
+        if (big_tiles < compute_units()) {
+            // Fewer big tiles than that: the largest of the small tilings that still gives every compute unit one
+            // and a half workgroups (two are resident at a time), else the smallest (1024^3: 64 x 64 tiles 8.8 us,
+            // 128 x 128 tiles 16.3 us).
+            const int64_t want = static_cast<int64_t>(compute_units()) * 3 / 2;
+            const int64_t tm128 = (p.M + 127) / 128, tn128 = (p.N + 127) / 128, tn64 = (p.N + 63) / 64;
+            if (tm128 * tn128 >= want) return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+            if (tm128 * tn64 >= want) return launch<TileSmallN, BF16, B_ROW_MAJOR>(p, stream);
+            return launch<TileTiny, BF16, B_ROW_MAJOR>(p, stream);
+        }
         if constexpr (!B_ROW_MAJOR) {
             if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % kBK == 0) return launch_persistent<TileBig, BF16>(p, stream);
         }
@@ -1196,6 +1210,8 @@ int launch_variant(const Params &p, hipStream_t stream) {
         case 6: return launch<Tiling<256, 256, 2, 4, 1, true, 0>, BF16, B_ROW_MAJOR>(p, stream);
         case 9: return launch<TileBig, BF16, B_ROW_MAJOR>(p, stream);
         case 10: return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+        case 11: return launch<TileTiny, BF16, B_ROW_MAJOR>(p, stream);
+        case 12: return launch<TileSmallN, BF16, B_ROW_MAJOR>(p, stream);
         case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);

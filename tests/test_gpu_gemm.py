@@ -9,7 +9,7 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19]
-GEMM16_VARIANTS = [0, 3, 6, 9, 10, 30, 50, 52, 53]
+GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 30, 50, 52, 53]
 
 
 @pytest.fixture
@@ -179,6 +179,22 @@ def test_gemm16_default_path_big(ko, bf16, k):
     idx = np.sort(np.random.default_rng(4).choice(m, 64, replace=False))
     _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, bf16=bf16)
     assert_gemm16_close(_to_f64(got[idx], bf16), ref64, ap, k, bf16=bf16)
+
+
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n", [(4096, 3072), (2048, 4096), (3072, 2816), (2048, 2048), (1024, 1536)])
+def test_gemm16_default_path_partly_filled_chip(ko, m, n, b_col_major):
+    """Between half a chip's and a chip's worth of 256 x 256 tiles (192, 128 and 132 of them): the default dispatch
+    still takes the pinned kernel, with fewer workgroups than compute units and, for 132 tiles, a grid that is not a
+    multiple of eight.  Fewer still (64 and 24 big tiles): the 128 x 64 and 64 x 64 tilings of the register
+    pipeline.  Sampled rows against the oracle, both layouts of B."""
+    k = 256
+    A = _bits16((m, k), 35, False)
+    B = _bits16((n, k) if b_col_major else (k, n), 36, False)
+    got = ko.gemm16_host(A, B, m, n, k, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
+    idx = np.sort(np.random.default_rng(5).choice(m, 64, replace=False))
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, b_col_major=b_col_major)
+    assert_gemm16_close(_to_f64(got[idx], False), ref64, ap, k)
 
 
 def test_gemm16_odd_n(ko):
