@@ -380,10 +380,11 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     hipStream_t s = as_stream(stream);
     int variant = tuning("sgemm.variant");
     if (variant <= 0) {
-        // Few tiles (fewer than two 128 x 128 tiles per compute unit): 64 x 64 tiles with K split four
-        // ways inside the workgroup; otherwise 128 x 128 tiles with K split two ways.
+        // Few tiles (fewer 128 x 128 tiles than compute units): 64 x 64 tiles with K split four ways inside
+        // the workgroup; otherwise 128 x 128 tiles with K split two ways (2048^3, one tile per compute unit:
+        // 136 us against 148 us).
         const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
-        variant = t128 >= 2 * compute_units() ? 16 : 13;
+        variant = t128 >= compute_units() ? 16 : 13;
     }
     switch (variant) {
         case 1: return launch<64, 64, 32, 2, 2, 1>(p, s);
