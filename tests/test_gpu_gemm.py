@@ -8,7 +8,7 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 
 pytestmark = pytest.mark.gpu
 
-SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19]
+SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 21]
 GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 30, 50, 52, 53]
 
 
