@@ -182,12 +182,13 @@ def test_gemm16_default_path_big(ko, bf16, k):
 
 
 @pytest.mark.parametrize("b_col_major", [True, False])
-@pytest.mark.parametrize("m,n", [(4096, 3072), (2048, 4096), (3072, 2816), (2048, 2048), (1024, 1536)])
+@pytest.mark.parametrize("m,n", [(4096, 3072), (2048, 4096), (3072, 2816), (2048, 2048), (1024, 1536), (4352, 4096)])
 def test_gemm16_default_path_partly_filled_chip(ko, m, n, b_col_major):
     """Between half a chip's and a chip's worth of 256 x 256 tiles (192, 128 and 132 of them): the default dispatch
     still takes the pinned kernel, with fewer workgroups than compute units and, for 132 tiles, a grid that is not a
     multiple of eight.  Fewer still (64 and 24 big tiles): the 128 x 64 and 64 x 64 tilings of the register
-    pipeline.  Sampled rows against the oracle, both layouts of B."""
+    pipeline.  272 tiles: sixteen workgroups walk two tiles, the others one.  Sampled rows against the oracle, both
+    layouts of B."""
     k = 256
     A = _bits16((m, k), 35, False)
     B = _bits16((n, k) if b_col_major else (k, n), 36, False)
