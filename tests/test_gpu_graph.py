@@ -1,0 +1,103 @@
+"""The operators are plain kernel launches on the caller's stream, so a caller can capture them into a HIP graph
+(the reference's drivers launch on one non-blocking stream as well, softmax/main.cu:28-29).  This test captures a
+softmax -> LayerNorm -> 16-bit GEMM -> SGEMM -> 16-bit GEMM (persistent kernel) sequence with the HIP runtime that libko.so itself is linked against,
+replays the graph several times with eager work and synchronisations in between, and compares every replay bit
+for bit with the eager results.  One eager pass comes first: the library's one-time set-up (device properties,
+kernel attributes) is not stream work and belongs in front of a capture."""
+import ctypes
+import re
+
+import numpy as np
+import pytest
+
+from kernel_optimization_amd import inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _hip_runtime():
+    """The libamdhip64 this process already has loaded (through libko.so)."""
+    with open("/proc/self/maps") as f:
+        paths = sorted(set(re.findall(r"(/\S*libamdhip64\.so[\w.]*)", f.read())))
+    assert paths, "libko.so is loaded, so the HIP runtime must be mapped"
+    hip = ctypes.CDLL(paths[0])
+    vp = ctypes.c_void_p
+    hip.hipStreamBeginCapture.argtypes = [vp, ctypes.c_int]
+    hip.hipStreamEndCapture.argtypes = [vp, ctypes.POINTER(vp)]
+    hip.hipGraphInstantiate.argtypes = [ctypes.POINTER(vp), vp, vp, vp, ctypes.c_size_t]
+    hip.hipGraphLaunch.argtypes = [vp, vp]
+    hip.hipGraphExecDestroy.argtypes = [vp]
+    hip.hipGraphDestroy.argtypes = [vp]
+    return hip
+
+
+def test_operators_replay_from_a_hip_graph(ko):
+    ko.lib()
+    hip = _hip_runtime()
+    stream = ko.Stream()
+    rows, cols = 1024, 768
+    m, n, k = 512, 768, 256
+    x = inputs.normal_f32((rows, cols), 501, 0.0, 4.0)
+    g = inputs.normal_f32((cols,), 502, 1.0, 0.1)
+    vl = np.array([700, 13, 768, 0], np.int32)
+    dx, dg, dvl = ko.DeviceBuffer.from_numpy(x), ko.DeviceBuffer.from_numpy(g), ko.DeviceBuffer.from_numpy(vl)
+    ds, dl = ko.DeviceBuffer(rows * cols * 4), ko.DeviceBuffer(rows * cols * 4)
+    dmean, drstd = ko.DeviceBuffer(rows * 4), ko.DeviceBuffer(rows * 4)
+    a16, b16, d16 = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(m * n * 2)
+    a32, b32, d32 = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
+    m2, n2, k2 = 4096, 2048, 256  # 128 tiles of 256 x 256: the persistent direct-to-LDS kernel
+    a2, b2, d2 = ko.DeviceBuffer(m2 * k2 * 2), ko.DeviceBuffer(n2 * k2 * 2), ko.DeviceBuffer(m2 * n2 * 2)
+    ko.fill_uniform_16(a2, m2 * k2, 507)
+    ko.fill_uniform_16(b2, n2 * k2, 508)
+    ko.fill_uniform_16(a16, m * k, 503)
+    ko.fill_uniform_16(b16, n * k, 504)
+    ko.fill_uniform_f32(a32, m * k, 505)
+    ko.fill_uniform_f32(b32, k * n, 506)
+    ko.synchronize()
+
+    def chain():
+        ko.softmax(dx, ds, rows, cols, dvl, rows // 4, stream=stream)
+        ko.layernorm(ds, dl, rows, cols, dmean, drstd, dg, None, 1e-5, False, stream=stream)
+        ko.gemm16(m, n, k, a16, b16, d16, stream=stream)
+        ko.sgemm(m, n, k, a32, b32, d32, stream=stream)
+        ko.gemm16(m2, n2, k2, a2, b2, d2, stream=stream)
+
+    def outputs():
+        return (dl.download(np.uint32, (rows, cols)), dmean.download(np.uint32, (rows,)),
+                d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)))
+
+    def clear():
+        for buf, nbytes in ((ds, rows * cols * 4), (dl, rows * cols * 4), (dmean, rows * 4), (d16, m * n * 2), (d32, m * n * 4),
+                            (d2, m2 * n2 * 2)):
+            buf.upload(np.zeros(nbytes, np.uint8))
+
+    chain()
+    stream.synchronize()
+    want = outputs()
+    assert want[0].any() and want[2].any() and want[3].any()
+
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 0) == 0  # hipStreamCaptureModeGlobal
+    try:
+        chain()
+    finally:
+        rc = hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
+    try:
+        for replay in range(3):
+            clear()
+            ko.synchronize()
+            assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+            stream.synchronize()
+            got = outputs()
+            for w, gt in zip(want, got):
+                np.testing.assert_array_equal(gt, w, err_msg="replay %d" % replay)
+            # eager work between replays, on the same stream and on the default one
+            ko.softmax(dx, ds, rows, cols, None, 0, stream=stream)
+            ko.copy_f32(dx, dl, rows * cols)
+            stream.synchronize()
+            ko.synchronize()
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
