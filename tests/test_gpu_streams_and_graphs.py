@@ -101,3 +101,54 @@ def test_operators_replay_from_a_hip_graph(ko):
     finally:
         hip.hipGraphExecDestroy(graph_exec)
         hip.hipGraphDestroy(graph)
+
+
+def test_operators_from_two_threads_on_two_streams(ko):
+    """Thread-compatible entry points: two host threads, each with its own stream and buffers, run the row
+    operators and the GEMMs at the same time; every result equals the single-threaded one bit for bit."""
+    import threading
+    ko.lib()
+    rows, cols = 2048, 512
+    m, n, k = 512, 512, 128
+
+    def work(seed, stream, out):
+        x = inputs.normal_f32((rows, cols), seed, 0.0, 4.0)
+        dx, dy, dl = ko.DeviceBuffer.from_numpy(x), ko.DeviceBuffer(rows * cols * 4), ko.DeviceBuffer(rows * cols * 4)
+        a, b, d = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
+        a16, b16, d16 = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(m * n * 2)
+        ko.fill_uniform_f32(a, m * k, seed + 1, stream=stream)
+        ko.fill_uniform_f32(b, k * n, seed + 2, stream=stream)
+        ko.fill_uniform_16(a16, m * k, seed + 3, stream=stream)
+        ko.fill_uniform_16(b16, n * k, seed + 4, stream=stream)
+        for _ in range(20):
+            ko.softmax(dx, dy, rows, cols, stream=stream)
+            ko.layernorm(dy, dl, rows, cols, stream=stream)
+            ko.sgemm(m, n, k, a, b, d, stream=stream)
+            ko.gemm16(m, n, k, a16, b16, d16, stream=stream)
+        if stream is not None:
+            stream.synchronize()
+        else:
+            ko.synchronize()
+        out[seed] = (dy.download(np.uint32, (rows, cols)), dl.download(np.uint32, (rows, cols)),
+                     d.download(np.uint32, (m, n)), d16.download(np.uint16, (m, n)))
+
+    want = {}
+    for seed in (610, 620):
+        work(seed, None, want)
+    got, errors = {}, []
+
+    def guarded(seed):
+        try:
+            work(seed, ko.Stream(), got)
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise be lost
+            errors.append(e)
+
+    threads = [threading.Thread(target=guarded, args=(seed,)) for seed in (610, 620)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    assert not errors, errors
+    for seed in (610, 620):
+        for w, g in zip(want[seed], got[seed]):
+            np.testing.assert_array_equal(g, w)
