@@ -346,17 +346,25 @@ __device__ __forceinline__ float exp_nonpositive(float d) {
     return __builtin_ldexpf(e, static_cast<int>(n));
 }
 
-// exp(d) for d <= 0 where the result is rounded to a 16-bit storage type afterwards: one rounded product
-// and the hardware exponential (with the compiler's scaling for results below the normal range).  The
-// product's rounding costs |d| * log2(e) * 2^-24 relative, about 3.5e-6 at d = -40: far inside half an
-// ulp of binary16 (4.9e-4) or bfloat16 (3.9e-3).
+// exp(d) for d <= 0 where the result is rounded to bfloat16 afterwards (which keeps fp32's exponent range, so
+// results below 2^-126 matter): 2^(d log2(e) + 64) from the bare instruction, always in the normal range, times
+// 2^-64 by a multiplication, which produces subnormal results correctly.  The rounded fused multiply-add costs
+// 2^-18 absolute in the exponent, 2.6e-6 relative in the result: far inside half an ulp of bfloat16 (3.9e-3).
 __device__ __forceinline__ float exp_nonpositive_fast(float d) {
-    return __builtin_exp2f(fmaxf(d, -150.0f) * 0x1.715476p+0f);
+    return __builtin_amdgcn_exp2f(__builtin_fmaf(fmaxf(d, -150.0f), 0x1.715476p+0f, 64.0f)) * 0x1p-64f;
+}
+
+// The same for binary16 storage: everything below 2^-25 rounds to zero there, so the exponent is clamped at
+// -126 and the bare instruction is used (its results below the normal range would need the compiler's
+// rescaling: a compare, two selects and an ldexp per value, a third of this kernel's vector ALU work).
+__device__ __forceinline__ float exp_nonpositive_f16(float d) {
+    return __builtin_amdgcn_exp2f(fmaxf(d * 0x1.715476p+0f, -126.0f));
 }
 
 template <int IO>
 __device__ __forceinline__ float exp_for_storage(float d) {
     if constexpr (IO == IO_F32) return exp_nonpositive(d);
+    else if constexpr (IO == IO_F16) return exp_nonpositive_f16(d);
     else return exp_nonpositive_fast(d);
 }
 
