@@ -92,36 +92,36 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     // gamma/beta of this lane's columns stay in registers across rows.  They are fetched behind the first
     // row's loads: memory returns in order, so loads issued ahead of the row would stand between the row
     // and the statistics, which do not need them.
-    float g[VPL][E], b[VPL][E];
+    // They are kept as loaded (16-bit storage: half the registers of converted values, which decides between
+    // four and six resident waves per SIMD at 768 columns) and converted where they are used.
+    typename Io<IO>::raw g_raw[VPL], b_raw[VPL];
     auto load_affine = [&]() {
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-#pragma unroll
-            for (int e = 0; e < E; ++e) {
-                g[k][e] = 1.0f;
-                b[k][e] = 0.0f;
-            }
+            g_raw[k] = typename Io<IO>::raw{};
+            b_raw[k] = typename Io<IO>::raw{};
             if (FULL || j < nvec) {
-                if (gamma) Io<IO>::template load<false>(gamma + E * j, g[k]);
-                if (beta) Io<IO>::template load<false>(beta + E * j, b[k]);
+                if (gamma) g_raw[k] = Io<IO>::template load_raw<false>(gamma + E * j);
+                if (beta) b_raw[k] = Io<IO>::template load_raw<false>(beta + E * j);
             }
         }
     };
 
+    // All loads of a row go out before any is converted: a conversion inside the branch that holds its load
+    // makes the compiler wait for that load before the next one is issued.
     auto load_rows = [&](float (&v)[VPL][E], int64_t row) {
         const bool row_ok = row < rows;
         const typename Io<IO>::elem *src = in + row * cols;
+        typename Io<IO>::raw loaded[VPL];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            if (row_ok && (FULL || j < nvec)) {
-                Io<IO>::template load<NT>(src + E * j, v[k]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
-            }
+            loaded[k] = typename Io<IO>::raw{};  // all-zero bits are 0.0 in every storage type
+            if (row_ok && (FULL || j < nvec)) loaded[k] = Io<IO>::template load_raw<NT>(src + E * j);
         }
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) Io<IO>::unpack(loaded[k], v[k]);
     };
 
     auto finish_rows = [&](float (&v)[VPL][E], int64_t row) {
@@ -149,9 +149,26 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
             if (row_ok && (FULL || j < nvec)) {
-                float y[E];
+                float y[E], g[E], b[E];
+                if constexpr (E == 8) {
+                    // the conversions stay here, per row: hoisted out of the row loop they would occupy the
+                    // registers that keeping the vectors unconverted is meant to save
+                    asm volatile("" : "+v"(g_raw[k]), "+v"(b_raw[k]));
+                }
+                if (gamma) {
+                    Io<IO>::unpack(g_raw[k], g);
+                } else {
 #pragma unroll
-                for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[k][e], b[k][e]);
+                    for (int e = 0; e < E; ++e) g[e] = 1.0f;
+                }
+                if (beta) {
+                    Io<IO>::unpack(b_raw[k], b);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) b[e] = 0.0f;
+                }
+#pragma unroll
+                for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[e], b[e]);
                 Io<IO>::template store<NT>(dst + E * j, y);
             }
         }
@@ -263,15 +280,16 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
         asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
         float v[VPL][E];
+        {
+            typename Io<IO>::raw loaded[VPL];  // all loads first, conversions afterwards
 #pragma unroll
-        for (int k = 0; k < VPL; ++k) {
-            const int j = threadIdx.x + k * THREADS;
-            if (j < nvec) {
-                Io<IO>::template load<true>(at_bytes(src, first + k * kStep), v[k]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < E; ++e) v[k][e] = 0.0f;
+            for (int k = 0; k < VPL; ++k) {
+                const int j = threadIdx.x + k * THREADS;
+                loaded[k] = typename Io<IO>::raw{};
+                if (j < nvec) loaded[k] = Io<IO>::template load_raw<true>(at_bytes(src, first + k * kStep));
             }
+#pragma unroll
+            for (int k = 0; k < VPL; ++k) Io<IO>::unpack(loaded[k], v[k]);
         }
         const float x0 = Io<IO>::scalar(src);
         wave::Welford w{0.0f, 0.0f, 0.0f};
@@ -341,9 +359,14 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
         constexpr int UNROLL = 4;
         for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
             float x[UNROLL][E];
+            typename Io<IO>::raw loaded[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) Io<IO>::template load<false>(src + E * (j0 + u * THREADS), x[u]);
+            for (int u = 0; u < UNROLL; ++u) {
+                loaded[u] = typename Io<IO>::raw{};
+                if (j0 + u * THREADS < nvec) loaded[u] = Io<IO>::template load_raw<false>(src + E * (j0 + u * THREADS));
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (j0 + u * THREADS >= nvec) break;
@@ -370,9 +393,14 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
         for (int t = trips - 1; t >= 0; --t) {
             const int j0 = threadIdx.x + t * (THREADS * UNROLL);
             float x[UNROLL][E];
+            typename Io<IO>::raw loaded[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) Io<IO>::template load<true>(src + E * (j0 + u * THREADS), x[u]);
+            for (int u = 0; u < UNROLL; ++u) {
+                loaded[u] = typename Io<IO>::raw{};
+                if (j0 + u * THREADS < nvec) loaded[u] = Io<IO>::template load_raw<true>(src + E * (j0 + u * THREADS));
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const int j = j0 + u * THREADS;

@@ -34,24 +34,25 @@ namespace {
 
 constexpr float kMaskValue = -10000.0f;
 
-// Loads vector j (columns E*j .. E*j+E-1) of a row whose first `vlen` columns are valid.
+// A row vector is fetched in two steps so that a thread can issue all of its loads before it looks at any of
+// them: unpacking or masking inside the branch that holds a load makes the compiler wait for that load before
+// the next one goes out.
+// fetch: the 16 bytes at `p` (vector j of the row) if the vector holds valid columns, else nothing is loaded.
 template <int IO, bool MASKED, bool NT>
-__device__ __forceinline__ void load_row_vec(const typename Io<IO>::elem *row, int j, int vlen,
-                                             float (&v)[Io<IO>::E]) {
+__device__ __forceinline__ typename Io<IO>::raw fetch_row_vec(const typename Io<IO>::elem *p, int j, int vlen) {
+    typename Io<IO>::raw r{};
+    if (!MASKED || Io<IO>::E * j < vlen) r = Io<IO>::template load_raw<NT>(p);
+    return r;
+}
+// finish: converted values of vector j, with the columns from `vlen` on replaced by the mask value.
+template <int IO, bool MASKED>
+__device__ __forceinline__ void finish_row_vec(typename Io<IO>::raw r, int j, int vlen, float (&v)[Io<IO>::E]) {
     constexpr int E = Io<IO>::E;
-    const int c = E * j;
-    if constexpr (!MASKED) {
-        Io<IO>::template load<NT>(row + c, v);
-    } else {
-        if (c < vlen) {
-            Io<IO>::template load<NT>(row + c, v);
+    Io<IO>::unpack(r, v);
+    if constexpr (MASKED) {
 #pragma unroll
-            for (int e = 1; e < E; ++e)
-                if (c + e >= vlen) v[e] = kMaskValue;
-        } else {
-#pragma unroll
-            for (int e = 0; e < E; ++e) v[e] = kMaskValue;
-        }
+        for (int e = 0; e < E; ++e)
+            if (E * j + e >= vlen) v[e] = kMaskValue;
     }
 }
 
@@ -96,13 +97,21 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
             if (row_ok) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
         }
 
+        // All of the lane's loads go out first and are unpacked and masked afterwards: with the unpacking inside
+        // the same branch as its load, each load would be waited for before the next one is issued.
+        typename Io<IO>::raw loaded[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = l + k * LPR;
+            loaded[k] = typename Io<IO>::raw{};
+            if (row_ok && j < nvec) loaded[k] = fetch_row_vec<IO, MASKED, NT>(src + E * j, j, vlen);
+        }
         float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
-            if (row_ok && j < nvec) {
-                load_row_vec<IO, MASKED, NT>(src, j, vlen, v[k]);
-            } else {
+            finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
+            if (!(row_ok && j < nvec)) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
             }
@@ -201,13 +210,19 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
         const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+        typename Io<IO>::raw loaded[VPL];
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            loaded[k] = typename Io<IO>::raw{};
+            if (j < nvec) loaded[k] = fetch_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), j, vlen);
+        }
         float v[VPL][E];
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
-            if (j < nvec) {
-                load_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), 0, vlen - E * j, v[k]);
-            } else {
+            finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
+            if (j >= nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
             }
@@ -276,9 +291,15 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
         constexpr int UNROLL = 4;
         for (int j0 = threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
             float x[UNROLL][E];
+            typename Io<IO>::raw loaded[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, false>(src, j0 + u * THREADS, vlen, x[u]);
+            for (int u = 0; u < UNROLL; ++u) {
+                const int j = j0 + u * THREADS;
+                loaded[u] = typename Io<IO>::raw{};
+                if (j < nvec) loaded[u] = fetch_row_vec<IO, MASKED, false>(src + E * j, j, vlen);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) finish_row_vec<IO, MASKED>(loaded[u], j0 + u * THREADS, vlen, x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (j0 + u * THREADS >= nvec) break;
@@ -298,9 +319,15 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
         for (int t = 0; t < trips; ++t) {
             const int j0 = threadIdx.x + (trips - 1 - t) * (THREADS * UNROLL);
             float x[UNROLL][E];
+            typename Io<IO>::raw loaded[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u)
-                if (j0 + u * THREADS < nvec) load_row_vec<IO, MASKED, true>(src, j0 + u * THREADS, vlen, x[u]);
+            for (int u = 0; u < UNROLL; ++u) {
+                const int j = j0 + u * THREADS;
+                loaded[u] = typename Io<IO>::raw{};
+                if (j < nvec) loaded[u] = fetch_row_vec<IO, MASKED, true>(src + E * j, j, vlen);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) finish_row_vec<IO, MASKED>(loaded[u], j0 + u * THREADS, vlen, x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const int j = j0 + u * THREADS;
