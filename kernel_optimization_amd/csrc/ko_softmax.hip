@@ -94,7 +94,22 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
         const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) {
-            if (row_ok) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+            // The rows of a wavefront are consecutive and start at a wave-uniform row: their sequence lengths are
+            // fetched with wave-uniform addresses (scalar loads through the constant cache, which the 6144 rows
+            // of a sequence keep hitting) instead of one vector load per lane, whose latency would stand in front
+            // of the row loads.
+            const uint64_t r0 = static_cast<uint64_t>(row0);
+            const int64_t first_row = static_cast<int64_t>(
+                (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0 >> 32))) << 32) |
+                __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0)));
+#pragma unroll
+            for (int r = 0; r < RPW; ++r) {
+                const int64_t rr = first_row + r;
+                if (rr < rows) {
+                    const int len = clamp_len(valid_len[rr / rows_per_seq], cols);
+                    if (sub == r) vlen = len;
+                }
+            }
         }
 
         // All of the lane's loads go out first and are unpacked and masked afterwards: with the unpacking inside
