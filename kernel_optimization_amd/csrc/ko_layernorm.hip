@@ -68,7 +68,11 @@ struct Args {
 // A wavefront takes one row group (64 / LPR rows, one per lane group) per trip.
 // FULL: cols == LPR * VPL vectors, every lane folds the same number of elements (no per-vector bounds
 // checks, and the lanes merge with the equal-count form).
-template <int IO, int LPR, int VPL, bool FULL>
+// AFFINE: gamma or beta (or both) given.  Their loads are then unconditional - a missing one is pointed at the
+// other and its values ignored - because loads inside `if (gamma)` branches leave the compiler unable to count
+// the loads in flight: it then makes the statistics wait for all but the last two of them, gamma and beta
+// included, instead of for the row alone.
+template <int IO, int LPR, int VPL, bool FULL, bool AFFINE>
 __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<IO>::elem *in,
                                                              typename Io<IO>::elem *out,
                                                              float *__restrict__ mean_out,
@@ -95,15 +99,18 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     // They are kept as loaded (16-bit storage: half the registers of converted values, which decides between
     // four and six resident waves per SIMD at 768 columns) and converted where they are used.
     typename Io<IO>::raw g_raw[VPL], b_raw[VPL];
+    const typename Io<IO>::elem *g_from = gamma ? gamma : beta, *b_from = beta ? beta : gamma;
     auto load_affine = [&]() {
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
             g_raw[k] = typename Io<IO>::raw{};
             b_raw[k] = typename Io<IO>::raw{};
-            if (FULL || j < nvec) {
-                if (gamma) g_raw[k] = Io<IO>::template load_raw<false>(gamma + E * j);
-                if (beta) b_raw[k] = Io<IO>::template load_raw<false>(beta + E * j);
+            if constexpr (AFFINE) {
+                if (FULL || j < nvec) {
+                    g_raw[k] = Io<IO>::template load_raw<false>(g_from + E * j);
+                    b_raw[k] = Io<IO>::template load_raw<false>(b_from + E * j);
+                }
             }
         }
     };
@@ -155,13 +162,13 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
                     // registers that keeping the vectors unconverted is meant to save
                     asm volatile("" : "+v"(g_raw[k]), "+v"(b_raw[k]));
                 }
-                if (gamma) {
+                if (AFFINE && gamma) {
                     Io<IO>::unpack(g_raw[k], g);
                 } else {
 #pragma unroll
                     for (int e = 0; e < E; ++e) g[e] = 1.0f;
                 }
-                if (beta) {
+                if (AFFINE && beta) {
                     Io<IO>::unpack(b_raw[k], b);
                 } else {
 #pragma unroll
@@ -178,14 +185,16 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         }
     };
 
-    bool have_affine = false;
-    for (int64_t row0 = wave * RPW; row0 < rows; row0 += stride) {
-        float v[VPL][E];
+    // The first row group stands outside the loop: its loads and those of gamma and beta are then one
+    // straight-line sequence, and the compiler can count which of them the statistics have to wait for.
+    int64_t row0 = wave * RPW;
+    if (row0 >= rows) return;
+    float v[VPL][E];
+    load_rows(v, row0 + sub);
+    load_affine();
+    finish_rows(v, row0 + sub);
+    for (row0 += stride; row0 < rows; row0 += stride) {
         load_rows(v, row0 + sub);
-        if (!have_affine) {
-            load_affine();
-            have_affine = true;
-        }
         finish_rows(v, row0 + sub);
     }
 }
@@ -434,8 +443,12 @@ int launch_wave_full(const Args<IO> &a) {
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    layernorm_wave_kernel<IO, LPR, VPL, FULL><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
-        a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
+    if (a.gamma || a.beta)
+        layernorm_wave_kernel<IO, LPR, VPL, FULL, true><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+            a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
+    else
+        layernorm_wave_kernel<IO, LPR, VPL, FULL, false><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+            a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
