@@ -225,21 +225,36 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
         const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
         if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
-        typename Io<IO>::raw loaded[VPL];
-#pragma unroll
-        for (int k = 0; k < VPL; ++k) {
-            const int j = threadIdx.x + k * THREADS;
-            loaded[k] = typename Io<IO>::raw{};
-            if (j < nvec) loaded[k] = fetch_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), j, vlen);
-        }
         float v[VPL][E];
+        if constexpr (IO == IO_F32 && !MASKED) {
+            // nothing to unpack or mask: the loaded registers are the values (the two-step form below costs ten
+            // registers more here, and with them the second resident workgroup at 32768 columns)
 #pragma unroll
-        for (int k = 0; k < VPL; ++k) {
-            const int j = threadIdx.x + k * THREADS;
-            finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
-            if (j >= nvec) {
+            for (int k = 0; k < VPL; ++k) {
+                const int j = threadIdx.x + k * THREADS;
+                if (j < nvec) {
+                    Io<IO>::template load<true>(at_bytes(src, first + k * kStep), v[k]);
+                } else {
 #pragma unroll
-                for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                    for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                }
+            }
+        } else {
+            typename Io<IO>::raw loaded[VPL];
+#pragma unroll
+            for (int k = 0; k < VPL; ++k) {
+                const int j = threadIdx.x + k * THREADS;
+                loaded[k] = typename Io<IO>::raw{};
+                if (j < nvec) loaded[k] = fetch_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), j, vlen);
+            }
+#pragma unroll
+            for (int k = 0; k < VPL; ++k) {
+                const int j = threadIdx.x + k * THREADS;
+                finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
+                if (j >= nvec) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                }
             }
         }
         float m = -FLT_MAX;
