@@ -547,17 +547,19 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
         constexpr int P = decltype(parity)::value;  // kt & 1
         constexpr int LOAD_SLOT = REG_STAGES == 2 ? P : 0;
         constexpr int STORE_SLOT = REG_STAGES == 2 ? (P ^ 1) : 0;
-        if (kt + REG_STAGES < KT) load_global(kt + REG_STAGES, std::integral_constant<int, LOAD_SLOT>{});
+        // Past the last K tile the loads and the LDS stores are not branched around but redirected to the last
+        // tile (fetched and stored once more, into the stage nobody reads any more): with loads under a branch
+        // the compiler cannot count the loads in flight and waits for all of them - the set issued one step
+        // ago included - before it reuses the registers of the older set.
+        load_global(kt + REG_STAGES < KT ? kt + REG_STAGES : KT - 1, std::integral_constant<int, LOAD_SLOT>{});
         compute_tile(P);
-        if (kt + 1 < KT) store_lds(P ^ 1, std::integral_constant<int, STORE_SLOT>{});
+        store_lds(P ^ 1, std::integral_constant<int, STORE_SLOT>{});
         lds_barrier();
     };
 
     load_global(0, std::integral_constant<int, 0>{});
     store_lds(0, std::integral_constant<int, 0>{});
-    if constexpr (REG_STAGES == 2) {
-        if (KT > 1) load_global(1, std::integral_constant<int, 1>{});
-    }
+    if constexpr (REG_STAGES == 2) load_global(KT > 1 ? 1 : 0, std::integral_constant<int, 1>{});
     lds_barrier();
     for (int kt = 0; kt < KT; kt += 2) {
         step(kt, std::integral_constant<int, 0>{});
