@@ -89,6 +89,29 @@ def test_masked_softmax_long_rows(ko, policy, cols):
     assert np.all(got[4:6, 5:] == 0.0) and np.all(got[2:4, 1:] == 0.0)
 
 
+@pytest.mark.parametrize("cols", [32, 64, 128, 256, 512])
+@pytest.mark.parametrize("rows_per_seq", [1, 3, 7])
+def test_masked_softmax_sequences_end_inside_a_wavefront(ko, cols, rows_per_seq):
+    """Short rows put 2 to 8 rows into one wavefront; with 1, 3 or 7 rows per sequence the rows of a wavefront
+    belong to different sequences, each with its own length (the kernel fetches the lengths of a wavefront's rows
+    with wave-uniform loads and hands each lane group its own)."""
+    rows = 1000
+    n_seq = -(-rows // rows_per_seq)
+    vl = (inputs.valid_lengths(n_seq, 77 + cols, 0, cols + 1)).astype(np.int32)
+    vl[::5] = cols
+    vl[1::11] = 0
+    x = inputs.normal_f32((rows, cols), 59 + cols, 0.0, 4.0)
+    got = ko.softmax_host(x, valid_len=vl, rows_per_seq=rows_per_seq)
+    assert_softmax_close(got, oracle.softmax(x, valid_len=vl, rows_per_seq=rows_per_seq))
+    for lpr in (8, 16, 32, 64):
+        ko.set_tuning("softmax.lanes_per_row", lpr)
+        try:
+            got = ko.softmax_host(x, valid_len=vl, rows_per_seq=rows_per_seq)
+        finally:
+            ko.set_tuning("softmax.lanes_per_row", 0)
+        assert_softmax_close(got, oracle.softmax(x, valid_len=vl, rows_per_seq=rows_per_seq))
+
+
 def test_softmax_properties(ko):
     cols = 128
     # constant row -> exactly 1/C; one-hot dominance; large magnitudes stay finite (max subtraction)
