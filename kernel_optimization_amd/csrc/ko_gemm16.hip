@@ -1083,12 +1083,9 @@ int launch_pinned(Params p, hipStream_t stream) {
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
     auto kernel = gemm16_pinned_kernel<T, BF16, B_ROW>;
-    static bool configured = false;
-    if (!configured) {
-        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+        return st;
     p.tiles_n = p.N / T::BN;
     const int tiles_m = p.M / T::BM;
     p.nblocks = tiles_m * p.tiles_n;
@@ -1116,12 +1113,9 @@ int launch_persistent(Params p, hipStream_t stream) {
     if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the persistent variant needs full tiles");
     auto kernel = gemm16_persistent_kernel<T, BF16>;
-    static bool configured = false;
-    if (!configured) {
-        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+        return st;
     p.tiles_n = p.N / T::BN;
     p.nblocks = (p.M / T::BM) * p.tiles_n;
     int grid = compute_units() / 8 * 8;  // a multiple of the XCD count keeps a workgroup's tiles on its XCD's band
@@ -1136,12 +1130,9 @@ int launch_edge(const Params &p, hipStream_t stream) {
     constexpr int THREADS = T::THREADS;
     constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     auto kernel = gemm16_kernel<T, BF16, B_ROW_MAJOR, EDGE>;
-    static bool configured = false;  // per instantiation
-    if (!configured) {
-        KO_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+        return st;
     kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;

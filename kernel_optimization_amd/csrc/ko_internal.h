@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -24,8 +25,13 @@ int tuning(const char *name);
 
 inline hipStream_t as_stream(ko_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
-// Number of compute units of the current device (cached).
+// Number of compute units of the current device (cached per device).
 int compute_units();
+
+// Raises the dynamic-LDS limit of `kernel` to `bytes` on the current device. The attribute belongs to the
+// device's copy of the kernel, so it is set once per device; `done` is the caller's per-kernel record of the
+// devices already served (bit d = device d; devices from 64 on are set every time).
+int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done);
 
 }  // namespace ko
 

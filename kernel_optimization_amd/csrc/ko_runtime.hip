@@ -49,15 +49,28 @@ int tuning(const char *name) {
 }
 
 int compute_units() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
+    constexpr int kCached = 64;
+    static std::atomic<int> cus[kCached];  // zero-initialised; 0 = not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev >= 0 && dev < kCached) {
+        const int known = cus[dev].load(std::memory_order_relaxed);
+        if (known > 0) return known;
     }
-    return cus;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (dev >= 0 && dev < kCached) cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done) {
+    int dev = 0;
+    KO_HIP(hipGetDevice(&dev));
+    const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t{1} << dev) : 0;
+    if (bit && (done.load(std::memory_order_acquire) & bit)) return KO_OK;
+    KO_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    if (bit) done.fetch_or(bit, std::memory_order_release);
+    return KO_OK;
 }
 
 }  // namespace ko
