@@ -28,6 +28,9 @@
 //   simt_gemm.h:287-292)
 #include "ko_internal.h"
 
+#include <type_traits>
+#include <utility>
+
 namespace ko {
 namespace {
 
@@ -74,6 +77,85 @@ __device__ __forceinline__ void tile_of(const Params &p, int b, int &tile_m, int
         tile_m = b / p.tiles_n;
         tile_n = b % p.tiles_n;
     }
+}
+
+// Sums the partial accumulators of the K splits through LDS (every wave must be past its last use of
+// the stages) and writes D = alpha * acc + beta * C.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT, int TM, int TN, bool FULL>
+__device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc)[TM][TN], float4v *lds, int wave,
+                                                 int lane, int m0, int n0) {
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    const int split = wave / (WAVES_M * WAVES_N);
+    const int wm = (wave / WAVES_N) % WAVES_M, wn = wave % WAVES_N;
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+    const int M = p.M, N = p.N;
+    if constexpr (KSPLIT > 1) {
+        // Sum the partial accumulators of the K splits into split 0 (fixed order: 1, 2, ...).
+        // Every wave is past the last barrier of the main loop, so the stages are free.
+        constexpr int PER_WAVE = TM * TN * 4 * 64;  // float4 slots of one wave's accumulators
+        const int sub = wave % (WAVES_M * WAVES_N);
+        if (split > 0) {
+            float4v *dst = lds + ((split - 1) * WAVES_M * WAVES_N + sub) * PER_WAVE;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                        dst[((i * TN + j) * 4 + q) * 64 + lane] = v;
+                    }
+        }
+        __syncthreads();
+        if (split > 0) return;
+#pragma unroll
+        for (int s = 1; s < KSPLIT; ++s) {
+            const float4v *src = lds + ((s - 1) * WAVES_M * WAVES_N + sub) * PER_WAVE;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float4v v = src[((i * TN + j) * 4 + q) * 64 + lane];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
+                        // one 32 x 32 accumulator at a time: with all reads issued first, a 128 x 128 tile
+                        // needs 64 more registers here than anywhere in the K loop
+                        if (q == 3) __builtin_amdgcn_sched_barrier(0);
+                    }
+        }
+    }
+
+    // acc[i][j][r] is D[m][n] with m = 8*(r/4) + 4*(lane/32) + r%4, n = lane%32 inside
+    // the 32x32 tile: for a fixed r the 32 lanes of a half-wave write 128 contiguous bytes.
+    const float alpha = p.alpha, beta = p.beta;
+    // The choice between "with C" and "without" is made once, not per element, and the 32 x 32 sub-tiles
+    // are written one after the other (the addresses of all of them at once would not fit the registers).
+    auto store_all = [&](auto with_c) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = n0 + wn * WTN + j * 32 + frow;
+                if (FULL || n < N) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int m = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
+                        if (!FULL && m >= M) continue;
+                        const int64_t off = static_cast<int64_t>(m) * N + n;
+                        float v = alpha * acc[i][j][r];
+                        if constexpr (decltype(with_c)::value) v += beta * p.C[off];
+                        __builtin_nontemporal_store(v, &p.D[off]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    if (p.C != nullptr && beta != 0.0f) store_all(std::true_type{});
+    else store_all(std::false_type{});
 }
 
 // VEC: K % 4 == 0, N % 4 == 0 and 16-byte aligned A and B (128-bit global loads);
@@ -283,62 +365,221 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_kernel(
         }
     }
 
-    if constexpr (KSPLIT > 1) {
-        // Sum the partial accumulators of the K splits into split 0 (fixed order: 1, 2, ...).
-        // Every wave is past the last barrier of the main loop, so the stages are free.
-        constexpr int PER_WAVE = TM * TN * 4 * 64;  // float4 slots of one wave's accumulators
-        const int sub = wave % (WAVES_M * WAVES_N);
-        if (split > 0) {
-            float4v *dst = lds + ((split - 1) * WAVES_M * WAVES_N + sub) * PER_WAVE;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                        dst[((i * TN + j) * 4 + q) * 64 + lane] = v;
-                    }
-        }
-        __syncthreads();
-        if (split > 0) return;
-#pragma unroll
-        for (int s = 1; s < KSPLIT; ++s) {
-            const float4v *src = lds + ((s - 1) * WAVES_M * WAVES_N + sub) * PER_WAVE;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float4v v = src[((i * TN + j) * 4 + q) * 64 + lane];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
-                    }
-        }
-    }
+    reduce_and_store<BM, BN, WAVES_M, WAVES_N, KSPLIT, TM, TN, FULL>(p, acc, lds, wave, lane, m0, n0);
+}
 
-    // acc[i][j][r] is D[m][n] with m = 8*(r/4) + 4*(lane/32) + r%4, n = lane%32 inside
-    // the 32x32 tile: for a fixed r the 32 lanes of a half-wave write 128 contiguous bytes.
-    const float alpha = p.alpha, beta = p.beta;
-    const bool use_c = p.C != nullptr && beta != 0.0f;
+template <int IMM>
+__device__ __forceinline__ void lds_read_b128(float4v &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(IMM));
+}
+template <int IMM>
+__device__ __forceinline__ void lds_read_b32(float &dst, uint32_t addr) {
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(IMM));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// Direct-to-LDS kernel for full tiles and an even number of K tiles: the same tiles, LDS layout, fragment
+// order and epilogue as the PIPE form of sgemm_kernel, but global_load_lds_dwordx4 moves 16 bytes per
+// lane from global memory straight into LDS (lane l of a wave-level load fills the l-th 16-byte slot
+// after the wave-uniform LDS base), so the staging registers, the LDS writes and their address
+// arithmetic leave the K loop.  The swizzles are applied on the global side: the lane that fills slot
+// (row, c) fetches chunk c ^ swz(row) of that row.  NSTAGE stages of LDS: while tile kt is multiplied
+// out of registers, the fragments of tile kt + 1 are read from its stage and tiles up to kt + NSTAGE are
+// in flight (the newest one into the stage tile kt has just left).
+//
+// The compiler counts a direct-to-LDS load as an LDS write that any LDS read may alias and would wait
+// for all of them (vmcnt(0)) before every fragment read it knows of; so the fragment reads and their
+// waits are inline assembly.  Registers filled by such a read pass through an empty assembly statement
+// behind the wait before the MFMAs use them, which keeps every use (and every copy) behind the wait.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT)
+__attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(const Params p) {
+    constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_ROW_CHUNKS = BK / 4;
+    constexpr int A_CHUNKS = BM * A_ROW_CHUNKS;
+    constexpr int B_CHUNKS = BK * BN / 4;
+    constexpr int BNC = BN / 4;
+    constexpr int CHUNKS = A_CHUNKS + B_CHUNKS;
+    constexpr int LOADS = CHUNKS / THREADS;      // wave-level loads per wave and K tile
+    constexpr int A_LOADS = A_CHUNKS / THREADS;  // the first A_LOADS of them fetch A
+    constexpr int KGROUPS = BK / 8;
+    constexpr int GROUPS = KGROUPS / KSPLIT;
+    constexpr int STAGE_BYTES = CHUNKS * 16;
+    static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "a wave-level load stays inside A or B");
+    static_assert(KGROUPS % KSPLIT == 0 && (BK == 16 || BK == 32 || BK == 64) && BN % 64 == 0 && NSTAGE >= 2, "");
+    static_assert((NSTAGE - 1) * LOADS < 64 && BK * BN * 4 < 65536 && TM * 32 * A_ROW_CHUNKS * 16 < 65536, "");
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+
+    extern __shared__ float4v lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int split = wave / (WAVES_M * WAVES_N);
+    const int wm = (wave / WAVES_N) % WAVES_M, wn = wave % WAVES_N;
+    int tile_m, tile_n;
+    tile_of(p, static_cast<int>(blockIdx.x), tile_m, tile_n);
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+    const int N = p.N, K = p.K;
+    const int KT = K / BK;
+
+    // A rows of 256 bytes fill a line of the 64 banks; of 128 (64) bytes two (four) rows share one, and
+    // the number of the row pair (quadruple) goes into the swizzle.
+    auto swz_a = [](int row) { return BK == 16 ? (row >> 2) & 3 : BK == 32 ? (row >> 1) & 7 : row & 15; };
+    auto swz_b = [](int k) { return ((k >> 2) & 1) << 3; };
+
+    // What this thread fetches with each of its loads: LDS slot tid + i * THREADS of the stage, K tile 0.
+    const char *src[LOADS];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + wn * WTN + j * 32 + frow;
-            if (!FULL && n >= N) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
-                if (!FULL && m >= M) continue;
-                const int64_t off = static_cast<int64_t>(m) * N + n;
-                float v = alpha * acc[i][j][r];
-                if (use_c) v += beta * p.C[off];
-                __builtin_nontemporal_store(v, &p.D[off]);
-            }
+    for (int i = 0; i < LOADS; ++i) {
+        const int idx = tid + i * THREADS;
+        if (i < A_LOADS) {
+            const int row = idx / A_ROW_CHUNKS, c = idx % A_ROW_CHUNKS;
+            src[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + row) * K + 4 * (c ^ swz_a(row)));
+        } else {
+            const int b = idx - A_CHUNKS;
+            const int kr = b / BNC, c = b % BNC;
+            src[i] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(kr) * N + n0 + 4 * (c ^ swz_b(kr)));
         }
     }
+    const int64_t step_a = BK * 4, step_b = static_cast<int64_t>(BK) * N * 4;
+    int ld_kt = 0;  // the K tile the sources point at
+    // Loads past the last K tile are not branched around: they fetch the last tile once more, into a
+    // stage nobody reads any more, so that the count of loads in flight is the same on every path.
+    auto issue = [&](int stage) {
+        char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
+        const bool more = ld_kt + 1 < KT;
+        ld_kt += more ? 1 : 0;
+        const int64_t da = more ? step_a : 0, db = more ? step_b : 0;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) src[i] += i < A_LOADS ? da : db;
+    };
+
+    // LDS byte addresses of this lane's fragments in stage 0 (see read_frags of sgemm_kernel): per group
+    // of 8 k for A (the swizzle depends on the chunk), per 32 columns for B; the rest are immediates.
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));  // LDS aperture offset
+    uint32_t addr_a[GROUPS], addr_b[TN];
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const int chunk = 2 * (split + g * KSPLIT) + fhalf;
+        const int row = wm * WTM + frow;  // rows 32 apart share the swizzle
+        addr_a[g] = lds_base + (row * A_ROW_CHUNKS + (chunk ^ swz_a(row))) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = (wn * WTN + j * 32 + frow) ^ (fhalf << 5);
+        addr_b[j] = lds_base + A_CHUNKS * 16 + ((8 * split + 4 * fhalf) * BN + col) * 4;
+    }
+    auto read_frags = [&](int stage, float4v (&af)[GROUPS][TM], float (&bf)[GROUPS][TN][4]) {
+        const uint32_t off = static_cast<uint32_t>(stage) * STAGE_BYTES;
+        static_for<GROUPS>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            const uint32_t a = addr_a[g] + off;
+            static_for<TM>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+                lds_read_b128<i * 32 * A_ROW_CHUNKS * 16>(af[g][i], a);
+            });
+        });
+        static_for<TN>([&](auto j_c) {
+            constexpr int j = decltype(j_c)::value;
+            const uint32_t b = addr_b[j] + off;
+            static_for<GROUPS * 4>([&](auto gt_c) {
+                constexpr int g = decltype(gt_c)::value / 4, t = decltype(gt_c)::value % 4;
+                lds_read_b32<(8 * g * KSPLIT + t) * BN * 4>(bf[g][j][t], b);
+            });
+        });
+    };
+    // All LDS reads of this wave have landed; the fragments become usable.
+    auto frags_ready = [&](float4v (&af)[GROUPS][TM], float (&bf)[GROUPS][TN][4]) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(af[g][i]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(bf[g][j][t]));
+        }
+    };
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    auto multiply = [&](const float4v (&af)[TM], const float (&bf)[TN][4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
+    };
+
+    float4v af0[GROUPS][TM], af1[GROUPS][TM];  // fragments of the even / odd K tile
+    float bf0[GROUPS][TN][4], bf1[GROUPS][TN][4];
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) issue(s);  // K tiles 0 .. NSTAGE - 1
+    wait_vm<(NSTAGE - 1) * LOADS>();
+    asm volatile("s_barrier" ::: "memory");
+    read_frags(0, af0, bf0);
+    int wr = 0, rd = 1;  // stages of K tiles kt and kt + 1
+    // One K tile.  Before the barrier: this wave's share of tile kt + 1 has landed and its reads of tile
+    // kt's stage are complete.  Behind it: that stage takes tile kt + NSTAGE, the fragments of tile
+    // kt + 1 are read under the MFMAs of tile kt.  After the last tile the reads fetch stale (in-bounds)
+    // LDS contents that nothing uses.
+    auto step = [&](float4v (&af_cur)[GROUPS][TM], float (&bf_cur)[GROUPS][TN][4], float4v (&af_next)[GROUPS][TM],
+                    float (&bf_next)[GROUPS][TN][4]) {
+        wait_vm<(NSTAGE - 2) * LOADS>();
+        frags_ready(af_cur, bf_cur);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(af_cur[0], bf_cur[0]);  // the matrix cores start right behind the barrier
+        __builtin_amdgcn_sched_barrier(0);
+        issue(wr);
+        read_frags(rd, af_next, bf_next);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 1; g < GROUPS; ++g) multiply(af_cur[g], bf_cur[g]);
+        __builtin_amdgcn_sched_barrier(0);
+        wr = rd;
+        rd = rd + 1 == NSTAGE ? 0 : rd + 1;
+    };
+    for (int kt = 0; kt < KT; kt += 2) {
+        step(af0, bf0, af1, bf1);
+        step(af1, bf1, af0, bf0);
+    }
+    // The redirected loads still in flight write LDS, and the last fragment reads are pending: both end
+    // before the reduction reuses the stages.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    reduce_and_store<BM, BN, WAVES_M, WAVES_N, KSPLIT, TM, TN, true>(p, acc, lds, wave, lane, m0, n0);
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, bool PIPE = false>
@@ -363,6 +604,32 @@ int launch(Params p, hipStream_t stream) {
     return KO_OK;
 }
 
+// The direct-to-LDS kernel where it applies (full tiles, 16-byte aligned operands, an even number of K
+// tiles), else the register pipeline with the same tiling.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, int FALLBACK_BK = BK>
+int launch_direct(Params p, hipStream_t stream) {
+    constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
+    constexpr size_t stage_bytes = static_cast<size_t>(NSTAGE) * (BM * BK + BK * BN) * 4;
+    constexpr size_t reduce_bytes = static_cast<size_t>(KSPLIT - 1) * BM * BN * 4;  // the split-K reduction reuses the stages
+    constexpr size_t lds_bytes = stage_bytes > reduce_bytes ? stage_bytes : reduce_bytes;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
+    const bool full = aligned && p.M % BM == 0 && p.N % BN == 0 && p.K % (2 * BK) == 0;
+    if (!full) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
+    const int tiles_m = p.M / BM;
+    p.tiles_n = p.N / BN;
+    const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
+    if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
+    p.blocked = tuning("sgemm.mapping") != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
+                ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
+    auto kernel = sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE>;
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+        return st;
+    kernel<<<dim3(static_cast<unsigned>(nblocks)), dim3(THREADS), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 }  // namespace
 }  // namespace ko
 
@@ -382,12 +649,14 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     if (variant <= 0) {
         // Few tiles (fewer 128 x 128 tiles than compute units): 64 x 64 tiles with K split four ways inside
         // the workgroup; otherwise 128 x 128 tiles with K split two ways (2048^3, one tile per compute unit:
-        // 136 us against 148 us).
-        // Very few (64 x 64 tiles for at most half of the compute units): 32 x 64 tiles (512^3: 8.8 us against
-        // 12.2 us).
+        // 130 us against 149 us).
+        // Very few (64 x 64 tiles for at most half of the compute units): 32 x 64 tiles (512^3: 8.0 us against
+        // 12.1 us).
+        // All three as direct-to-LDS kernels; shapes those do not take fall back to the register pipeline
+        // with the same tiling.
         const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
         const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64);
-        variant = t128 >= compute_units() ? 16 : (2 * t64 <= compute_units() ? 21 : 13);
+        variant = t128 >= compute_units() ? 36 : (2 * t64 <= compute_units() ? 41 : 33);
     }
     switch (variant) {
         case 1: return launch<64, 64, 32, 2, 2, 1>(p, s);
@@ -410,6 +679,13 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
         case 18: return launch<128, 64, 32, 2, 2, 2, true>(p, s);
         case 19: return launch<128, 64, 64, 2, 2, 2, true>(p, s);
         case 21: return launch<32, 64, 64, 1, 2, 4, true>(p, s);
+        case 33: return launch_direct<64, 64, 64, 2, 2, 4, 3>(p, s);
+        case 34: return launch_direct<64, 64, 64, 2, 2, 4, 4>(p, s);
+        case 36: return launch_direct<128, 128, 32, 2, 2, 2, 2>(p, s);
+        case 37: return launch_direct<128, 128, 32, 2, 2, 2, 3>(p, s);
+        case 38: return launch_direct<128, 128, 16, 2, 2, 2, 3, 32>(p, s);
+        case 39: return launch_direct<128, 128, 16, 2, 2, 2, 4, 32>(p, s);
+        case 41: return launch_direct<32, 64, 64, 1, 2, 4, 3>(p, s);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: unknown variant %d", variant);
     }
 }

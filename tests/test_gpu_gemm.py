@@ -8,7 +8,8 @@ from tolerances import assert_gemm16_close, assert_sgemm_close
 
 pytestmark = pytest.mark.gpu
 
-SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 21]
+SGEMM_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 21, 33, 34, 36, 37, 38, 39, 41]
+SGEMM_PIPELINED = [12, 13, 14, 15, 16, 17, 18, 19, 21, 33, 34, 36, 37, 38, 39, 41]  # two K tiles per loop trip; 33 on: direct-to-LDS
 GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 30, 50, 52, 53]
 
 
@@ -30,12 +31,27 @@ def gemm16_variant(ko, request):
 
 @pytest.mark.parametrize("sgemm_variant", SGEMM_VARIANTS, indirect=True)
 @pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 256, 96), (200, 136, 40), (1, 4, 4), (65, 129, 33),
-                                   (37, 50, 7)])
+                                   (37, 50, 7), (128, 256, 128), (256, 128, 384)])
 def test_sgemm_matches_oracle(ko, sgemm_variant, m, n, k):
     A = inputs.uniform_f32((m, k), 11 + m)
     B = inputs.uniform_f32((k, n), 13 + n)
     ref, ap = oracle.sgemm(A, B, want_absprod=True)
     assert_sgemm_close(ko.sgemm_host(A, B), ref, ap, k)
+
+
+@pytest.mark.parametrize("sgemm_variant", SGEMM_PIPELINED, indirect=True)
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (512, 384, 512), (256, 640, 1152), (1024, 1024, 256)])
+def test_sgemm_pipelined_variants_are_exact_on_small_integers(ko, sgemm_variant, m, n, k):
+    """Full tiles and an even number of K tiles put the pipelined kernels (register staging or direct-to-LDS
+    loads, two to four LDS stages) on their fast path; with small integers every product and sum is exact, so
+    any misplaced element of a tile shows as a wrong integer."""
+    rng = np.random.default_rng(1000 * sgemm_variant + m + k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B), A.astype(np.float64) @ B.astype(np.float64))
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0),
+                                  2.0 * (A.astype(np.float64) @ B.astype(np.float64)) - C)
 
 
 def test_sgemm_cfg3_full(ko):
