@@ -181,3 +181,33 @@ def test_softmax_full_size_cfg1_properties(ko):
     # the device fill is the same generator as the host one
     host = inputs.normal_f32((64, cols), inputs.tensor_seed(1, 0), 0.0, 4.0)
     assert np.all(np.abs(host - x[:64]) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))
+
+
+def test_masked_softmax_full_size_cfg5(ko):
+    """[786432,512] with per-sequence valid lengths in [64,512] at full size (1.6 GB in, 1.6 GB out; byte
+    offsets pass 2^31), inputs filled on the device: the whole output against the oracle on the very bytes the
+    kernel read, sequence block by sequence block, plus the properties that hold at any size."""
+    c = inputs.CONFIGS[5]
+    rows, cols, rows_per_seq, n_seq = c["rows"], c["cols"], c["rows_per_seq"], c["n_seq"]
+    assert (rows, cols, rows_per_seq * n_seq) == (786432, 512, 786432)
+    n = rows * cols
+    dx, dy, dl = ko.DeviceBuffer(n * 4), ko.DeviceBuffer(n * 4), ko.DeviceBuffer(n_seq * 4)
+    ko.fill_normal_f32(dx, n, inputs.tensor_seed(5, 0), 0.0, 4.0)
+    ko.fill_lengths_i32(dl, n_seq, inputs.tensor_seed(5, 1), c["len_lo"], c["len_hi"])
+    ko.softmax(dx, dy, rows, cols, valid_len=dl, rows_per_seq=rows_per_seq)
+    ko.synchronize()
+    vl = dl.download(np.int32, (n_seq,))
+    np.testing.assert_array_equal(vl, inputs.valid_lengths(n_seq, inputs.tensor_seed(5, 1), c["len_lo"], c["len_hi"]))
+    assert vl.min() >= 64 and vl.max() <= 512 and len(np.unique(vl)) > 64
+    x = dx.download(np.float32, (rows, cols))
+    y = dy.download(np.float32, (rows, cols))
+    seqs_per_block = 16
+    for s0 in range(0, n_seq, seqs_per_block):
+        r0, r1 = s0 * rows_per_seq, (s0 + seqs_per_block) * rows_per_seq
+        yb, lens = y[r0:r1], vl[s0:s0 + seqs_per_block]
+        assert_softmax_close(yb, oracle.softmax(x[r0:r1], valid_len=lens, rows_per_seq=rows_per_seq))
+        assert np.abs(yb.sum(1, dtype=np.float64) - 1).max() <= cols * 2.0 ** -24
+        for i, L in enumerate(lens):
+            blk = yb[i * rows_per_seq:(i + 1) * rows_per_seq]
+            assert np.all(blk[:, L:] == 0.0)  # padded columns are exact zeros
+            assert blk[:, :L].min() >= 0.0
