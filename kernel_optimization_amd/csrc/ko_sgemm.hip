@@ -463,16 +463,19 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     int ld_kt = 0;  // the K tile the sources point at
     // Loads past the last K tile are not branched around: they fetch the last tile once more, into a
     // stage nobody reads any more, so that the count of loads in flight is the same on every path.
-    auto issue = [&](int stage) {
-        char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * 1024;
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
+    auto advance = [&]() {
         const bool more = ld_kt + 1 < KT;
         ld_kt += more ? 1 : 0;
         const int64_t da = more ? step_a : 0, db = more ? step_b : 0;
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) src[i] += i < A_LOADS ? da : db;
+    };
+    auto issue = [&](int stage) {
+        char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
+        advance();
     };
 
     // LDS byte addresses of this lane's fragments in stage 0 (see read_frags of sgemm_kernel): per group
@@ -532,16 +535,6 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-    auto multiply = [&](const float4v (&af)[TM], const float (&bf)[TN][4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
-    };
-
     float4v af0[GROUPS][TM], af1[GROUPS][TM];  // fragments of the even / odd K tile
     float bf0[GROUPS][TN][4], bf1[GROUPS][TN][4];
 #pragma unroll
@@ -560,14 +553,35 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
         frags_ready(af_cur, bf_cur);
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
-        multiply(af_cur[0], bf_cur[0]);  // the matrix cores start right behind the barrier
-        __builtin_amdgcn_sched_barrier(0);
-        issue(wr);
-        read_frags(rd, af_next, bf_next);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int g = 1; g < GROUPS; ++g) multiply(af_cur[g], bf_cur[g]);
-        __builtin_amdgcn_sched_barrier(0);
+        // The loads of tile kt + NSTAGE and the fragment reads of tile kt + 1 are spread over the MFMAs
+        // of tile kt, PER of them behind each MFMA until they run out, loads first: the wave never
+        // stands between two MFMAs for longer than that, so the matrix core's queue does not run dry
+        // while all waves of the workgroup are in the same part of the step.
+        constexpr int NMFMA = GROUPS * 4 * TM * TN;
+        constexpr int A_READS = GROUPS * TM, B_READS = TN * GROUPS * 4;
+        constexpr int PIECES = LOADS + A_READS + B_READS;
+        constexpr int PER = (PIECES + NMFMA - 1) / NMFMA;
+        char *dst = reinterpret_cast<char *>(lds) + wr * STAGE_BYTES + wave * 1024;
+        const uint32_t off = static_cast<uint32_t>(rd) * STAGE_BYTES;
+        static_for<NMFMA>([&](auto q_c) {
+            constexpr int q = decltype(q_c)::value;
+            constexpr int g = q / (4 * TM * TN), t = (q / (TM * TN)) % 4, i = (q / TN) % TM, j = q % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af_cur[g][i][t], bf_cur[g][j][t], acc[i][j], 0, 0, 0);
+            static_for<PER>([&](auto r_c) {
+                constexpr int pc = q * PER + decltype(r_c)::value;
+                if constexpr (pc < LOADS) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)src[pc], (lptr_t)(dst + pc * THREADS * 16), 16, 0, 0);
+                    if constexpr (pc == LOADS - 1) advance();
+                } else if constexpr (pc < LOADS + A_READS) {
+                    constexpr int u = pc - LOADS, g2 = u / TM, i2 = u % TM;
+                    lds_read_b128<i2 * 32 * A_ROW_CHUNKS * 16>(af_next[g2][i2], addr_a[g2] + off);
+                } else if constexpr (pc < PIECES) {
+                    constexpr int u = pc - LOADS - A_READS, j2 = u / (GROUPS * 4), g2 = (u / 4) % GROUPS, t2 = u % 4;
+                    lds_read_b32<(8 * g2 * KSPLIT + t2) * BN * 4>(bf_next[g2][j2][t2], addr_b[j2] + off);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
         wr = rd;
         rd = rd + 1 == NSTAGE ? 0 : rd + 1;
     };
