@@ -421,7 +421,7 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     constexpr int GROUPS = KGROUPS / KSPLIT;
     constexpr int STAGE_BYTES = CHUNKS * 16;
     static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "a wave-level load stays inside A or B");
-    static_assert(KGROUPS % KSPLIT == 0 && (BK == 16 || BK == 32 || BK == 64) && BN % 64 == 0 && NSTAGE >= 2, "");
+    static_assert(KGROUPS % KSPLIT == 0 && (BK == 16 || BK == 32 || BK == 64 || BK == 128) && BN % 64 == 0 && NSTAGE >= 2, "");
     static_assert((NSTAGE - 1) * LOADS < 64 && BK * BN * 4 < 65536 && TM * 32 * A_ROW_CHUNKS * 16 < 65536, "");
     typedef const __attribute__((address_space(1))) void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
@@ -667,10 +667,14 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
         // Very few (64 x 64 tiles for at most half of the compute units): 32 x 64 tiles (512^3: 8.0 us against
         // 12.1 us).
         // All three as direct-to-LDS kernels; shapes those do not take fall back to the register pipeline
-        // with the same tiling.
+        // with the same tiling.  The 64 x 64 tiles take 128 k per step (two LDS stages of 64 KB) where K
+        // allows: half as many barriers of the 16 waves (1024 x 1024 x 4096: 67 us against 73 us).
+        // The 128 x 128 tiles take 64 k per step from K = 2048 on (2048^3: 126 us against 143 us; the same
+        // at 4096^3; shallower K loses more to the larger first tile than it gains).
         const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
         const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64);
-        variant = t128 >= compute_units() ? 36 : (2 * t64 <= compute_units() ? 41 : 33);
+        variant = t128 >= compute_units() ? (k >= 2048 && k % 128 == 0 ? 40 : 36)
+                                           : (2 * t64 <= compute_units() ? 41 : (k % 256 == 0 ? 35 : 33));
     }
     switch (variant) {
         case 1: return launch<64, 64, 32, 2, 2, 1>(p, s);
@@ -695,10 +699,12 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
         case 21: return launch<32, 64, 64, 1, 2, 4, true>(p, s);
         case 33: return launch_direct<64, 64, 64, 2, 2, 4, 3>(p, s);
         case 34: return launch_direct<64, 64, 64, 2, 2, 4, 4>(p, s);
+        case 35: return launch_direct<64, 64, 128, 2, 2, 4, 2, 64>(p, s);
         case 36: return launch_direct<128, 128, 32, 2, 2, 2, 2>(p, s);
         case 37: return launch_direct<128, 128, 32, 2, 2, 2, 3>(p, s);
         case 38: return launch_direct<128, 128, 16, 2, 2, 2, 3, 32>(p, s);
         case 39: return launch_direct<128, 128, 16, 2, 2, 2, 4, 32>(p, s);
+        case 40: return launch_direct<128, 128, 64, 2, 2, 2, 2, 32>(p, s);
         case 41: return launch_direct<32, 64, 64, 1, 2, 4, 3>(p, s);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: unknown variant %d", variant);
     }
