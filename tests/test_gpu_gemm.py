@@ -40,7 +40,7 @@ def test_sgemm_matches_oracle(ko, sgemm_variant, m, n, k):
 
 
 @pytest.mark.parametrize("sgemm_variant", SGEMM_PIPELINED, indirect=True)
-@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (512, 384, 512), (256, 640, 1152), (1024, 1024, 256)])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (512, 384, 512), (256, 640, 1152), (1024, 1024, 256), (512, 256, 96)])
 def test_sgemm_pipelined_variants_are_exact_on_small_integers(ko, sgemm_variant, m, n, k):
     """Full tiles and an even number of K tiles put the pipelined kernels (register staging or direct-to-LDS
     loads, two to four LDS stages) on their fast path; with small integers every product and sum is exact, so
