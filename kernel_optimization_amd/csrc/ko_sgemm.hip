@@ -644,22 +644,9 @@ int launch_direct(Params p, hipStream_t stream) {
     return KO_OK;
 }
 
-}  // namespace
-}  // namespace ko
-
-KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A,
-                           const float *B, float beta, const float *C, float *D,
-                           ko_stream_t stream) {
-    using namespace ko;
-    if (m < 0 || n < 0 || k < 0)
-        return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
-    if (m == 0 || n == 0) return KO_OK;
-    if (k == 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: k must be positive");
-    if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: dimension too large");
-    if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
-    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0};
-    hipStream_t s = as_stream(stream);
-    int variant = tuning("sgemm.variant");
+// One launch: the tiling by shape (variant <= 0) or the one asked for.
+int run(Params p, hipStream_t s, int variant) {
+    const int64_t m = p.M, n = p.N, k = p.K;
     if (variant <= 0) {
         // Few tiles (fewer 128 x 128 tiles than compute units): 64 x 64 tiles with K split four ways inside
         // the workgroup; otherwise 128 x 128 tiles with K split two ways (2048^3, one tile per compute unit:
@@ -708,4 +695,45 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
         case 41: return launch_direct<32, 64, 64, 1, 2, 4, 3>(p, s);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: unknown variant %d", variant);
     }
+}
+
+}  // namespace
+}  // namespace ko
+
+KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A,
+                           const float *B, float beta, const float *C, float *D,
+                           ko_stream_t stream) {
+    using namespace ko;
+    if (m < 0 || n < 0 || k < 0)
+        return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
+    if (m == 0 || n == 0) return KO_OK;
+    if (k == 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: k must be positive");
+    if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: dimension too large");
+    if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
+    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0};
+    hipStream_t s = as_stream(stream);
+    const int variant = tuning("sgemm.variant");
+    if (variant <= 0 && tuning("sgemm.split_rows") != 1 && k >= 512) {
+        // A last round of 128 x 128 tiles that fills at most half of the compute units costs a whole round:
+        // the tile rows that fill whole rounds go out as one launch, the rows below them as a second one
+        // with the smaller tiles its own size asks for (4096 x 4224 x 4096, 1056 tiles on 256 compute
+        // units: 1023 tiles in four rounds plus 132 tiles of 64 x 64 instead of five rounds).
+        const int64_t cu = compute_units();
+        const int64_t tm = (m + 127) / 128, tn = (n + 127) / 128;
+        const int64_t rounds = tm * tn / cu;
+        const int64_t rows1 = rounds * cu / tn;          // whole tile rows within the full rounds
+        const int64_t below = (tm - rows1) * tn;         // 128 x 128 tiles left for the second launch
+        if (rounds >= 1 && rows1 >= 1 && rows1 < tm && (tm * tn) % cu != 0 && 2 * below <= cu) {
+            const int64_t m1 = rows1 * 128;
+            Params top = p, bottom = p;
+            top.M = static_cast<int>(m1);
+            bottom.M = static_cast<int>(m - m1);
+            bottom.A = A + m1 * k;
+            bottom.C = C ? C + m1 * n : nullptr;
+            bottom.D = D + m1 * n;
+            if (const int st = run(top, s, 0); st != KO_OK) return st;
+            return run(bottom, s, 0);
+        }
+    }
+    return run(p, s, variant);
 }

@@ -54,6 +54,26 @@ def test_sgemm_pipelined_variants_are_exact_on_small_integers(ko, sgemm_variant,
                                   2.0 * (A.astype(np.float64) @ B.astype(np.float64)) - C)
 
 
+@pytest.mark.parametrize("m,n,k", [(2176, 2048, 512), (2100, 2050, 520), (4224, 2048, 512)])
+def test_sgemm_uneven_last_round_goes_out_as_two_launches(ko, m, n, k):
+    """A few more 128 x 128 tiles than a whole number of rounds on 256 compute units: the tile rows of the full
+    rounds and the rows below them are separate launches with different tilings.  Small integers make every
+    sum exact, so a row computed twice, skipped or offset shows as a wrong integer; with the split switched
+    off the same call gives the same matrix."""
+    rng = np.random.default_rng(m + n + k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B), ref)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C)
+    ko.set_tuning("sgemm.split_rows", 1)
+    try:
+        np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C)
+    finally:
+        ko.set_tuning("sgemm.split_rows", 0)
+
+
 def test_sgemm_cfg3_full(ko):
     """1024^3, U(-1,1), alpha=1, beta=0, C null: the whole output against the oracle, with the
     reference's own abs <= 1e-3 gate (nn_operators/gemm/main.cu:169-170) as well."""
