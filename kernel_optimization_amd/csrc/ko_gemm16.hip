@@ -1178,6 +1178,29 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // multiple of 128), else as the register pipeline.
         // Fewer: smaller tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
+        // A last round of a few big tiles costs a whole round: the tile rows that fill whole rounds go out as
+        // one launch, the rows below them as a second one with the tiling their own size asks for.  Pays while
+        // the rows below hold at most a sixth of a round (4352 x 4096 x 1024, 272 tiles on 256 compute units:
+        // 52.7 -> 42.7 us; 8192 x 2304 x 768, 288 tiles: 41.1 -> 37.4 us; with 65 or 72 tiles below the cut the
+        // small tilings take as long as the round they replace).
+        if (tuning("gemm16.split_rows") != 1 && p.K >= 256) {
+            const int64_t cu = compute_units();
+            const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+            const int64_t rounds = big_tiles / cu;
+            const int64_t rows1 = rounds * cu / tn;     // whole tile rows within the full rounds
+            const int64_t below = (tm - rows1) * tn;    // big tiles left for the second launch
+            if (rounds >= 1 && rows1 >= 1 && rows1 < tm && big_tiles % cu != 0 && 6 * below <= cu) {
+                const int64_t m1 = rows1 * 256;
+                Params top = p, bottom = p;
+                top.M = static_cast<int>(m1);
+                bottom.M = p.M - static_cast<int>(m1);
+                bottom.A = p.A + m1 * p.K;
+                bottom.C = p.C ? p.C + m1 * p.N : nullptr;
+                bottom.D = p.D + m1 * p.N;
+                if (const int st = launch_variant<BF16, B_ROW_MAJOR>(top, stream); st != KO_OK) return st;
+                return launch_variant<BF16, B_ROW_MAJOR>(bottom, stream);
+            }
+        }
         // The pinned kernel is so much faster per tile that it wins from half a chip's worth of full tiles on
         // (192 tiles on 256 CUs: 16384 x 768 x 3072 takes 69 us against 103 us with 128 x 128 tiles; at 96 tiles
         // the two are level).

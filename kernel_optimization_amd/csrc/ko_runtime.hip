@@ -36,7 +36,7 @@ static std::map<std::string, int> &tuning_table() {
         {"softmax.block_threads", 0},
         {"layernorm.lanes_per_row", 0}, {"layernorm.blocks_per_cu", 0},
         {"layernorm.block_threads", 0}, {"layernorm.wave_threads", 0}, {"softmax.wave_threads", 0},
-        {"sgemm.variant", 0}, {"sgemm.mapping", 0}, {"sgemm.split_rows", 0}, {"gemm16.variant", 0}, {"gemm16.mapping", 0}, {"copy.blocks_per_cu", 0},
+        {"sgemm.variant", 0}, {"sgemm.mapping", 0}, {"sgemm.split_rows", 0}, {"gemm16.variant", 0}, {"gemm16.mapping", 0}, {"gemm16.split_rows", 0}, {"copy.blocks_per_cu", 0},
         {"copy.nontemporal", 0},
     };
     return t;
