@@ -171,7 +171,7 @@ def bench_sgemm(cfg, steps, warmup, vendor):
     res = dict(workload=c["name"], metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
                roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f32"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=None),
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=_traffic(c["name"])),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -207,7 +207,7 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False):
     res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
                roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=None),
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=_traffic(name)),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
