@@ -59,6 +59,7 @@ struct Params {
     float alpha, beta;
     int tiles_n;
     int blocked;  // 1: the tile grid is cut into 4 x 8 blocks, one per XCD and round (see tile_of)
+    int lda;      // floats between rows of A (K, or more when A is a column range of a wider matrix)
 };
 
 // Workgroup -> output tile.  Workgroups go to the 8 XCDs round-robin by index, each XCD has its own
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_kernel(
                 int gr = m0 + row;
                 if constexpr (!FULL) gr = gr < M ? gr : M - 1;
                 const int kc = k0 + c * 4;
-                const float *src = p.A + static_cast<int64_t>(gr) * K + kc;
+                const float *src = p.A + static_cast<int64_t>(gr) * p.lda + kc;
                 if constexpr (FULL) {
                     v = *reinterpret_cast<const float4v *>(src);
                 } else if constexpr (VEC) {
@@ -391,7 +392,10 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// Direct-to-LDS kernel for full tiles and an even number of K tiles: the same tiles, LDS layout, fragment
+// What lanes fetch in place of operand elements past the end of K.
+__device__ __attribute__((aligned(16))) const float zero_chunk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+// Direct-to-LDS kernel (EDGE false: full tiles and an even number of K tiles): the same tiles, LDS layout, fragment
 // order and epilogue as the PIPE form of sgemm_kernel, but global_load_lds_dwordx4 moves 16 bytes per
 // lane from global memory straight into LDS (lane l of a wave-level load fills the l-th 16-byte slot
 // after the wave-uniform LDS base), so the staging registers, the LDS writes and their address
@@ -404,7 +408,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 // for all of them (vmcnt(0)) before every fragment read it knows of; so the fragment reads and their
 // waits are inline assembly.  Registers filled by such a read pass through an empty assembly statement
 // behind the wait before the MFMAs use them, which keeps every use (and every copy) behind the wait.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, bool EDGE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT)
 __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(const Params p) {
     constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
@@ -438,7 +442,8 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
     const int N = p.N, K = p.K;
-    const int KT = K / BK;
+    // EDGE: K (a multiple of 4) is padded with zeros up to the next pair of K tiles.
+    const int KT = EDGE ? 2 * ((K + 2 * BK - 1) / (2 * BK)) : K / BK;
 
     // A rows of 256 bytes fill a line of the 64 banks; of 128 (64) bytes two (four) rows share one, and
     // the number of the row pair (quadruple) goes into the swizzle.
@@ -447,20 +452,33 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
 
     // What this thread fetches with each of its loads: LDS slot tid + i * THREADS of the stage, K tile 0.
     const char *src[LOADS];
+    int koff[EDGE ? LOADS : 1];  // EDGE: the k, within a K tile, of the chunk (A) or row (B) this lane fetches
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
         const int idx = tid + i * THREADS;
         if (i < A_LOADS) {
             const int row = idx / A_ROW_CHUNKS, c = idx % A_ROW_CHUNKS;
-            src[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + row) * K + 4 * (c ^ swz_a(row)));
+            if constexpr (EDGE) koff[i] = 4 * (c ^ swz_a(row));
+            int gr = m0 + row;
+            if constexpr (EDGE) gr = gr < p.M ? gr : p.M - 1;  // rows past M fetch the last row again; never stored
+            src[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(gr) * p.lda + 4 * (c ^ swz_a(row)));
         } else {
             const int b = idx - A_CHUNKS;
             const int kr = b / BNC, c = b % BNC;
-            src[i] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(kr) * N + n0 + 4 * (c ^ swz_b(kr)));
+            if constexpr (EDGE) koff[i] = kr;
+            int gn = n0 + 4 * (c ^ swz_b(kr));
+            if constexpr (EDGE) gn = gn < N ? gn : N - 4;  // columns past N (a multiple of 4) fetch the last chunk again
+            src[i] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(kr) * N + gn);
         }
     }
     const int64_t step_a = BK * 4, step_b = static_cast<int64_t>(BK) * N * 4;
     int ld_kt = 0;  // the K tile the sources point at
+    int k_left = K;  // EDGE: K - ld_kt * BK; chunks and rows at or past it are fetched from zeros instead
+    const char *zeros = reinterpret_cast<const char *>(&zero_chunk);
+    auto source = [&](int i) {
+        if constexpr (EDGE) return koff[i] < k_left ? src[i] : zeros;
+        else return src[i];
+    };
     // Loads past the last K tile are not branched around: they fetch the last tile once more, into a
     // stage nobody reads any more, so that the count of loads in flight is the same on every path.
     auto advance = [&]() {
@@ -469,12 +487,13 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
         const int64_t da = more ? step_a : 0, db = more ? step_b : 0;
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) src[i] += i < A_LOADS ? da : db;
+        if constexpr (EDGE) k_left = K - ld_kt * BK;
     };
     auto issue = [&](int stage) {
         char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)source(i), (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
         advance();
     };
 
@@ -570,7 +589,7 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
             static_for<PER>([&](auto r_c) {
                 constexpr int pc = q * PER + decltype(r_c)::value;
                 if constexpr (pc < LOADS) {
-                    __builtin_amdgcn_global_load_lds((gptr_t)src[pc], (lptr_t)(dst + pc * THREADS * 16), 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((gptr_t)source(pc), (lptr_t)(dst + pc * THREADS * 16), 16, 0, 0);
                     if constexpr (pc == LOADS - 1) advance();
                 } else if constexpr (pc < LOADS + A_READS) {
                     constexpr int u = pc - LOADS, g2 = u / TM, i2 = u % TM;
@@ -593,7 +612,7 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     // before the reduction reuses the stages.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    reduce_and_store<BM, BN, WAVES_M, WAVES_N, KSPLIT, TM, TN, true>(p, acc, lds, wave, lane, m0, n0);
+    reduce_and_store<BM, BN, WAVES_M, WAVES_N, KSPLIT, TM, TN, !EDGE>(p, acc, lds, wave, lane, m0, n0);
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, bool PIPE = false>
@@ -605,7 +624,7 @@ int launch(Params p, hipStream_t stream) {
     if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
     p.blocked = tuning("sgemm.mapping") != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
                 ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
-    const bool vec = (p.K % 4 == 0) && (p.N % 4 == 0) &&
+    const bool vec = (p.K % 4 == 0) && (p.lda % 4 == 0) && (p.N % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
     const bool full = vec && p.M % BM == 0 && p.N % BN == 0 && p.K % BK == 0;
     dim3 grid(static_cast<unsigned>(nblocks)), block(THREADS);
@@ -618,7 +637,7 @@ int launch(Params p, hipStream_t stream) {
     return KO_OK;
 }
 
-// The direct-to-LDS kernel where it applies (full tiles, 16-byte aligned operands, an even number of K
+// The direct-to-LDS kernel where it applies (operand rows on 16-byte boundaries, at least one pair of K
 // tiles), else the register pipeline with the same tiling.
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, int FALLBACK_BK = BK>
 int launch_direct(Params p, hipStream_t stream) {
@@ -626,18 +645,23 @@ int launch_direct(Params p, hipStream_t stream) {
     constexpr size_t stage_bytes = static_cast<size_t>(NSTAGE) * (BM * BK + BK * BN) * 4;
     constexpr size_t reduce_bytes = static_cast<size_t>(KSPLIT - 1) * BM * BN * 4;  // the split-K reduction reuses the stages
     constexpr size_t lds_bytes = stage_bytes > reduce_bytes ? stage_bytes : reduce_bytes;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
-    const bool full = aligned && p.M % BM == 0 && p.N % BN == 0 && p.K % (2 * BK) == 0;
-    if (!full) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
-    const int tiles_m = p.M / BM;
-    p.tiles_n = p.N / BN;
+    // Ragged shapes are handled in the kernel's EDGE form (rows past M and columns past N fetch valid data
+    // that is never stored, K is padded with zeros up to a pair of K tiles, stores are bounds-checked).
+    // Operand rows have to start on 16-byte boundaries and K must not end inside a 16-byte chunk.
+    const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
+                         p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
+    if (!aligned) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
+    const bool edge = p.M % BM != 0 || p.N % BN != 0 || p.K % (2 * BK) != 0;
+    const int tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
     if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
     p.blocked = tuning("sgemm.mapping") != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
                 ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
-    auto kernel = sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE>;
-    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
-    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+    auto kernel = edge ? sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, true>
+                       : sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, false>;
+    static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge]); st != KO_OK)
         return st;
     kernel<<<dim3(static_cast<unsigned>(nblocks)), dim3(THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
@@ -710,7 +734,7 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     if (k == 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: k must be positive");
     if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: dimension too large");
     if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
-    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0};
+    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, static_cast<int>(k)};
     hipStream_t s = as_stream(stream);
     const int variant = tuning("sgemm.variant");
     if (variant <= 0 && tuning("sgemm.split_rows") != 1 && k >= 512) {

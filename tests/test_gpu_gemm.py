@@ -31,7 +31,8 @@ def gemm16_variant(ko, request):
 
 @pytest.mark.parametrize("sgemm_variant", SGEMM_VARIANTS, indirect=True)
 @pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 256, 96), (200, 136, 40), (1, 4, 4), (65, 129, 33),
-                                   (37, 50, 7), (128, 256, 128), (256, 128, 384)])
+                                   (37, 50, 7), (128, 256, 128), (256, 128, 384), (200, 136, 264), (130, 260, 128),
+                                   (61, 68, 520)])
 def test_sgemm_matches_oracle(ko, sgemm_variant, m, n, k):
     A = inputs.uniform_f32((m, k), 11 + m)
     B = inputs.uniform_f32((k, n), 13 + n)
@@ -40,7 +41,8 @@ def test_sgemm_matches_oracle(ko, sgemm_variant, m, n, k):
 
 
 @pytest.mark.parametrize("sgemm_variant", SGEMM_PIPELINED, indirect=True)
-@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (512, 384, 512), (256, 640, 1152), (1024, 1024, 256), (512, 256, 96)])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (512, 384, 512), (256, 640, 1152), (1024, 1024, 256), (512, 256, 96),
+                                   (300, 520, 392), (1000, 1000, 1000)])
 def test_sgemm_pipelined_variants_are_exact_on_small_integers(ko, sgemm_variant, m, n, k):
     """Full tiles and an even number of K tiles put the pipelined kernels (register staging or direct-to-LDS
     loads, two to four LDS stages) on their fast path; with small integers every product and sum is exact, so
