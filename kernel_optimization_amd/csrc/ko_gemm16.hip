@@ -1178,19 +1178,25 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // multiple of 128), else as the register pipeline.
         // Fewer: smaller tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
-        // A last round of a few big tiles costs a whole round: the tile rows that fill whole rounds go out as
-        // one launch, the rows below them as a second one with the tiling their own size asks for.  Pays while
-        // the rows below hold at most a sixth of a round (4352 x 4096 x 1024, 272 tiles on 256 compute units:
-        // 52.7 -> 42.7 us; 8192 x 2304 x 768, 288 tiles: 41.1 -> 37.4 us; with 65 or 72 tiles below the cut the
-        // small tilings take as long as the round they replace).
+        // Two reasons to send the last rows out as a launch of their own, with the tiling their size asks for:
+        // rows that do not fill the last row of big tiles would take the whole problem off the pinned kernel
+        // (16000 x 3072 x 768: 123 us, against 78 us as 15872 + 128 rows), and a last round of a few big
+        // tiles costs a whole round - that one pays while the rows cut off hold at most a sixth of a round
+        // (4352 x 4096 x 1024, 272 tiles on 256 compute units: 52.7 -> 42.7 us; 8192 x 2304 x 768, 288 tiles:
+        // 41.1 -> 37.4 us; with 65 or 72 tiles below the cut the small tilings take as long as the round they
+        // replace).
         if (tuning("gemm16.split_rows") != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
-            const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
-            const int64_t rounds = big_tiles / cu;
-            const int64_t rows1 = rounds * cu / tn;     // whole tile rows within the full rounds
-            const int64_t below = (tm - rows1) * tn;    // big tiles left for the second launch
-            if (rounds >= 1 && rows1 >= 1 && rows1 < tm && big_tiles % cu != 0 && 6 * below <= cu) {
-                const int64_t m1 = rows1 * 256;
+            const int64_t tn = (p.N + 255) / 256;
+            const bool pinned_ok = p.N % 256 == 0 && p.K % (2 * kBK) == 0;
+            int64_t rows_top = p.M % 256 != 0 && pinned_ok ? p.M / 256 : (p.M + 255) / 256;  // in tile rows
+            const int64_t tiles = rows_top * tn, rounds = tiles / cu;
+            if (rounds >= 1 && tiles % cu != 0) {
+                const int64_t rows1 = rounds * cu / tn;  // whole tile rows within the full rounds
+                if (rows1 >= 1 && 6 * (rows_top - rows1) * tn <= cu) rows_top = rows1;
+            }
+            if (rows_top * 256 < p.M && 2 * rows_top * tn >= cu) {
+                const int64_t m1 = rows_top * 256;
                 Params top = p, bottom = p;
                 top.M = static_cast<int>(m1);
                 bottom.M = p.M - static_cast<int>(m1);

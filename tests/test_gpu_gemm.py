@@ -220,7 +220,8 @@ def test_gemm16_default_path_big(ko, bf16, k):
 
 
 @pytest.mark.parametrize("b_col_major", [True, False])
-@pytest.mark.parametrize("m,n", [(4096, 3072), (2048, 4096), (3072, 2816), (2048, 2048), (1024, 1536), (4352, 4096)])
+@pytest.mark.parametrize("m,n", [(4096, 3072), (2048, 4096), (3072, 2816), (2048, 2048), (1024, 1536), (4352, 4096),
+                                 (4136, 2048)])
 def test_gemm16_default_path_partly_filled_chip(ko, m, n, b_col_major):
     """Between half a chip's and a chip's worth of 256 x 256 tiles (192, 128 and 132 of them): the default dispatch
     still takes the pinned kernel, with fewer workgroups than compute units and, for 132 tiles, a grid that is not a
@@ -233,7 +234,9 @@ def test_gemm16_default_path_partly_filled_chip(ko, m, n, b_col_major):
     got = ko.gemm16_host(A, B, m, n, k, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
     idx = np.random.default_rng(5).choice(m, 64, replace=False)
     # 272 tiles go out as two launches (tile rows 0..15, then the last 256 rows): both sides of the cut
-    idx = np.unique(np.concatenate([idx, [0, m - 257, m - 256, m - 255, m - 1]]))
+    # 4136 rows: the 4096 rows of full tiles on the pinned kernel, the last 40 as a launch of their own
+    idx = np.unique(np.concatenate([idx, [0, m - 257, m - 256, m - 255, m - 1, m // 256 * 256 - 1,
+                                          min(m // 256 * 256, m - 1)]]))
     _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, b_col_major=b_col_major)
     assert_gemm16_close(_to_f64(got[idx], False), ref64, ap, k)
 
