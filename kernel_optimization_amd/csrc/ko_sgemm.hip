@@ -684,8 +684,10 @@ int run(Params p, hipStream_t s, int variant) {
         // at 4096^3; shallower K loses more to the larger first tile than it gains).
         const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
         const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64);
-        variant = t128 >= compute_units() ? (k >= 2048 && k % 128 == 0 ? 40 : 36)
-                                           : (2 * t64 <= compute_units() ? 41 : (k % 256 == 0 ? 35 : 33));
+        // K is padded up to a pair of K tiles: the deeper step is taken where its padding costs less than it gains.
+        const int64_t k_pad128 = (k + 127) / 128 * 128, k_pad256 = (k + 255) / 256 * 256;
+        variant = t128 >= compute_units() ? (k >= 2048 ? 40 : 36)
+                                           : (2 * t64 <= compute_units() ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
     }
     switch (variant) {
         case 1: return launch<64, 64, 32, 2, 2, 1>(p, s);
