@@ -409,8 +409,7 @@ __device__ __attribute__((aligned(16))) const float zero_chunk[4] = {0.0f, 0.0f,
 // waits are inline assembly.  Registers filled by such a read pass through an empty assembly statement
 // behind the wait before the MFMAs use them, which keeps every use (and every copy) behind the wait.
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, bool EDGE>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT)
-__attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(const Params p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_kernel(const Params p) {
     constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -425,7 +424,7 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     constexpr int GROUPS = KGROUPS / KSPLIT;
     constexpr int STAGE_BYTES = CHUNKS * 16;
     static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "a wave-level load stays inside A or B");
-    static_assert(KGROUPS % KSPLIT == 0 && (BK == 16 || BK == 32 || BK == 64 || BK == 128) && BN % 64 == 0 && NSTAGE >= 2, "");
+    static_assert(KGROUPS % KSPLIT == 0 && (BK == 32 || BK == 64 || BK == 128) && BN % 64 == 0 && NSTAGE >= 2, "");
     static_assert((NSTAGE - 1) * LOADS < 64 && BK * BN * 4 < 65536 && TM * 32 * A_ROW_CHUNKS * 16 < 65536, "");
     typedef const __attribute__((address_space(1))) void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
@@ -445,9 +444,9 @@ __attribute__((amdgpu_waves_per_eu(BK == 16 ? 4 : 1))) void sgemm_direct_kernel(
     // EDGE: K (a multiple of 4) is padded with zeros up to the next pair of K tiles.
     const int KT = EDGE ? 2 * ((K + 2 * BK - 1) / (2 * BK)) : K / BK;
 
-    // A rows of 256 bytes fill a line of the 64 banks; of 128 (64) bytes two (four) rows share one, and
-    // the number of the row pair (quadruple) goes into the swizzle.
-    auto swz_a = [](int row) { return BK == 16 ? (row >> 2) & 3 : BK == 32 ? (row >> 1) & 7 : row & 15; };
+    // A rows of 256 bytes or more fill lines of the 64 banks; of 128 bytes two rows share one, and the
+    // number of the row pair goes into the swizzle.
+    auto swz_a = [](int row) { return BK == 32 ? (row >> 1) & 7 : row & 15; };
     auto swz_b = [](int k) { return ((k >> 2) & 1) << 3; };
 
     // What this thread fetches with each of its loads: LDS slot tid + i * THREADS of the stage, K tile 0.
@@ -690,33 +689,13 @@ int run(Params p, hipStream_t s, int variant) {
                                            : (2 * t64 <= compute_units() ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
     }
     switch (variant) {
-        case 1: return launch<64, 64, 32, 2, 2, 1>(p, s);
-        case 2: return launch<128, 64, 32, 2, 2, 1>(p, s);
-        case 3: return launch<128, 128, 32, 2, 2, 1>(p, s);
-        case 4: return launch<64, 64, 32, 1, 1, 1>(p, s);
-        case 5: return launch<64, 128, 32, 2, 2, 1>(p, s);
-        case 6: return launch<64, 64, 32, 2, 2, 2>(p, s);
-        case 7: return launch<64, 64, 32, 2, 2, 4>(p, s);
-        case 8: return launch<64, 64, 64, 2, 2, 2>(p, s);
-        case 9: return launch<64, 64, 64, 2, 2, 4>(p, s);
-        case 10: return launch<128, 128, 32, 2, 2, 2>(p, s);
-        case 11: return launch<128, 64, 32, 2, 2, 2>(p, s);
-        case 12: return launch<64, 64, 64, 2, 2, 2, true>(p, s);
         case 13: return launch<64, 64, 64, 2, 2, 4, true>(p, s);
-        case 14: return launch<64, 64, 32, 2, 2, 4, true>(p, s);
-        case 15: return launch<64, 64, 32, 2, 2, 2, true>(p, s);
         case 16: return launch<128, 128, 32, 2, 2, 2, true>(p, s);
-        case 17: return launch<128, 128, 32, 2, 2, 1, true>(p, s);
-        case 18: return launch<128, 64, 32, 2, 2, 2, true>(p, s);
-        case 19: return launch<128, 64, 64, 2, 2, 2, true>(p, s);
         case 21: return launch<32, 64, 64, 1, 2, 4, true>(p, s);
         case 33: return launch_direct<64, 64, 64, 2, 2, 4, 3>(p, s);
-        case 34: return launch_direct<64, 64, 64, 2, 2, 4, 4>(p, s);
         case 35: return launch_direct<64, 64, 128, 2, 2, 4, 2, 64>(p, s);
         case 36: return launch_direct<128, 128, 32, 2, 2, 2, 2>(p, s);
         case 37: return launch_direct<128, 128, 32, 2, 2, 2, 3>(p, s);
-        case 38: return launch_direct<128, 128, 16, 2, 2, 2, 3, 32>(p, s);
-        case 39: return launch_direct<128, 128, 16, 2, 2, 2, 4, 32>(p, s);
         case 40: return launch_direct<128, 128, 64, 2, 2, 2, 2, 32>(p, s);
         case 41: return launch_direct<32, 64, 64, 1, 2, 4, 3>(p, s);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: unknown variant %d", variant);
