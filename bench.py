@@ -156,11 +156,13 @@ def bench_layernorm(cfg, steps, warmup):
     return res, None
 
 
-def bench_sgemm(cfg, steps, warmup, vendor):
+def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
+    """Configuration 3, or with shape = (m, n, k) the same operator on a shape that does not fill its tiles."""
     c = inputs.CONFIGS[cfg]
-    m, n, k = c["m"], c["n"], c["k"]
-    flops = inputs.algorithmic_work(cfg)
-    nsets = 32  # 12 MB per set: rotate through 400 MB
+    m, n, k = shape or (c["m"], c["n"], c["k"])
+    flops = 2 * m * n * k
+    nsets = 32 if shape is None else 2  # 12 MB per set: rotate through 400 MB (192 MB per set at 4000^3)
+    wname = c["name"] if shape is None else "sgemm_f32_%dx%dx%d" % (m, n, k)
     As = [ko.DeviceBuffer(m * k * 4) for _ in range(nsets)]
     Bs = [ko.DeviceBuffer(k * n * 4) for _ in range(nsets)]
     Ds = [ko.DeviceBuffer(m * n * 4) for _ in range(nsets)]
@@ -168,10 +170,10 @@ def bench_sgemm(cfg, steps, warmup, vendor):
         ko.fill_uniform_f32(a, m * k, inputs.tensor_seed(cfg, 0))
         ko.fill_uniform_f32(b, k * n, inputs.tensor_seed(cfg, 1))
     wall, dev = _time_steps(lambda i: ko.sgemm(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
-    res = dict(workload=c["name"], metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
+    res = dict(workload=wname, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
                roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f32"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=_traffic(c["name"])),
+                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=_traffic(wname)),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -187,12 +189,12 @@ def bench_sgemm(cfg, steps, warmup, vendor):
     return res, None
 
 
-def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False):
+def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
     """Configuration 4 (B column-major, both operands K-contiguous) or, with b_row_major, the same product with B
     handed over as [K][N], the layout of the reference's own tensor-core kernel (tensor_core_gemm.h:178)."""
     c = inputs.CONFIGS[cfg]
-    m, n, k = c["m"], c["n"], c["k"]
-    flops = inputs.algorithmic_work(cfg)
+    m, n, k = shape or (c["m"], c["n"], c["k"])  # shape: the same operator on a row count that does not fill its tiles
+    flops = 2 * m * n * k
     nsets = 4  # 130 MB per set
     As = [ko.DeviceBuffer(m * k * 2) for _ in range(nsets)]
     Bs = [ko.DeviceBuffer(k * n * 2) for _ in range(nsets)]
@@ -203,7 +205,9 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False):
     layout = ko.ROW_MAJOR if b_row_major else ko.COL_MAJOR
     wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets], b_layout=layout),
                             steps, warmup)
-    name = c["name"].replace("gemm_f16_", "gemm_f16_rowmajorB_") if b_row_major else c["name"]
+    name = c["name"] if shape is None else "gemm_f16_%dx%dx%d" % (m, n, k)
+    if b_row_major:
+        name = name.replace("gemm_f16_", "gemm_f16_rowmajorB_")
     res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
                roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
@@ -451,6 +455,14 @@ def main():
             res["steps"], res["warmup"] = args.steps, args.warmup
             others.append(res)
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, b_row_major=True)
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
+        # shapes that do not fill their tiles: fp32 4000^3 (edge form of the kernel), 16-bit with 16000 rows (the
+        # last 128 rows go out as a launch of their own)
+        res, _ = bench_sgemm(3, args.steps, args.warmup, vendor, shape=(4000, 4000, 4000))
+        res["steps"], res["warmup"] = args.steps, args.warmup
+        others.append(res)
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16000, 3072, 768))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
         res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
