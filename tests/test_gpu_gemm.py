@@ -381,3 +381,33 @@ def test_gemm16_bias_act_errors(ko):
     assert L.ko_gemm_f16f32acc_bias_act(16, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, None, 7, d.ptr, ko.F16, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert L.ko_gemm_f16f32acc_bias_act(16, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, d.ptr + 2, 1, d.ptr, ko.F16, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert L.ko_gemm_f16f32acc_bias_act(0, 16, 16, 1.0, d.ptr, d.ptr, ko.COL_MAJOR, 0.0, None, None, 1, d.ptr, ko.F16, None) == ko.KO_OK
+
+
+def test_sgemm_ragged_shapes_are_exact_on_small_integers(ko):
+    """Shapes that fill neither their tiles nor their K tiles, through the default dispatch (edge form of the
+    direct-to-LDS kernels where operand rows start on 16-byte boundaries): rows past M and columns past N are
+    fetched from clamped addresses and K is padded with zeros, none of which may reach the output.  Small
+    integers make every sum exact."""
+    rng = np.random.default_rng(7)
+    shapes = [(int(rng.integers(1, 3000)), int(rng.integers(1, 750)) * 4, int(rng.integers(1, 500)) * 4) for _ in range(10)]
+    shapes += [(2305, 2048, 516), (4100, 2052, 260), (129, 4, 4), (1, 128, 2048), (3000, 36, 1000), (257, 1028, 132)]
+    for m, n, k in shapes:
+        A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+        B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+        C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+        ref = A.astype(np.float64) @ B.astype(np.float64)
+        np.testing.assert_array_equal(ko.sgemm_host(A, B), ref, err_msg=str((m, n, k)))
+        np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=str((m, n, k)))
+
+
+@pytest.mark.parametrize("m,n,k", [(4136, 2048, 256), (8000, 2304, 768), (4353, 4096, 128)])
+def test_gemm16_ragged_row_counts_whole_output(ko, m, n, k):
+    """Row counts that do not fill the last row of 256 x 256 tiles: the full tile rows run on the pinned kernel,
+    the rest as a launch of its own (8000 x 2304: two cuts, at the last full round and at the last full tile
+    row).  Small integers: the fp32 sums are exact, so the whole output equals the rounded exact product."""
+    rng = np.random.default_rng(m + k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float16)
+    B = rng.integers(-4, 5, (n, k)).astype(np.float16)
+    got = ko.gemm16_host(A.view(np.uint16), B.view(np.uint16), m, n, k).view(np.float16)
+    ref = (A.astype(np.float64) @ B.astype(np.float64).T).astype(np.float16)
+    np.testing.assert_array_equal(got, ref)
