@@ -121,6 +121,7 @@ struct Params {
     int block_cols;
     const uint16_t *bias;       // [N] or null: added to every row before the activation
     int act;                    // KO_ACT_*
+    int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
 };
 
 // x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
@@ -190,6 +191,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                                            int lane, int row0, int col0) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     const int M = p.M, N = p.N;
+    const int64_t ldd = p.ldd;
     const int frow = lane & 31, fhalf = lane >> 5;
     const float alpha = p.alpha;
     const bool use_c = p.C != nullptr && p.beta != 0.0f;
@@ -232,7 +234,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 // C of this 32-row block: all loads first, so that their latencies overlap
                 u32x2 c_q[TN][4];
                 if (use_c) {
-                    const uint16_t *crow = p.C + static_cast<int64_t>(row0 + i * 32 + frow) * N + col0 + 4 * fhalf;
+                    const uint16_t *crow = p.C + (row0 + i * 32 + frow) * ldd + col0 + 4 * fhalf;
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -269,13 +271,13 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int gm = row0 + part * PROWS + row;
                 const int gn = col0 + c * 8;
                 // streaming store: D is written once and not read again by this kernel
-                __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p.D + static_cast<int64_t>(gm) * N + gn));
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p.D + gm * ldd + gn));
             }
         }
         return;
     }
 
-    const bool vec_ok = (N & 3) == 0;
+    const bool vec_ok = (N & 3) == 0 && (ldd & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = row0 + i * 32 + frow;
@@ -286,7 +288,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
             for (int q = 0; q < 4; ++q) {
                 const int n = col0 + j * 32 + 8 * q + 4 * fhalf;
                 if (EDGE && n >= N) continue;
-                const int64_t off = static_cast<int64_t>(m) * N + n;
+                const int64_t off = m * ldd + n;
                 float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                 if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
                     u32x2 c2 = {0, 0}, b2 = {0, 0};
@@ -1185,6 +1187,24 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // (4352 x 4096 x 1024, 272 tiles on 256 compute units: 52.7 -> 42.7 us; 8192 x 2304 x 768, 288 tiles:
         // 41.1 -> 37.4 us; with 65 or 72 tiles below the cut the small tilings take as long as the round they
         // replace).
+        // Columns that do not fill the last column of big tiles (column-major B): the full tile columns go
+        // out on their own - to the pinned kernel when the rest of the shape allows - and the remaining
+        // columns (fewer than 256) as a launch of their own; C and D keep their row stride.
+        if constexpr (!B_ROW_MAJOR) {
+            if (tuning("gemm16.split_rows") != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.K % (2 * kBK) == 0 &&
+                2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
+                const int n1 = p.N - p.N % 256;
+                Params left = p, right = p;
+                left.N = n1;
+                right.N = p.N - n1;
+                right.B = p.B + static_cast<int64_t>(n1) * p.K;
+                right.C = p.C ? p.C + n1 : nullptr;
+                right.D = p.D + n1;
+                right.bias = p.bias ? p.bias + n1 : nullptr;
+                if (const int st = launch_variant<BF16, B_ROW_MAJOR>(left, stream); st != KO_OK) return st;
+                return launch_variant<BF16, B_ROW_MAJOR>(right, stream);
+            }
+        }
         if (tuning("gemm16.split_rows") != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
             const int64_t tn = (p.N + 255) / 256;
@@ -1201,8 +1221,8 @@ int launch_variant(const Params &p, hipStream_t stream) {
                 top.M = static_cast<int>(m1);
                 bottom.M = p.M - static_cast<int>(m1);
                 bottom.A = p.A + m1 * p.K;
-                bottom.C = p.C ? p.C + m1 * p.N : nullptr;
-                bottom.D = p.D + m1 * p.N;
+                bottom.C = p.C ? p.C + m1 * p.ldd : nullptr;
+                bottom.D = p.D + m1 * p.ldd;
                 if (const int st = launch_variant<BF16, B_ROW_MAJOR>(top, stream); st != KO_OK) return st;
                 return launch_variant<BF16, B_ROW_MAJOR>(bottom, stream);
             }
@@ -1269,7 +1289,7 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
              static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0,
-             static_cast<const uint16_t *>(bias), activation};
+             static_cast<const uint16_t *>(bias), activation, static_cast<int>(n)};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);
