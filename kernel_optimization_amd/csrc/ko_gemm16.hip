@@ -122,6 +122,7 @@ struct Params {
     const uint16_t *bias;       // [N] or null: added to every row before the activation
     int act;                    // KO_ACT_*
     int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
+    int ldb;                    // row-major B: elements between its rows (N, or more likewise)
 };
 
 // x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
@@ -447,8 +448,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
                 const int gn = n0 + c * 8;
                 u32x4 v = {0u, 0u, 0u, 0u};
                 if (!EDGE || gk < K) {
-                    const uint16_t *src = p.B + static_cast<int64_t>(gk) * N + gn;
-                    if (!EDGE || (gn + 8 <= N && (N & 7) == 0)) {
+                    const uint16_t *src = p.B + static_cast<int64_t>(gk) * p.ldb + gn;
+                    if (!EDGE || (gn + 8 <= N && (p.ldb & 7) == 0)) {
                         v = *reinterpret_cast<const u32x4 *>(src);
                     } else {
                         uint16_t t[8];
@@ -807,7 +808,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     uint32_t lane_off_b = lane_off;
     if constexpr (B_ROW) {
         const int r = lane >> 5;
-        lane_off_b = static_cast<uint32_t>(r * p.N + 8 * ((lane & 31) ^ ((2 * (wave & 1) + r) << 2))) * 2u;
+        lane_off_b = static_cast<uint32_t>(r * p.ldb + 8 * ((lane & 31) ^ ((2 * (wave & 1) + r) << 2))) * 2u;
     }
 
     typedef const __attribute__((address_space(1))) void *gptr_t;
@@ -830,13 +831,13 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         int m0, n0;
         tile_origin(ld_t, m0, n0);
         cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
-        if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(2 * wave) * p.N + n0);
+        if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(2 * wave) * p.ldb + n0);
         else cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
     };
     set_cursor();
     const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
-    const int64_t group_stride_b = B_ROW ? static_cast<int64_t>(2 * WAVES) * p.N * 2 : group_stride;
-    const int64_t ktile_step_b = B_ROW ? static_cast<int64_t>(kBK) * p.N * 2 : kBK * 2;  // bytes from a K tile to the next
+    const int64_t group_stride_b = B_ROW ? static_cast<int64_t>(2 * WAVES) * p.ldb * 2 : group_stride;
+    const int64_t ktile_step_b = B_ROW ? static_cast<int64_t>(kBK) * p.ldb * 2 : kBK * 2;  // bytes from a K tile to the next
     auto advance_cursor = [&]() {
         if (ld_kt + 1 < KT) {
             ++ld_kt;
@@ -1187,23 +1188,21 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // (4352 x 4096 x 1024, 272 tiles on 256 compute units: 52.7 -> 42.7 us; 8192 x 2304 x 768, 288 tiles:
         // 41.1 -> 37.4 us; with 65 or 72 tiles below the cut the small tilings take as long as the round they
         // replace).
-        // Columns that do not fill the last column of big tiles (column-major B): the full tile columns go
-        // out on their own - to the pinned kernel when the rest of the shape allows - and the remaining
-        // columns (fewer than 256) as a launch of their own; C and D keep their row stride.
-        if constexpr (!B_ROW_MAJOR) {
-            if (tuning("gemm16.split_rows") != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.K % (2 * kBK) == 0 &&
-                2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
-                const int n1 = p.N - p.N % 256;
-                Params left = p, right = p;
-                left.N = n1;
-                right.N = p.N - n1;
-                right.B = p.B + static_cast<int64_t>(n1) * p.K;
-                right.C = p.C ? p.C + n1 : nullptr;
-                right.D = p.D + n1;
-                right.bias = p.bias ? p.bias + n1 : nullptr;
-                if (const int st = launch_variant<BF16, B_ROW_MAJOR>(left, stream); st != KO_OK) return st;
-                return launch_variant<BF16, B_ROW_MAJOR>(right, stream);
-            }
+        // Columns that do not fill the last column of big tiles: the full tile columns go out on their own -
+        // to the pinned kernel when the rest of the shape allows - and the remaining columns (fewer than 256)
+        // as a launch of their own; C, D and a row-major B keep their row strides.
+        if (tuning("gemm16.split_rows") != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.ldb % 8 == 0 &&
+            p.K % (2 * kBK) == 0 && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
+            const int n1 = p.N - p.N % 256;
+            Params left = p, right = p;
+            left.N = n1;
+            right.N = p.N - n1;
+            right.B = B_ROW_MAJOR ? p.B + n1 : p.B + static_cast<int64_t>(n1) * p.K;
+            right.C = p.C ? p.C + n1 : nullptr;
+            right.D = p.D + n1;
+            right.bias = p.bias ? p.bias + n1 : nullptr;
+            if (const int st = launch_variant<BF16, B_ROW_MAJOR>(left, stream); st != KO_OK) return st;
+            return launch_variant<BF16, B_ROW_MAJOR>(right, stream);
         }
         if (tuning("gemm16.split_rows") != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
@@ -1289,7 +1288,7 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
              static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0,
-             static_cast<const uint16_t *>(bias), activation, static_cast<int>(n)};
+             static_cast<const uint16_t *>(bias), activation, static_cast<int>(n), static_cast<int>(n)};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);

@@ -413,11 +413,12 @@ def test_gemm16_ragged_row_counts_whole_output(ko, m, n, k):
     np.testing.assert_array_equal(got, ref)
 
 
+@pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k", [(4096, 2200, 256), (4136, 2312, 128), (8192, 1288, 384)])
-def test_gemm16_ragged_column_counts_whole_output(ko, m, n, k):
-    """Column counts (multiples of 8) that do not fill the last column of 256 x 256 tiles, column-major B: the full
+def test_gemm16_ragged_column_counts_whole_output(ko, m, n, k, b_col_major):
+    """Column counts (multiples of 8) that do not fill the last column of 256 x 256 tiles, both layouts of B: the full
     tile columns and the remaining ones are separate launches that write column ranges of the same D (row stride
-    n), each with its part of B, C and the bias.  With 4136 rows the full-tile part is cut along the rows as well.
+    n), each with its part of B (a row-major B keeps its row stride too), C and the bias.  With 4136 rows the full-tile part is cut along the rows as well.
     Small integers: every fp32 sum is exact, so the whole output equals the rounded exact result."""
     rng = np.random.default_rng(n + k)
     A = rng.integers(-4, 5, (m, k)).astype(np.float16)
@@ -425,8 +426,10 @@ def test_gemm16_ragged_column_counts_whole_output(ko, m, n, k):
     C = rng.integers(-8, 9, (m, n)).astype(np.float16)
     bias = rng.integers(-8, 9, (n,)).astype(np.float16)
     exact = A.astype(np.float64) @ B.astype(np.float64).T
-    got = ko.gemm16_host(A.view(np.uint16), B.view(np.uint16), m, n, k).view(np.float16)
+    Bm = B if b_col_major else np.ascontiguousarray(B.T)
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    got = ko.gemm16_host(A.view(np.uint16), Bm.view(np.uint16), m, n, k, b_layout=layout).view(np.float16)
     np.testing.assert_array_equal(got, exact.astype(np.float16))
-    got = ko.gemm16_host(A.view(np.uint16), B.view(np.uint16), m, n, k, C_bits=C.view(np.uint16), alpha=1.0, beta=2.0,
-                         bias_bits=bias.view(np.uint16)).view(np.float16)
+    got = ko.gemm16_host(A.view(np.uint16), Bm.view(np.uint16), m, n, k, C_bits=C.view(np.uint16), alpha=1.0, beta=2.0,
+                         b_layout=layout, bias_bits=bias.view(np.uint16)).view(np.float16)
     np.testing.assert_array_equal(got, (exact + 2.0 * C.astype(np.float64) + bias.astype(np.float64)).astype(np.float16))
