@@ -47,6 +47,10 @@ def test_operators_replay_from_a_hip_graph(ko):
     a32, b32, d32 = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
     m2, n2, k2 = 4096, 2048, 256  # 128 tiles of 256 x 256: the persistent direct-to-LDS kernel
     a2, b2, d2 = ko.DeviceBuffer(m2 * k2 * 2), ko.DeviceBuffer(n2 * k2 * 2), ko.DeviceBuffer(m2 * n2 * 2)
+    m3, n3, k3 = 4136, 2200, 128  # cut along rows and columns: four launches behind one call
+    a3, b3, d3 = ko.DeviceBuffer(m3 * k3 * 2), ko.DeviceBuffer(n3 * k3 * 2), ko.DeviceBuffer(m3 * n3 * 2)
+    ko.fill_uniform_16(a3, m3 * k3, 509)
+    ko.fill_uniform_16(b3, n3 * k3, 510)
     ko.fill_uniform_16(a2, m2 * k2, 507)
     ko.fill_uniform_16(b2, n2 * k2, 508)
     ko.fill_uniform_16(a16, m * k, 503)
@@ -61,14 +65,16 @@ def test_operators_replay_from_a_hip_graph(ko):
         ko.gemm16(m, n, k, a16, b16, d16, stream=stream)
         ko.sgemm(m, n, k, a32, b32, d32, stream=stream)
         ko.gemm16(m2, n2, k2, a2, b2, d2, stream=stream)
+        ko.gemm16(m3, n3, k3, a3, b3, d3, stream=stream)
 
     def outputs():
         return (dl.download(np.uint32, (rows, cols)), dmean.download(np.uint32, (rows,)),
-                d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)))
+                d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)),
+                d3.download(np.uint16, (m3, n3)))
 
     def clear():
         for buf, nbytes in ((ds, rows * cols * 4), (dl, rows * cols * 4), (dmean, rows * 4), (d16, m * n * 2), (d32, m * n * 4),
-                            (d2, m2 * n2 * 2)):
+                            (d2, m2 * n2 * 2), (d3, m3 * n3 * 2)):
             buf.upload(np.zeros(nbytes, np.uint8))
 
     chain()
