@@ -685,8 +685,14 @@ int run(Params p, hipStream_t s, int variant) {
         const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64);
         // K is padded up to a pair of K tiles: the deeper step is taken where its padding costs less than it gains.
         const int64_t k_pad128 = (k + 127) / 128 * 128, k_pad256 = (k + 255) / 256 * 256;
-        variant = t128 >= compute_units() ? (k >= 2048 ? 40 : 36)
-                                           : (2 * t64 <= compute_units() ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
+        // A round of 64 x 64 tiles takes 0.29-0.31 of the time of a round of 128 x 128 tiles (2048 x 3072 x 1024:
+        // 19 us against 62 us; K = 2048: 35 against 121): the big tiles do the same work in 0.8 of the time
+        // when their rounds are full, but one and a half rounds of them cost two (384 tiles on 256 compute
+        // units: 125 us, as 1536 small tiles in six rounds 114 us).
+        const int64_t cu = compute_units();
+        const bool big = t128 >= cu && 97 * ((t128 + cu - 1) / cu) <= 31 * ((t64 + cu - 1) / cu);
+        variant = big ? (k >= 2048 ? 40 : 36)
+                      : (2 * t64 <= cu ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
     }
     switch (variant) {
         case 13: return launch<64, 64, 64, 2, 2, 4, true>(p, s);
