@@ -34,14 +34,27 @@ WORKLOADS = {c["name"]: k for k, c in inputs.CONFIGS.items()}
 HEADLINE = 5
 
 
-def _traffic(name):
-    """HBM bytes per launch measured offline with rocprofv3 --pmc (profiles/hbm_traffic.json), or None."""
+def _traffic_table():
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(name, {}).get("traffic_bytes")
+            return json.load(f)
     except (OSError, ValueError):
-        return None
+        return {}
+
+
+def _traffic(name):
+    """HBM bytes per launch measured offline with rocprofv3 --pmc (profiles/hbm_traffic.json), or None.  The
+    counters cannot be read from inside this process, so the figure is the one of the profiled commit."""
+    return _traffic_table().get(name, {}).get("traffic_bytes")
+
+
+def _roofline(bound, achieved, peak, unit, name):
+    roof = dict(bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak, traffic=_traffic(name))
+    if roof["traffic"] is not None:
+        roof["traffic_source"] = "profiles/hbm_traffic.json @ %s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE)" % \
+            _traffic_table().get("_measured_at_commit", "unknown commit")
+    return roof
 
 
 SECONDARY_MIN_WARMUP = 300
@@ -80,6 +93,8 @@ def _vendor():
                                             ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ci)]
     V.kov_sgemm_sets.argtypes = [i64, i64, i64, pp, pp, pp, ci, ci, ci, ctypes.POINTER(ctypes.c_float),
                                  ctypes.POINTER(ci)]
+    if hasattr(V, "kov_rocblas_sgemm_sets"):
+        V.kov_rocblas_sgemm_sets.argtypes = [i64, i64, i64, pp, pp, pp, ci, ci, ctypes.POINTER(ctypes.c_float)]
     return V
 
 
@@ -103,8 +118,14 @@ def _add_copy_floor(res, floor_us):
     res["vs_copy_same_bytes"] = floor_us / res["kernel_us"]
 
 
-def bench_softmax(cfg, steps, warmup):
-    c = inputs.CONFIGS[cfg]
+def bench_softmax(cfg, steps, warmup, unmasked=False):
+    """Configurations 1 and 5.  unmasked: the shape of the masked configuration without its mask, so that every
+    algorithmic byte really moves (with the mask a third of the reads is skipped)."""
+    c = dict(inputs.CONFIGS[cfg])
+    if unmasked:
+        c["name"] = c["name"].replace("masked_", "") + "_unmasked"
+        for key in ("n_seq", "rows_per_seq", "len_lo", "len_hi"):
+            c.pop(key, None)
     rows, cols = c["rows"], c["cols"]
     n = rows * cols
     work = inputs.algorithmic_work(cfg)
@@ -121,8 +142,7 @@ def bench_softmax(cfg, steps, warmup):
     wall, dev = _time_steps(lambda i: ko.softmax(xs[i % nsets], ys[i % nsets], rows, cols, vl, rps), steps, warmup)
     res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"]),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
     keep = dict(x=xs[0], y=ys[0], vl=vl, rows=rows, cols=cols, rps=rps)
@@ -149,11 +169,11 @@ def bench_layernorm(cfg, steps, warmup):
                                                    rs[i % nsets], g, b, c["eps"]), steps, warmup)
     res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=_traffic(c["name"])),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"]),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
-    return res, None
+    keep = dict(x=xs[0], y=ys[0], mean=ms[0], rstd=rs[0], g=g, b=b, rows=rows, cols=cols, eps=c["eps"])
+    return res, keep
 
 
 def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
@@ -172,8 +192,7 @@ def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
     wall, dev = _time_steps(lambda i: ko.sgemm(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
     res = dict(workload=wname, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f32"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f32"], traffic=_traffic(wname)),
+               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f32"], "TFLOP/s", wname),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -186,7 +205,15 @@ def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
             res["vs_hipblaslt"] = (flops / dev / 1e12) / res["hipblaslt_tflops"]
             ref = tmp.download(np.float32, (m, n))
             res["max_abs_diff_vs_hipblaslt"] = float(np.abs(Ds[0].download(np.float32, (m, n)) - ref).max())
-    return res, None
+        # rocblas_sgemm: the call-for-call counterpart of the reference's cublasSgemm check (gemm/main.cu:146-150)
+        if hasattr(vendor, "kov_rocblas_sgemm_sets") and vendor.kov_rocblas_sgemm_sets(
+                m, n, k, _ptr_array(As), _ptr_array(Bs), _ptr_array(Vs), nsets, 2 * nsets, ctypes.byref(us)) == 0:
+            res["rocblas_tflops"] = flops / us.value / 1e6
+            res["vs_rocblas"] = (flops / dev / 1e12) / res["rocblas_tflops"]
+            ref = tmp.download(np.float32, (m, n))
+            res["max_abs_diff_vs_rocblas"] = float(np.abs(Ds[0].download(np.float32, (m, n)) - ref).max())
+    keep = dict(A=As[0], B=Bs[0], D=Ds[0], m=m, n=n, k=k) if shape is None else None
+    return res, keep
 
 
 def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
@@ -210,8 +237,7 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
         name = name.replace("gemm_f16_", "gemm_f16_rowmajorB_")
     res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
-               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=_traffic(name)),
+               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", name),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -224,7 +250,8 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
             ref = tmp.download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
             got = Ds[0].download(np.uint16, (m, n)).view(np.float16).astype(np.float32)
             res["max_abs_diff_vs_hipblaslt"] = float(np.abs(got - ref).max())
-    return res, None
+    keep = dict(A=As[0], B=Bs[0], D=Ds[0], m=m, n=n, k=k, b_row_major=b_row_major) if shape is None else None
+    return res, keep
 
 
 def bench_gemm16_bias_gelu(steps, warmup, vendor):
@@ -244,10 +271,10 @@ def bench_gemm16_bias_gelu(steps, warmup, vendor):
         ko.fill_uniform_16(b, k * n, inputs.tensor_seed(4, 1))
     wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets], bias=bias,
                                                 act=ko.ACT_GELU_TANH), steps, warmup)
-    res = dict(workload="gemm_f16_bias_gelu_%dx%dx%d" % (m, n, k), metric="tflops", unit="TFLOP/s",
+    res_name = "gemm_f16_bias_gelu_%dx%dx%d" % (m, n, k)
+    res = dict(workload=res_name, metric="tflops", unit="TFLOP/s",
                value=flops / wall / 1e12, ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
-               roofline=dict(bound="mfma", achieved=flops / dev / 1e12, peak=MFMA_PEAK_TFLOPS["f16"], unit="TFLOP/s",
-                             frac=flops / dev / 1e12 / MFMA_PEAK_TFLOPS["f16"], traffic=None),
+               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", res_name),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -300,10 +327,10 @@ def bench_long_rows(op, rows, cols, policy, steps, warmup):
         launch = lambda i: ko.layernorm(xs[i % nsets], ys[i % nsets], rows, cols, m, r, g, b, 1e-5, False, policy)
     wall, dev = _time_steps(launch, steps, warmup)
     names = {ko.POLICY_AUTO: "auto", ko.POLICY_WARP: "warp", ko.POLICY_BLOCK: "block", ko.POLICY_BLOCK_NOCACHE: "nocache"}
-    res = dict(workload="%s_f32_%dx%d_%s" % (op, rows, cols, names[policy]), metric="hbm_gbytes_per_s", unit="GB/s",
+    res_name = "%s_f32_%dx%d_%s" % (op, rows, cols, names[policy])
+    res = dict(workload=res_name, metric="hbm_gbytes_per_s", unit="GB/s",
                value=work / wall / 1e9, ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
     return res
@@ -343,10 +370,10 @@ def bench_rows16(kind, dtype_name, steps, warmup):
         name = "layernorm_%s_%dx%d" % (dtype_name, rows, cols)
     floor_us = _copy_floor_us(xs, ys, n // 2, steps, warmup)
     wall, dev = _time_steps(launch, steps, warmup)
+    res_name = name
     res = dict(workload=name, metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype=dtype_name + " storage, f32 arithmetic", buffer_sets=nsets,
-               roofline=dict(bound="hbm", achieved=work / dev / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                             frac=work / dev / 1e9 / HBM_PEAK_GBS, traffic=None),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
     return res
@@ -403,6 +430,158 @@ def cpu_baseline_softmax(keep, cfg):
                                    sample="first %d rows, 1 thread, one run" % rows1, seconds=single)), parity
 
 
+def cpu_baseline_layernorm(keep):
+    """The CPU oracle's LayerNorm on the rows the GPU just processed: all host threads, best of 3, and one thread
+    on a sixteenth of the rows; also checks y, mean and rstd of the GPU against it."""
+    import oracle
+    rows, cols = keep["rows"], keep["cols"]
+    x = keep["x"].download(np.float32, (rows, cols))
+    g, b = keep["g"].download(np.float32, (cols,)), keep["b"].download(np.float32, (cols,))
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ry, rm, rr = oracle.layernorm(x, g, b, eps=keep["eps"])
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    nthreads = oracle.max_threads()
+    rows1 = max(1, rows // 16)
+    oracle.set_threads(1)
+    t0 = time.perf_counter()
+    oracle.layernorm(x[:rows1], g, b, eps=keep["eps"])
+    single = time.perf_counter() - t0
+    oracle.set_threads(nthreads)
+    y = keep["y"].download(np.float32, (rows, cols)).astype(np.float64)
+    mean = keep["mean"].download(np.float32, (rows,)).astype(np.float64)
+    rstd = keep["rstd"].download(np.float32, (rows,)).astype(np.float64)
+    ey = float((np.abs(y - ry) / np.maximum(np.abs(ry), 1.0)).max())
+    er = float((np.abs(rstd - rr) / rr).max())
+    em = float((np.abs(mean - rm) / np.maximum(np.abs(rm), 1.0 / rr)).max())
+    parity = dict(rows_checked=rows, max_y_err=ey, max_rstd_rel_err=er, max_mean_err=em,
+                  gate="|dy| <= 1e-5 max(|y|, 1); rstd 1e-5 relative; mean 1e-5 of max(|mean|, std)",
+                  ok=bool(ey <= 1e-5 and er <= 1e-5 and em <= 1e-5))
+    work = 2 * rows * cols * 4
+    return dict(value=work / best / 1e9, unit="GB/s", cores=nthreads, kind="port",
+                sample="all %d rows x %d cols, %d threads, best of 3; host cpus visible: %d" % (
+                    rows, cols, nthreads, os.cpu_count() or 0), seconds=best,
+                single_thread=dict(value=2 * rows1 * cols * 4 / single / 1e9, unit="GB/s", cores=1,
+                                   sample="first %d rows, 1 thread, one run" % rows1, seconds=single)), parity
+
+
+def cpu_baseline_sgemm(keep):
+    """The CPU oracle's SGEMM - the reference's commented-out CPU loop (nn_operators/gemm/main.cu:162-167) with a
+    double accumulator - on the same operands, all host threads, best of 3; checks the GPU's D against it."""
+    import oracle
+    m, n, k = keep["m"], keep["n"], keep["k"]
+    A, B = keep["A"].download(np.float32, (m, k)), keep["B"].download(np.float32, (k, n))
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ref, ap = oracle.sgemm(A, B, want_absprod=True)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    d = np.abs(keep["D"].download(np.float32, (m, n)).astype(np.float64) - ref)
+    worst = float((d / (2.0 * k * 2.0 ** -24 * ap + 1e-30)).max())
+    parity = dict(elements_checked=m * n, max_abs_err=float(d.max()), worst_over_bound=worst,
+                  gate="|d| <= 2 K 2^-24 sum|a||b| and |d| <= 1e-3 (gemm/main.cu:169-170)",
+                  ok=bool(worst <= 1.0 and d.max() <= 1e-3))
+    return dict(value=2.0 * m * n * k / best / 1e12, unit="TFLOP/s", cores=oracle.max_threads(), kind="port",
+                sample="the whole %dx%dx%d product, %d threads, best of 3" % (m, n, k, oracle.max_threads()),
+                seconds=best), parity
+
+
+def cpu_baseline_gemm16(keep, sample_rows=1024):
+    """The CPU oracle's 16-bit GEMM on the first `sample_rows` rows of A (the operator is independent per output
+    row; the whole product would take about a minute of host time), all host threads, one run; checks those rows of
+    the GPU's D against it."""
+    import oracle
+    m, n, k = keep["m"], keep["n"], keep["k"]
+    ms = min(m, sample_rows)
+    A = keep["A"].download(np.uint16, (ms, k))
+    B = keep["B"].download(np.uint16, (k, n) if keep["b_row_major"] else (n, k))
+    t0 = time.perf_counter()
+    _, ref64, ap = oracle.gemm16(A, B, ms, n, k, b_col_major=not keep["b_row_major"])
+    dt = time.perf_counter() - t0
+    got = oracle.f16_to_f64(keep["D"].download(np.uint16, (ms, n)))
+    d = np.abs(got - ref64)
+    worst = float((d / (2.0 ** -11 * np.abs(ref64) + k * 2.0 ** -24 * ap + 2.0 ** -24)).max())
+    parity = dict(elements_checked=ms * n, max_abs_err=float(d.max()), worst_over_bound=worst,
+                  gate="|d| <= 2^-11 |ref| + K 2^-24 sum|a||b| + 2^-24", ok=bool(worst <= 1.0))
+    return dict(value=2.0 * ms * n * k / dt / 1e12, unit="TFLOP/s", cores=oracle.max_threads(), kind="port",
+                sample="first %d of %d rows of A (x %d x %d), %d threads, one run" % (ms, m, n, k, oracle.max_threads()),
+                seconds=dt), parity
+
+
+def cpu_baseline(cfg, keep):
+    op = inputs.CONFIGS[cfg]["op"]
+    if op == "softmax":
+        return cpu_baseline_softmax(keep, cfg)
+    if op == "layernorm":
+        return cpu_baseline_layernorm(keep)
+    if op == "sgemm":
+        return cpu_baseline_sgemm(keep)
+    return cpu_baseline_gemm16(keep)
+
+
+# ------------------------------------------------------------------------- streaming ceilings
+
+def _probe_rate(nbytes, moved, launch, steps, warmup):
+    _, dev = _time_steps(launch, steps, warmup)
+    return dict(us=dev * 1e6, gbps=moved / dev / 1e9, frac_of_peak=moved / dev / 1e9 / HBM_PEAK_GBS)
+
+
+def bench_ceilings(steps, warmup, nbytes=1 << 30, full=False):
+    """What a read stream, a write stream and a read+write stream reach on this device, from independent sources
+    in the same run: the runtime's own device-to-device copy and memset, and the streaming probe kernel in the
+    launch shapes that matter (workgroup size, vectors per thread, cache-policy bits of the stores, residency cap).
+    full: the whole sweep (for profiles/), else the handful of shapes that bracket the best."""
+    x, y = ko.DeviceBuffer(nbytes), ko.DeviceBuffer(nbytes)
+    ko.fill_uniform_f32(x, nbytes // 4, 1)
+    out = dict(bytes_per_direction=nbytes, steps=steps, warmup=warmup)
+    out["runtime_memcpy_d2d"] = _probe_rate(nbytes, 2 * nbytes, lambda i: ko.memcpy_d2d(y, x, nbytes), steps, warmup)
+    out["runtime_memset"] = _probe_rate(nbytes, nbytes, lambda i: ko.memset(y, 0, nbytes), steps, warmup)
+    out["copy_f32_kernel"] = _probe_rate(nbytes, 2 * nbytes, lambda i: ko.copy_f32(x, y, nbytes // 4), steps, warmup)
+    rows = []
+
+    def probe(mode, name, moved, **kw):
+        r = _probe_rate(nbytes, moved, lambda i: ko.stream_probe(x, y, nbytes, mode, **kw), steps, warmup)
+        r.update(kind=name, **kw)
+        rows.append(r)
+        return r
+
+    lp, sp = ko.LOAD_POLICIES, ko.STORE_POLICIES
+    threads_list = (64, 128, 256, 512, 1024) if full else (128, 256)
+    vpts = (1, 2, 4) if full else (1, 2)
+    grids = (0, 2, 8) if full else (0,)
+    for t in threads_list:
+        for v in vpts:
+            for g in grids:
+                for l in ((lp["plain"], lp["nt"]) if full else (lp["nt"],)):
+                    probe(ko.PROBE_READ, "read", nbytes, threads=t, vectors_per_thread=v, blocks_per_cu=g, load_policy=l)
+                for st in (sp.values() if full else (sp["nt"], sp["sc1 nt"])):
+                    probe(ko.PROBE_WRITE, "write", nbytes, threads=t, vectors_per_thread=v, blocks_per_cu=g, store_policy=st)
+                    probe(ko.PROBE_COPY, "copy", 2 * nbytes, threads=t, vectors_per_thread=v, blocks_per_cu=g,
+                          load_policy=lp["nt"], store_policy=st)
+                if full:
+                    probe(ko.PROBE_COPY, "copy", 2 * nbytes, threads=t, vectors_per_thread=v, blocks_per_cu=g,
+                          load_policy=lp["plain"], store_policy=sp["plain"])
+    # residency cap: two vectors per thread with all 32 wavefronts of a CU resident, and with 16
+    for pad in ((0, 5120, 10240, 20480, 40960) if full else (0, 10240)):
+        for v in (1, 2, 4):
+            probe(ko.PROBE_COPY, "copy", 2 * nbytes, threads=64, vectors_per_thread=v, load_policy=lp["nt"],
+                  store_policy=sp["sc1 nt"], lds_pad_bytes=pad)
+    # the traffic mix of the masked-softmax configuration: every vector written, 81 of 128 read
+    for t in ((64, 128, 256) if full else (128,)):
+        for st in ((sp["nt"], sp["sc1 nt"]) if full else (sp["sc1 nt"],)):
+            probe(ko.PROBE_PARTIAL, "copy reading 81/128", nbytes + nbytes * 81 // 128, threads=t, vectors_per_thread=1,
+                  load_policy=lp["nt"], store_policy=st, read_of_128=81)
+    for kind in ("read", "write", "copy", "copy reading 81/128"):
+        best = max((r for r in rows if r["kind"] == kind), key=lambda r: r["gbps"])
+        out["best_" + kind.replace(" ", "_").replace("/", "_of_")] = best
+    if full:
+        out["rows"] = rows
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -410,7 +589,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches before the timed ones; the device takes a few hundred short launches "
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
-    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS) + ["copy_f32"])
+    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS) + ["copy_f32", "hbm_ceilings", "softmax_f32_786432x512_unmasked"])
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
     ap.add_argument("--no-all", dest="all", action="store_false")
@@ -426,25 +605,41 @@ def main():
     if args.workload == "copy_f32":  # calibration run for the traffic counters
         print(json.dumps(bench_copy(args.steps, args.warmup)))
         return
+    if args.workload == "hbm_ceilings":  # the whole streaming sweep, for profiles/
+        print(json.dumps(bench_ceilings(min(args.steps, 10), 3, full=True)))
+        return
+    if args.workload == "softmax_f32_786432x512_unmasked":  # for the traffic counters and traces
+        res, _ = bench_softmax(5, args.steps, args.warmup, unmasked=True)
+        print(json.dumps(res))
+        return
     cfg = WORKLOADS[args.workload]
     head, keep = run_workload(cfg, args.steps, args.warmup, vendor)
     cpu, parity = (None, None)
     if not args.no_cpu and keep is not None:
-        cpu, parity = cpu_baseline_softmax(keep, cfg)
+        cpu, parity = cpu_baseline(cfg, keep)
     del keep
 
     others = []
     copy = None
+    ceilings = None
     if args.all:
         copy = bench_copy(args.steps, args.warmup)
+        ceilings = bench_ceilings(min(args.steps, 10), 3)
         for other in sorted(inputs.CONFIGS):
             if other == cfg:
                 continue
             warm = max(args.warmup, SECONDARY_MIN_WARMUP)
             res, k2 = run_workload(other, args.steps, warm, vendor)
+            if not args.no_cpu and k2 is not None:
+                res["cpu_baseline"], res["parity"] = cpu_baseline(other, k2)
             del k2
             res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
+        # the masked configuration's shape without the mask: every algorithmic byte moves
+        res, k2 = bench_softmax(5, args.steps, args.warmup, unmasked=True)
+        del k2
+        res["steps"], res["warmup"] = args.steps, args.warmup
+        others.append(res)
         for op, rows, cols, policy in (("softmax", 49152, 1024, ko.POLICY_WARP), ("softmax", 8192, 16384, ko.POLICY_BLOCK),
                                        ("softmax", 2048, 65536, ko.POLICY_BLOCK),
                                        ("softmax", 1024, 131072, ko.POLICY_BLOCK_NOCACHE),
@@ -484,7 +679,7 @@ def main():
         "roofline": head["roofline"], "cpu_baseline": cpu, "parity": parity,
         "kernel_us": head["kernel_us"], "copy_same_bytes_us": head.get("copy_same_bytes_us"),
         "copy_ceiling": None if copy is None else {"GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"],
-                                                   "workload": copy["workload"]},
+                                                   "workload": copy["workload"], "independent_sources": ceilings},
         "workloads": others,
     }
     for key in ("hipblaslt_tflops", "vs_hipblaslt", "max_abs_diff_vs_hipblaslt"):

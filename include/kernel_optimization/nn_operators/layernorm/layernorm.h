@@ -35,6 +35,11 @@ KO_LAYERNORM_DESCRIPTOR(LayerNormBlockNoCacheImpl, KO_POLICY_BLOCK_NOCACHE, 32 *
 
 // Element = float, half (ko_half) or ko_bfloat16 (storage of in, out, gamma, beta; fp32 arithmetic;
 // mean and rstd are always float).
+// Variance divisor: `unbiased = false` (the default) divides the sum of squared deviations by num_column, what
+// BERT and every framework's LayerNorm compute; `unbiased = true` divides by num_column - 1, which is what
+// the reference's merge is written to do (layernorm.h:48).  A driver ported verbatim from the reference therefore
+// gets the population variance unless it passes `true` here; the two differ by a factor num_column/(num_column-1)
+// in the variance (1.3e-3 at 768 columns).
 template <typename LayerNormKernel>
 void layer_normalization(int grid_dim, int block_dim, int smem_in_bytes, ko_stream_t stream,
                          typename LayerNormKernel::Element *in_data, typename LayerNormKernel::Element *out_data,

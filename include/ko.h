@@ -154,7 +154,8 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * D[m,n] = alpha * A[m,k] * B[k,n] + beta * C[m,n], all row-major fp32.
  * C may be NULL (then beta is ignored); the reference's epilogue is alpha = beta = 1
  * with C given, or D = A*B with C null (simt_gemm.h:325-373).
- * m, n multiples of 4 are not required; any positive sizes are accepted. */
+ * m, n multiples of 4 are not required; any positive sizes are accepted.  m == 0 or n == 0 is a no-op;
+ * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries. */
 int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
                  float beta, const float *C, float *D, ko_stream_t stream);
 
@@ -201,6 +202,17 @@ int ko_fill_lengths_i32(int32_t *out, int64_t n, uint64_t seed, int32_t lo, int3
 /* out[i] = in[i] for n floats, 128-bit accesses: the plain copy whose rate is the
  * practical HBM ceiling the bandwidth kernels are compared with. */
 int ko_copy_f32(const float *in, float *out, int64_t n, ko_stream_t stream);
+/* Streaming-rate probe: one launch that streams `nbytes` (a multiple of threads * vectors_per_thread * 16)
+ * from `in` and/or to `out`: mode 0 write-only, 1 read-only, 2 copy, 3 copy that reads only the vectors whose
+ * index modulo 128 is below `read_of_128` (a 512-column fp32 row with a padded tail) and writes all.
+ * threads: workgroup size (multiple of 64); vectors_per_thread: 1, 2 or 4 16-byte vectors;
+ * blocks_per_cu: 0 = one chunk per workgroup, else a grid of that many workgroups per compute unit walking
+ * the chunks; load_policy: 0 plain, 1 non-temporal; store_policy: 0 plain, 1 nt, 2 sc1, 3 sc1 nt,
+ * 4 sc0 sc1 nt (the cache-policy bits of the store instruction); lds_pad_bytes: dynamic LDS per workgroup,
+ * never touched, which caps how many workgroups are resident per compute unit. */
+int ko_stream_probe(const void *in, void *out, int64_t nbytes, int mode, int vectors_per_thread,
+                    int threads, int blocks_per_cu, int load_policy, int store_policy, int read_of_128,
+                    int lds_pad_bytes, ko_stream_t stream);
 /* Integer tuning knobs by name ("softmax.lanes_per_row", ...); value 0 restores the default.
  * Unknown names return KO_ERR_INVALID_ARGUMENT. */
 int ko_set_tuning(const char *name, int value);

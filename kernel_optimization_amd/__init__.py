@@ -76,6 +76,7 @@ SIGNATURES = {
     "ko_fill_uniform_16": (_int, [_vp, _i64, _u64, _d, _d, _i64, _int, _vp]),
     "ko_fill_lengths_i32": (_int, [_vp, _i64, _u64, ctypes.c_int32, ctypes.c_int32, _vp]),
     "ko_copy_f32": (_int, [_vp, _vp, _i64, _vp]),
+    "ko_stream_probe": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _int, _int, _vp]),
     "ko_set_tuning": (_int, [ctypes.c_char_p, _int]),
     "ko_get_tuning": (_int, [ctypes.c_char_p, ctypes.POINTER(_int)]),
     "ko_debug_wave_allreduce": (_int, [_vp, _vp, _int, _int, _vp]),
@@ -304,6 +305,25 @@ def fill_lengths_i32(out, n, seed, lo, hi, stream=None):
 
 def copy_f32(inp, out, n, stream=None):
     check(lib().ko_copy_f32(_p(inp), _p(out), n, _h(stream)))
+
+
+PROBE_WRITE, PROBE_READ, PROBE_COPY, PROBE_PARTIAL = 0, 1, 2, 3
+LOAD_POLICIES = {"plain": 0, "nt": 1}
+STORE_POLICIES = {"plain": 0, "nt": 1, "sc1": 2, "sc1 nt": 3, "sc0 sc1 nt": 4}
+
+
+def stream_probe(inp, out, nbytes, mode, vectors_per_thread=1, threads=128, blocks_per_cu=0, load_policy=1,
+                 store_policy=3, read_of_128=128, lds_pad_bytes=0, stream=None):
+    check(lib().ko_stream_probe(_p(inp), _p(out), nbytes, mode, vectors_per_thread, threads, blocks_per_cu,
+                                load_policy, store_policy, read_of_128, lds_pad_bytes, _h(stream)))
+
+
+def memcpy_d2d(dst, src, nbytes, stream=None):
+    check(lib().ko_memcpy_d2d_async(_p(dst), _p(src), nbytes, _h(stream)))
+
+
+def memset(dst, value, nbytes, stream=None):
+    check(lib().ko_memset_async(_p(dst), value, nbytes, _h(stream)))
 
 
 # ---- host-array conveniences (upload, run, download): used by tests and examples --------------

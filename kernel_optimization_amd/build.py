@@ -1,7 +1,7 @@
 """Builds the native parts in-tree: libko.so (HIP kernels + C ABI, gfx950) and the
 pure C++ host layer (Tensor, benchmark drivers) that sits on top of the C ABI.
 
-Usage: python -m kernel_optimization_amd.build [--jobs N] [--only lib|host]
+Usage: python -m kernel_optimization_amd.build [--jobs N] [--only lib|host|vendor] [--cmake]
 """
 import argparse
 import concurrent.futures
@@ -63,12 +63,12 @@ def build_lib(jobs=4, verbose=False):
 
 
 def build_vendor(verbose=False):
-    """libko_vendor.so: hipBLASLt timed on the same buffers (comparison harness, not product)."""
+    """libko_vendor.so: hipBLASLt and rocBLAS timed on the same buffers (comparison harness, not product)."""
     os.makedirs(LIB_DIR, exist_ok=True)
     out_path = os.path.join(LIB_DIR, "libko_vendor.so")
     out = _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-x", "hip",
                 f"--offload-arch={ARCH}", os.path.join(PKG, "vendor", "ko_vendor.cpp"), "-o", out_path,
-                "-lhipblaslt"])
+                "-lhipblaslt", "-lrocblas"])
     if verbose and out.strip():
         print(out)
     return out_path
@@ -95,6 +95,20 @@ def build_host(verbose=False):
     return built
 
 
+def build_cmake(jobs=4, verbose=False, targets=()):
+    """The same build through the CMakeLists.txt at the repository root (targets ko, ko_vendor, common, softmax,
+    layernorm, gemm, host_selftest; the names of the reference's CMake tree)."""
+    bdir = os.path.join(OBJ_DIR, "cmake")
+    out = _run(["cmake", "-S", ROOT, "-B", bdir])
+    cmd = ["cmake", "--build", bdir, "-j", str(max(1, jobs))]
+    for t in targets:
+        cmd += ["--target", t]
+    out += _run(cmd)
+    if verbose:
+        print(out)
+    return bdir
+
+
 def build_all(jobs=4, verbose=False):
     lib = build_lib(jobs=jobs, verbose=verbose)
     vendor = build_vendor(verbose=verbose)
@@ -107,7 +121,11 @@ def main(argv=None):
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     ap.add_argument("--only", choices=["lib", "host", "vendor"])
     ap.add_argument("-v", "--verbose", action="store_true")
+    ap.add_argument("--cmake", action="store_true", help="build everything through CMakeLists.txt instead")
     args = ap.parse_args(argv)
+    if args.cmake:
+        print("built with cmake in", build_cmake(args.jobs, args.verbose))
+        return
     if args.only in (None, "lib"):
         print("built", build_lib(args.jobs, args.verbose))
     if args.only in (None, "vendor"):

@@ -1098,7 +1098,7 @@ int launch_pinned(Params p, hipStream_t stream) {
     p.band_rows = 0;
     p.block_cols = 0;
     const int per_xcd = grid / 8;
-    if (tuning("gemm16.mapping") != 1 && grid % 8 == 0 && tiles_m % 8 == 0) {
+    if (tuning(knob_gemm16_mapping) != 1 && grid % 8 == 0 && tiles_m % 8 == 0) {
         const int band = tiles_m / 8;
         if (band <= per_xcd && per_xcd % band == 0 && p.tiles_n % (per_xcd / band) == 0) {
             p.band_rows = band;
@@ -1172,9 +1172,17 @@ int launch_direct(const Params &p, hipStream_t stream) {
     }
 }
 
+// One call becomes at most five launches: one column cut (left, right), then at most two row cuts in the left
+// part (the rows below the last full round, and of those the rows below the last full tile row) and one in the
+// right part.  col_cut / row_cuts are what a (sub-)problem may still spend; the knobs are read once per call.
 template <bool BF16, bool B_ROW_MAJOR>
-int launch_variant(const Params &p, hipStream_t stream) {
-    const int variant = tuning("gemm16.variant");
+int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int row_cuts = 2, int variant = -1,
+                   int split_knob = -1) {
+    if (variant < 0) {
+        variant = tuning(knob_gemm16_variant);
+        split_knob = tuning(knob_gemm16_split_rows);
+        if (variant < 0) variant = 0;
+    }
     if (variant <= 0) {
         // Enough 256x256 tiles to fill the chip: the big tiling - as a persistent direct-to-LDS kernel
         // when the tiles are full and both operands are K-contiguous (the pinned one when K is a
@@ -1191,7 +1199,7 @@ int launch_variant(const Params &p, hipStream_t stream) {
         // Columns that do not fill the last column of big tiles: the full tile columns go out on their own -
         // to the pinned kernel when the rest of the shape allows - and the remaining columns (fewer than 256)
         // as a launch of their own; C, D and a row-major B keep their row strides.
-        if (tuning("gemm16.split_rows") != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.ldb % 8 == 0 &&
+        if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.ldb % 8 == 0 &&
             p.K % (2 * kBK) == 0 && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
             const int n1 = p.N - p.N % 256;
             Params left = p, right = p;
@@ -1201,10 +1209,11 @@ int launch_variant(const Params &p, hipStream_t stream) {
             right.C = p.C ? p.C + n1 : nullptr;
             right.D = p.D + n1;
             right.bias = p.bias ? p.bias + n1 : nullptr;
-            if (const int st = launch_variant<BF16, B_ROW_MAJOR>(left, stream); st != KO_OK) return st;
-            return launch_variant<BF16, B_ROW_MAJOR>(right, stream);
+            if (const int st = launch_variant<BF16, B_ROW_MAJOR>(left, stream, false, 2, variant, split_knob); st != KO_OK)
+                return st;
+            return launch_variant<BF16, B_ROW_MAJOR>(right, stream, false, 1, variant, split_knob);
         }
-        if (tuning("gemm16.split_rows") != 1 && p.K >= 256) {
+        if (row_cuts > 0 && split_knob != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
             const int64_t tn = (p.N + 255) / 256;
             const bool pinned_ok = p.N % 256 == 0 && p.K % (2 * kBK) == 0;
@@ -1222,8 +1231,10 @@ int launch_variant(const Params &p, hipStream_t stream) {
                 bottom.A = p.A + m1 * p.K;
                 bottom.C = p.C ? p.C + m1 * p.ldd : nullptr;
                 bottom.D = p.D + m1 * p.ldd;
-                if (const int st = launch_variant<BF16, B_ROW_MAJOR>(top, stream); st != KO_OK) return st;
-                return launch_variant<BF16, B_ROW_MAJOR>(bottom, stream);
+                // the top part holds whole rounds or whole tile rows: it is not cut again
+                if (const int st = launch_variant<BF16, B_ROW_MAJOR>(top, stream, false, 0, variant, split_knob); st != KO_OK)
+                    return st;
+                return launch_variant<BF16, B_ROW_MAJOR>(bottom, stream, false, row_cuts - 1, variant, split_knob);
             }
         }
         // The pinned kernel is so much faster per tile that it wins from half a chip's worth of full tiles on

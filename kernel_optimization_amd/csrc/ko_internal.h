@@ -20,8 +20,41 @@ int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)))
 // Maps a hipError_t to a ko_status, recording file:line and the HIP error name.
 int hip_fail(hipError_t err, const char *expr, const char *file, int line);
 
-// Integer tuning knobs (0 = use the built-in default).
-int tuning(const char *name);
+// Integer tuning knobs (0 = use the built-in default).  One relaxed atomic per knob, indexed by an enum: a
+// launch path reads several of them per call and takes no lock and builds no string to do so.  The names are
+// what ko_set_tuning / ko_get_tuning accept.
+#define KO_TUNING_KNOBS(X)                                                                                  \
+    X(softmax_lanes_per_row, "softmax.lanes_per_row") X(softmax_blocks_per_cu, "softmax.blocks_per_cu")     \
+    X(softmax_nontemporal, "softmax.nontemporal") X(softmax_block_threads, "softmax.block_threads")         \
+    X(softmax_wave_threads, "softmax.wave_threads") X(layernorm_lanes_per_row, "layernorm.lanes_per_row")   \
+    X(layernorm_blocks_per_cu, "layernorm.blocks_per_cu") X(layernorm_block_threads, "layernorm.block_threads") \
+    X(layernorm_wave_threads, "layernorm.wave_threads") X(softmax_wave_lds, "softmax.wave_lds") X(layernorm_wave_lds, "layernorm.wave_lds")           \
+    X(sgemm_variant, "sgemm.variant") X(sgemm_mapping, "sgemm.mapping") X(sgemm_split_rows, "sgemm.split_rows") \
+    X(gemm16_variant, "gemm16.variant") X(gemm16_mapping, "gemm16.mapping")                                 \
+    X(gemm16_split_rows, "gemm16.split_rows") X(copy_blocks_per_cu, "copy.blocks_per_cu")                   \
+    X(copy_nontemporal, "copy.nontemporal")
+enum Knob {
+#define KO_KNOB_ENUM(id, name) knob_##id,
+    KO_TUNING_KNOBS(KO_KNOB_ENUM)
+#undef KO_KNOB_ENUM
+    knob_count
+};
+extern std::atomic<int> g_knobs[knob_count];
+inline int tuning(Knob k) { return g_knobs[k].load(std::memory_order_relaxed); }
+
+// Residency cap for the streaming row kernels.  A one-pass kernel over HBM runs fastest on MI355X with about
+// 32-40 KB of loads in flight per compute unit; with more resident wavefronts than that needs, the requests
+// of a CU spread over a wider address window and the achieved rate drops (a 1 GiB copy with 2 KB per
+// wavefront: 6.32 TB/s at 32 resident wavefronts per CU, 6.84 TB/s at 16).  A single-wavefront workgroup
+// therefore asks for dynamic LDS it never touches, sized so that `bytes_in_flight / bytes_per_wave`
+// workgroups fit into the 160 KB of a CU.  Returns 0 (no cap) when the hardware limit of 32 is no more.
+inline int lds_pad_for_residency(int64_t bytes_per_wave, int64_t bytes_in_flight) {
+    if (bytes_per_wave <= 0) return 0;
+    int64_t waves = (bytes_in_flight + bytes_per_wave - 1) / bytes_per_wave;
+    if (waves >= 32) return 0;
+    if (waves < 8) waves = 8;  // fewer leave the memory latency uncovered (8 KB rows: 5 resident 75.7 us, 8 64.0 us)
+    return static_cast<int>((160 * 1024 / waves) & ~int64_t{511});
+}
 
 inline hipStream_t as_stream(ko_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

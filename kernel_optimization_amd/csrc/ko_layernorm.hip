@@ -19,6 +19,12 @@
 // spread, not of the offset, and x - x0 itself is exact or nearly so.
 // mean = x0 + mean(x - x0); its error is relative to the spread of the row.
 //
+// A row that holds a NaN or an infinity has no statistics: M2 becomes NaN (the
+// update multiplies inf by inf - inf), and with it rstd and every y of the row;
+// mean is reported as NaN as well, whatever the running mean happened to be (the
+// reference's own update turns mu into NaN as soon as an element follows an
+// infinity: d = x - mu = -inf, mu += d/n, layernorm.h:16-18).
+//
 // Mappings as in the reference: WARP (LayerNormWarpImpl :145-201) = row in the
 // registers of LPR lanes of a wavefront; BLOCK (LayerNormBlockImpl :204-252) =
 // row in the registers of a workgroup, per-wave triplets through LDS;
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
             }
         }
         if (row_ok && l == 0) {
-            if (mean_out) mean_out[row] = x0 + mean;
+            if (mean_out) mean_out[row] = rstd != rstd ? rstd : x0 + mean;  // no statistics for a row with NaN or inf
             if (rstd_out) rstd_out[row] = rstd;
         }
     };
@@ -340,7 +346,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
             }
         }
         if (threadIdx.x == 0) {
-            if (mean_out) mean_out[row] = x0 + mean;
+            if (mean_out) mean_out[row] = rstd != rstd ? rstd : x0 + mean;  // no statistics for a row with NaN or inf
             if (rstd_out) rstd_out[row] = rstd;
         }
     }
@@ -422,7 +428,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
             }
         }
         if (threadIdx.x == 0) {
-            if (mean_out) mean_out[row] = x0 + mean;
+            if (mean_out) mean_out[row] = rstd != rstd ? rstd : x0 + mean;  // no statistics for a row with NaN or inf
             if (rstd_out) rstd_out[row] = rstd;
         }
     }
@@ -433,21 +439,28 @@ template <int IO, int LPR, int VPL, bool FULL>
 int launch_wave_full(const Args<IO> &a) {
     constexpr int RPW = 64 / LPR;
     // Single-wavefront workgroups by default (measured slightly faster than 256 threads).
-    int threads = tuning("layernorm.wave_threads");
+    int threads = tuning(knob_layernorm_wave_threads);
     if (threads != 128 && threads != 256) threads = 64;
     const int64_t rows_per_block = static_cast<int64_t>(RPW) * (threads / 64);
     const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
     // One row group per wavefront by default; a positive knob caps the grid (grid-stride loop) instead.
     int64_t grid = needed;
-    const int per_cu = tuning("layernorm.blocks_per_cu");
+    const int per_cu = tuning(knob_layernorm_blocks_per_cu);
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
+    // Residency cap (see lds_pad_for_residency).  The statistics keep a wavefront busy for a while after its
+    // loads have landed, so more bytes' worth of wavefronts are kept resident than for softmax: 72 KB
+    // ([16384, 768]: 24 wavefronts per CU 18.7 us, 32 19.2 us, 16 19.0 us, 12 20.0 us).  Knob: bytes, or -1.
+    int lds = tuning(knob_layernorm_wave_lds);
+    if (lds == 0 && threads == 64)
+        lds = lds_pad_for_residency(static_cast<int64_t>(RPW) * a.cols * sizeof(typename Io<IO>::elem), 72 * 1024);
+    if (lds < 0) lds = 0;
     if (a.gamma || a.beta)
-        layernorm_wave_kernel<IO, LPR, VPL, FULL, true><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+        layernorm_wave_kernel<IO, LPR, VPL, FULL, true><<<dim3(static_cast<unsigned>(grid)), dim3(threads), lds, a.stream>>>(
             a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     else
-        layernorm_wave_kernel<IO, LPR, VPL, FULL, false><<<dim3(static_cast<unsigned>(grid)), dim3(threads), 0, a.stream>>>(
+        layernorm_wave_kernel<IO, LPR, VPL, FULL, false><<<dim3(static_cast<unsigned>(grid)), dim3(threads), lds, a.stream>>>(
             a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();
     return KO_OK;
@@ -517,7 +530,7 @@ int default_lanes_per_row(int nvec) {
 template <int IO>
 int launch_wave_any(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
-    int lpr = tuning("layernorm.lanes_per_row");
+    int lpr = tuning(knob_layernorm_lanes_per_row);
     if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec);
     while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
     return launch_wave_lpr<IO>(a, lpr);
@@ -556,7 +569,7 @@ int launch_block_threads(const Args<IO> &a) {
 template <int IO>
 int launch_block(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
-    int threads = tuning("layernorm.block_threads");
+    int threads = tuning(knob_layernorm_block_threads);
     if (threads != 256 && threads != 512 && threads != 1024) {
         // up to eight vectors per thread before the workgroup grows: gamma and beta then still fit the registers
         // next to the row at 256 and 512 threads ([8192, 16384]: 512 threads 181 us, 1024 threads 186 us)

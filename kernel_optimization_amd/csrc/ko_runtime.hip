@@ -4,9 +4,6 @@
 #include "ko_internal.h"
 
 #include <cstring>
-#include <map>
-#include <mutex>
-#include <string>
 
 namespace ko {
 
@@ -29,23 +26,19 @@ int hip_fail(hipError_t err, const char *expr, const char *file, int line) {
                 hipGetErrorName(err), expr);
 }
 
-static std::mutex g_tuning_mutex;
-static std::map<std::string, int> &tuning_table() {
-    static std::map<std::string, int> t = {
-        {"softmax.lanes_per_row", 0}, {"softmax.blocks_per_cu", 0}, {"softmax.nontemporal", 0},
-        {"softmax.block_threads", 0},
-        {"layernorm.lanes_per_row", 0}, {"layernorm.blocks_per_cu", 0},
-        {"layernorm.block_threads", 0}, {"layernorm.wave_threads", 0}, {"softmax.wave_threads", 0},
-        {"sgemm.variant", 0}, {"sgemm.mapping", 0}, {"sgemm.split_rows", 0}, {"gemm16.variant", 0}, {"gemm16.mapping", 0}, {"gemm16.split_rows", 0}, {"copy.blocks_per_cu", 0},
-        {"copy.nontemporal", 0},
-    };
-    return t;
-}
+std::atomic<int> g_knobs[knob_count];  // zero-initialised: every knob starts at its default
 
-int tuning(const char *name) {
-    std::lock_guard<std::mutex> lock(g_tuning_mutex);
-    auto it = tuning_table().find(name);
-    return it == tuning_table().end() ? 0 : it->second;
+static const char *const kKnobNames[knob_count] = {
+#define KO_KNOB_NAME(id, name) name,
+    KO_TUNING_KNOBS(KO_KNOB_NAME)
+#undef KO_KNOB_NAME
+};
+
+// Index of the knob called `name`, or -1.  Only ko_set_tuning / ko_get_tuning look names up.
+static int find_knob(const char *name) {
+    for (int i = 0; i < knob_count; ++i)
+        if (std::strcmp(kKnobNames[i], name) == 0) return i;
+    return -1;
 }
 
 int compute_units() {
@@ -91,21 +84,17 @@ KO_EXPORT const char *ko_status_name(int status) {
 
 KO_EXPORT int ko_set_tuning(const char *name, int value) {
     if (!name) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: null name");
-    std::lock_guard<std::mutex> lock(ko::g_tuning_mutex);
-    auto it = ko::tuning_table().find(name);
-    if (it == ko::tuning_table().end())
-        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: unknown knob \"%s\"", name);
-    it->second = value;
+    const int k = ko::find_knob(name);
+    if (k < 0) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: unknown knob \"%s\"", name);
+    ko::g_knobs[k].store(value, std::memory_order_relaxed);
     return KO_OK;
 }
 
 KO_EXPORT int ko_get_tuning(const char *name, int *value) {
     if (!name || !value) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: null argument");
-    std::lock_guard<std::mutex> lock(ko::g_tuning_mutex);
-    auto it = ko::tuning_table().find(name);
-    if (it == ko::tuning_table().end())
-        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: unknown knob \"%s\"", name);
-    *value = it->second;
+    const int k = ko::find_knob(name);
+    if (k < 0) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: unknown knob \"%s\"", name);
+    *value = ko::g_knobs[k].load(std::memory_order_relaxed);
     return KO_OK;
 }
 

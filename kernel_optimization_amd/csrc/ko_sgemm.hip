@@ -621,7 +621,7 @@ int launch(Params p, hipStream_t stream) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
     if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
-    p.blocked = tuning("sgemm.mapping") != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
+    p.blocked = tuning(knob_sgemm_mapping) != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
                 ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
     const bool vec = (p.K % 4 == 0) && (p.lda % 4 == 0) && (p.N % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
@@ -655,7 +655,7 @@ int launch_direct(Params p, hipStream_t stream) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
     if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
-    p.blocked = tuning("sgemm.mapping") != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
+    p.blocked = tuning(knob_sgemm_mapping) != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
                 ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
     auto kernel = edge ? sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, true>
                        : sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, false>;
@@ -723,8 +723,8 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
     Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, static_cast<int>(k)};
     hipStream_t s = as_stream(stream);
-    const int variant = tuning("sgemm.variant");
-    if (variant <= 0 && tuning("sgemm.split_rows") != 1 && k >= 512) {
+    const int variant = tuning(knob_sgemm_variant);
+    if (variant <= 0 && tuning(knob_sgemm_split_rows) != 1 && k >= 512) {
         // A last round of 128 x 128 tiles that fills at most half of the compute units costs a whole round:
         // the tile rows that fill whole rounds go out as one launch, the rows below them as a second one
         // with the smaller tiles its own size asks for (4096 x 4224 x 4096, 1056 tiles on 256 compute

@@ -20,6 +20,14 @@
 // intended x - m, not the x + m the reference's Subtract functor computes,
 // common/functors.h:168).
 //
+// Special values follow from that arithmetic as they do in the reference: a NaN
+// element, or a +inf element (inf - inf), makes exp(x - m) NaN and with it the
+// row's sum and every output of the row; -inf elements get probability 0; a row
+// of nothing but -inf keeps m = -FLT_MAX, sums to 0 and comes out as 0/0 = NaN.
+// The maximum itself ignores NaN (fmaxf), which changes nothing: the sum is NaN
+// either way.  Vector slots past the end of a row hold -inf, so they add
+// nothing to any sum.  Masked columns are replaced before any of this.
+//
 // Mask: columns j >= valid_len[row / rows_per_seq] take the value -10000.  Vectors
 // that lie wholly in the padded part are not loaded.
 #include "ko_internal.h"
@@ -128,7 +136,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
             finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
             if (!(row_ok && j < nvec)) {
 #pragma unroll
-                for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                for (int e = 0; e < E; ++e) v[k][e] = -INFINITY;
             }
         }
 
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                     Io<IO>::template load<true>(at_bytes(src, first + k * kStep), v[k]);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                    for (int e = 0; e < E; ++e) v[k][e] = -INFINITY;
                 }
             }
         } else {
@@ -253,7 +261,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                 finish_row_vec<IO, MASKED>(loaded[k], j, vlen, v[k]);
                 if (j >= nvec) {
 #pragma unroll
-                    for (int e = 0; e < E; ++e) v[k][e] = -FLT_MAX;
+                    for (int e = 0; e < E; ++e) v[k][e] = -INFINITY;
                 }
             }
         }
@@ -387,18 +395,25 @@ int launch_wave(const Args<IO> &a) {
     constexpr int RPW = 64 / LPR;
     // Single-wavefront workgroups by default (measured 1-4 % faster than 256 threads: the dispatcher
     // places waves more freely); the knob selects 128 or 256.
-    int kThreads = tuning("softmax.wave_threads");
+    int kThreads = tuning(knob_softmax_wave_threads);
     if (kThreads != 128 && kThreads != 256) kThreads = 64;
     const int64_t rows_per_block = RPW * (kThreads / 64);
     const int64_t needed = (a.rows + rows_per_block - 1) / rows_per_block;
     // One row batch per wavefront by default (measured faster than a persistent grid-stride
     // launch: the hardware keeps more loads in flight); a positive knob caps the grid instead.
     int64_t grid = needed;
-    const int per_cu = tuning("softmax.blocks_per_cu");
+    const int per_cu = tuning(knob_softmax_blocks_per_cu);
     if (per_cu > 0 && grid > static_cast<int64_t>(compute_units()) * per_cu)
         grid = static_cast<int64_t>(compute_units()) * per_cu;
     if (grid > 0x7fffffff) grid = 0x7fffffff;
-    softmax_wave_kernel<IO, LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, a.stream>>>(
+    // Residency cap (see lds_pad_for_residency): 40 KB of row loads in flight per CU; with a mask about a third
+    // of the nominal row bytes are never loaded, hence 64 KB of nominal bytes.  Knob: bytes, or -1 for none.
+    int lds = tuning(knob_softmax_wave_lds);
+    if (lds == 0 && kThreads == 64)
+        lds = lds_pad_for_residency(static_cast<int64_t>(RPW) * a.cols * sizeof(typename Io<IO>::elem),
+                                    (MASKED ? 64 : 40) * 1024);
+    if (lds < 0) lds = 0;
+    softmax_wave_kernel<IO, LPR, VPL, MASKED, NT><<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, a.stream>>>(
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
     KO_CHECK_LAUNCH();
     return KO_OK;
@@ -446,7 +461,7 @@ constexpr int kBlockMaxVecsMasked = 1024 * (64 / Io<IO>::E);
 // of the group then covers the longest contiguous piece of the row.  With a padding mask at least two
 // vectors per lane are preferred: a lane whose only vector lies in the padding idles through the whole
 // row (measured on [786432, 512] binary16, mean valid length 288: 64 x 1 309 us, 32 x 2 230 us).
-int default_lanes_per_row(int nvec, bool masked) {
+int default_lanes_per_row(int nvec, bool masked, int masked_min_vpl) {
     int best = 64, best_waste = 1 << 30;
     for (int lpr = 8; lpr <= 64; lpr <<= 1) {
         int vpl = (nvec + lpr - 1) / lpr;
@@ -454,7 +469,8 @@ int default_lanes_per_row(int nvec, bool masked) {
         if (vpl == 5) vpl = 6;
         if (vpl == 7) vpl = 8;
         const int waste = lpr * vpl - nvec;
-        if (waste < best_waste || (waste == best_waste && !(masked && vpl < 2))) {
+        // with a mask, four vectors per lane before two (fp32 [786432, 512]: 32 x 4 391 us, 64 x 2 395 us)
+        if (waste < best_waste || (waste == best_waste && !(masked && vpl < masked_min_vpl))) {
             best_waste = waste;
             best = lpr;
         }
@@ -465,13 +481,13 @@ int default_lanes_per_row(int nvec, bool masked) {
 template <int IO, bool MASKED>
 int launch_wave_any(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
-    int lpr = tuning("softmax.lanes_per_row");
-    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec, MASKED);
+    int lpr = tuning(knob_softmax_lanes_per_row);
+    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec, MASKED, IO == IO_F32 ? 4 : 2);
     while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
     // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off
     // (fp32 storage only; the 16-bit kernels are built with streaming accesses).
     if constexpr (IO == IO_F32) {
-        if (tuning("softmax.nontemporal") == 2) return launch_wave_lpr<IO, MASKED, false>(a, lpr);
+        if (tuning(knob_softmax_nontemporal) == 2) return launch_wave_lpr<IO, MASKED, false>(a, lpr);
     }
     return launch_wave_lpr<IO, MASKED, true>(a, lpr);
 }
@@ -509,7 +525,7 @@ int launch_block_threads(const Args<IO> &a) {
 template <int IO, bool MASKED>
 int launch_block(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
-    int threads = tuning("softmax.block_threads");
+    int threads = tuning(knob_softmax_block_threads);
     if (threads != 256 && threads != 512 && threads != 1024) {
         threads = 256;
         while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;

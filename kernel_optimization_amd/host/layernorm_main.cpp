@@ -55,6 +55,7 @@ void run_benchmark(float epsilon) {
     printf("======Num row %d, num column %d======\n", num_row, num_column);
     printf("Average time %.2fms\n", time_in_ms / n_iter);
     printf("Algorithmic bandwidth %.0f GB/s\n", 2.0 * count * sizeof(T) / (time_in_ms / n_iter * 1e-3) / 1e9);
+    printf("Variance divisor: num_column (population variance; pass unbiased = true for num_column - 1)\n");
 
     // Sampled rows against a two-pass computation in double.
     out_data.device_to_host_async(stream);

@@ -204,6 +204,10 @@ ORACLE_API int oracle_softmax_f32(const float *in, float *out, int64_t rows, int
  * (nn_operators/layernorm/layernorm.h:184-195, with the intended x - mean).
  * var divides by N (unbiased == 0) or N - 1 (unbiased != 0; the reference's
  * intent at layernorm.h:48).  mean, rstd, gamma, beta may be NULL.
+ * A row holding a NaN or an infinity has no statistics: the sum of squared
+ * deviations is NaN (inf - inf), so rstd and y are NaN, and mean is reported as
+ * NaN too (the reference's streaming update makes its mean NaN as soon as an
+ * element follows an infinity: d = x - mu = -inf, mu += d/n, layernorm.h:16-18).
  */
 ORACLE_API int oracle_layernorm_f32(const float *in, float *out, float *mean_out, float *rstd_out,
                                     const float *gamma, const float *beta,
@@ -222,6 +226,7 @@ ORACLE_API int oracle_layernorm_f32(const float *in, float *out, float *mean_out
             m2 += d * d;
         }
         double var = m2 / (double)(unbiased ? cols - 1 : cols);
+        if (isnan(m2)) mean = NAN;
         double rstd = 1.0 / sqrt(var + eps);
         if (out) {
             float *y = out + r * cols;
@@ -298,6 +303,7 @@ ORACLE_API int oracle_layernorm_16(const uint16_t *in, uint16_t *out, double *ou
             m2 += d * d;
         }
         double var = m2 / (double)(unbiased ? cols - 1 : cols);
+        if (isnan(m2)) mean = NAN;
         double rstd = 1.0 / sqrt(var + eps);
         for (int64_t j = 0; j < cols; ++j) {
             double v = (bits16_to_double(x[j], bf16) - mean) * rstd;

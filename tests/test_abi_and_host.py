@@ -116,6 +116,31 @@ def test_gemm_driver_on_gpu():
 
 
 @pytest.mark.gpu
+def test_softmax_driver_on_gpu():
+    """The softmax driver prints the reference's two lines per run (nn_operators/softmax/main.cu:72-73) for its
+    own run and for the two it leaves commented out (:78-79), plus the masked configuration, each checked."""
+    out = subprocess.run([os.path.join(BIN, "softmax")], capture_output=True, text=True, timeout=200)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "======Num row 196608, num column 128======" in out.stdout
+    assert out.stdout.count("======Num row 49152, num column 1024======") == 2
+    assert "======Num row 786432, num column 512======" in out.stdout
+    assert out.stdout.count("Average time ") == 4 and out.stdout.count("Passed.") == 4
+    assert "FAILED" not in out.stdout
+
+
+@pytest.mark.gpu
+def test_layernorm_driver_on_gpu():
+    """The LayerNorm driver: the reference's two runs (nn_operators/layernorm/main.cu:75-76) and the affine
+    configuration, with the reference's lines (:71-72) and a check of sampled rows."""
+    out = subprocess.run([os.path.join(BIN, "layernorm")], capture_output=True, text=True, timeout=200)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.count("======Num row 16384, num column 768======") == 3
+    assert "======Num row 49152, num column 1024======" in out.stdout
+    assert out.stdout.count("Average time ") == 4 and out.stdout.count("Passed.") == 4
+    assert "Variance divisor: num_column" in out.stdout and "FAILED" not in out.stdout
+
+
+@pytest.mark.gpu
 def test_device_fill_matches_host_generator(ko):
     from kernel_optimization_amd import inputs
     n = 1 << 16
@@ -138,6 +163,22 @@ def test_device_fill_matches_host_generator(ko):
     dev = buf.download(np.float32, (n,))
     assert np.all(np.abs(dev - host) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))  # libm vs device log/cos: <= 1 ulp
     assert (dev != host).mean() < 0.01
+
+
+def test_cmake_tree_has_the_reference_targets(tmp_path):
+    """CMakeLists.txt configures and offers the reference's target names (common, softmax, layernorm, gemm,
+    nn_operators; /root/reference CMakeLists.txt:10-17, nn_operators/CMakeLists.txt:5-14) next to ko."""
+    import shutil
+    if shutil.which("cmake") is None:
+        pytest.skip("cmake is not installed")
+    r = subprocess.run(["cmake", "-S", ROOT, "-B", str(tmp_path)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    r = subprocess.run(["cmake", "--build", str(tmp_path), "--target", "help"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    for target in ("common", "softmax", "layernorm", "gemm", "nn_operators", "kernel-optimization", "ko", "ko_vendor"):
+        assert any(line.split()[-1] == target or line.split(":")[0].strip(". ") == target
+                   for line in r.stdout.splitlines() if line.strip()), (target, r.stdout)
 
 
 def test_bench_refuses_more_than_one_gpu():

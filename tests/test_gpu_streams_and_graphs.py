@@ -47,7 +47,7 @@ def test_operators_replay_from_a_hip_graph(ko):
     a32, b32, d32 = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
     m2, n2, k2 = 4096, 2048, 256  # 128 tiles of 256 x 256: the persistent direct-to-LDS kernel
     a2, b2, d2 = ko.DeviceBuffer(m2 * k2 * 2), ko.DeviceBuffer(n2 * k2 * 2), ko.DeviceBuffer(m2 * n2 * 2)
-    m3, n3, k3 = 4136, 2200, 128  # cut along rows and columns: four launches behind one call
+    m3, n3, k3 = 8000, 2312, 256  # cut along columns and twice along rows: the most launches behind one call
     a3, b3, d3 = ko.DeviceBuffer(m3 * k3 * 2), ko.DeviceBuffer(n3 * k3 * 2), ko.DeviceBuffer(m3 * n3 * 2)
     ko.fill_uniform_16(a3, m3 * k3, 509)
     ko.fill_uniform_16(b3, n3 * k3, 510)

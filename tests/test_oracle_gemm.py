@@ -90,3 +90,84 @@ def test_gemm16_identity_kat_and_epilogue():
     C = inputs.uniform_f16((n, n), 4, -2.0, 2.0)
     D, d64, _ = oracle.gemm16(A.view(np.uint16), I.view(np.uint16), n, n, n, C_bits=C.view(np.uint16), alpha=1.0, beta=1.0)
     np.testing.assert_array_equal(d64, A.reshape(n, n).astype(np.float64) + C.astype(np.float64))
+
+
+# ---- epilogue of oracle_gemm_16_bias_act: D = act(alpha A B + beta C + bias) ----------------------------
+
+def _epilogue_case(bf16=False):
+    """A small non-square product whose pre-activation values span about [-6, 6]."""
+    m, n, k = 13, 24, 16
+    to64 = oracle.bf16_to_f64 if bf16 else oracle.f16_to_f64
+    if bf16:
+        A = inputs.uniform_bf16_bits((m, k), 11)
+        Bt = inputs.uniform_bf16_bits((n, k), 12)
+        bias = inputs.uniform_bf16_bits((n,), 13, -3.0, 3.0)
+        C = inputs.uniform_bf16_bits((m, n), 14, -2.0, 2.0)
+    else:
+        A = inputs.uniform_f16((m, k), 11).view(np.uint16)
+        Bt = inputs.uniform_f16((n, k), 12).view(np.uint16)
+        bias = inputs.uniform_f16((n,), 13, -3.0, 3.0).view(np.uint16)
+        C = inputs.uniform_f16((m, n), 14, -2.0, 2.0).view(np.uint16)
+    acc = to64(A) @ to64(Bt).T
+    return (m, n, k), A, Bt, bias, C, acc, to64(bias), to64(C)
+
+
+def _gelu_erf64(x):
+    import math
+    return np.array([0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))) for v in x.ravel()]).reshape(x.shape)
+
+
+def _gelu_tanh64(x):
+    return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm16_bias_is_added_per_column_before_the_activation(bf16):
+    (m, n, k), A, Bt, bias, C, acc, bias64, C64 = _epilogue_case(bf16)
+    # bias only: one value per output column, broadcast over rows (a per-row bias fails: m != n)
+    _, d64, _ = oracle.gemm16(A, Bt, m, n, k, bf16=bf16, bias_bits=bias)
+    np.testing.assert_allclose(d64, acc + bias64[None, :], rtol=1e-13, atol=1e-13)
+    # alpha, beta, C and bias together, no activation
+    _, d64, _ = oracle.gemm16(A, Bt, m, n, k, bf16=bf16, C_bits=C, alpha=0.75, beta=-1.5, bias_bits=bias)
+    pre = 0.75 * acc - 1.5 * C64 + bias64[None, :]
+    np.testing.assert_allclose(d64, pre, rtol=1e-13, atol=1e-13)
+    # both activations of the full pre-activation value, in independent float64 formulations
+    for act, f in ((oracle.ACT_GELU_ERF, _gelu_erf64), (oracle.ACT_GELU_TANH, _gelu_tanh64)):
+        _, d64, _ = oracle.gemm16(A, Bt, m, n, k, bf16=bf16, C_bits=C, alpha=0.75, beta=-1.5, bias_bits=bias, act=act)
+        np.testing.assert_allclose(d64, f(pre), rtol=1e-12, atol=1e-14)
+        # bias added after the activation, or C/bias left out of it, must not pass
+        assert np.abs(f(0.75 * acc - 1.5 * C64) + bias64[None, :] - d64).max() > 1e-2
+        assert np.abs(f(0.75 * acc) - 1.5 * C64 + bias64[None, :] - d64).max() > 1e-2
+
+
+def test_gemm16_gelu_known_values_and_symmetries():
+    """The activation alone: A = x as a column, B = [1], so the pre-activation value is x itself."""
+    x = np.array([0.0, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, 3.0, -3.0, 8.0, -8.0, 12.0, -12.0, 0.25, -0.25, 6.0],
+                 np.float16)
+    m = x.size
+    one = np.ones((1, 8), np.float16)
+    A = np.zeros((m, 8), np.float16)
+    A[:, 0] = x
+    x64 = x.astype(np.float64)
+    out = {}
+    for act in (oracle.ACT_NONE, oracle.ACT_GELU_ERF, oracle.ACT_GELU_TANH):
+        D, d64, _ = oracle.gemm16(A.view(np.uint16), one.view(np.uint16), m, 1, 8, act=act)
+        out[act] = d64[:, 0]
+        np.testing.assert_array_equal(D[:, 0], oracle.f64_to_f16(d64[:, 0]))  # one rounding of the activated value
+    np.testing.assert_array_equal(out[oracle.ACT_NONE], x64)
+    erf, tanh = out[oracle.ACT_GELU_ERF], out[oracle.ACT_GELU_TANH]
+    for g in (erf, tanh):
+        assert g[0] == 0.0                                              # GELU(0) = 0
+        np.testing.assert_allclose(g[1:15:2] - g[2:15:2], x64[1:15:2], rtol=1e-14)  # GELU(x) - GELU(-x) = x
+        np.testing.assert_allclose(g[9], 8.0, rtol=1e-14)               # large x: identity
+        assert abs(g[10]) < 1e-13 and abs(g[12]) < 1e-30                # large -x: 0 from below
+        assert g[10] <= 0.0
+    # published values: GELU(1) = Phi(1) = 0.8413447460685429; tanh form 0.8411919906082768
+    np.testing.assert_allclose(erf[1], 0.8413447460685429, rtol=1e-14)
+    np.testing.assert_allclose(tanh[1], 0.8411919906082768, rtol=1e-13)
+    np.testing.assert_allclose(erf[5], 2.0 * 0.9772498680518208, rtol=1e-14)   # 2 Phi(2)
+    # the two forms differ (by up to 5e-4 around |x| = 2..3) and must not be interchangeable
+    assert 1e-4 < np.abs(erf - tanh).max() < 1e-3
+    # scipy's erf as a second opinion on the exact form
+    from scipy.special import erf as sp_erf
+    np.testing.assert_allclose(erf, 0.5 * x64 * (1.0 + sp_erf(x64 / np.sqrt(2.0))), rtol=1e-13, atol=1e-300)

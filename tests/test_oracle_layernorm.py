@@ -112,3 +112,23 @@ def test_reference_bug_is_not_reproduced():
     x = inputs.normal_f32((1, 768), 29, 0.5, 2.0)
     _, _, r = oracle.layernorm(x, eps=0.0, unbiased=True)
     np.testing.assert_allclose(r, 1 / x.astype(np.float64).std(ddof=1), rtol=1e-7)
+
+
+def test_special_values_leave_a_row_without_statistics():
+    """A NaN or an infinity in a row: y, mean and rstd of that row are NaN (the sum of squared deviations is
+    inf - inf); other rows are untouched."""
+    import special_values as sv
+    cols = 40
+    base = inputs.normal_f32((5, cols), 78, 0.5, 2.0)
+    x, classes = sv.build(sv.LAYERNORM_ROWS, cols, base)
+    g = inputs.normal_f32((cols,), 79, 1.0, 0.1)
+    b = inputs.normal_f32((cols,), 80, 0.0, 0.1)
+    y, mean, rstd = oracle.layernorm(x, g, b)
+    ok = sv.check_rows(y, y, classes, "oracle layernorm y")
+    sv.check_rows(mean, mean, classes, "oracle layernorm mean")
+    sv.check_rows(rstd, rstd, classes, "oracle layernorm rstd")
+    clean = np.array([base[i % 5] for i in range(x.shape[0])], np.float32)
+    yc, mc, rc = oracle.layernorm(clean, g, b)
+    np.testing.assert_array_equal(y[ok], yc[ok])
+    np.testing.assert_array_equal(mean[ok], mc[ok])
+    np.testing.assert_array_equal(rstd[ok], rc[ok])

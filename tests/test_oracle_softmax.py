@@ -101,3 +101,30 @@ def test_mask_semantics():
 def test_bad_arguments():
     with pytest.raises(ValueError):
         oracle.softmax(np.zeros((2, 4), np.float32), valid_len=np.array([1], np.int32), rows_per_seq=0)
+
+
+def test_special_values_follow_the_reference_arithmetic():
+    """NaN and +inf poison their row (exp(x - max) is NaN), -inf elements get probability 0, a row of -inf is
+    0/0 = NaN, a row of -FLT_MAX is uniform (softmax.h:33: the running maximum starts at -FLT_MAX)."""
+    import special_values as sv
+    cols = 24
+    base = inputs.normal_f32((5, cols), 77, 0.0, 4.0)
+    x, classes = sv.build(sv.SOFTMAX_ROWS, cols, base)
+    y = oracle.softmax(x)
+    ok = sv.check_rows(y, y, classes, "oracle softmax")
+    names = [n for n, _, _ in sv.SOFTMAX_ROWS]
+    # ordinary rows: equal to a float64 numpy softmax over the finite part, exact zeros at -inf
+    for i in np.nonzero(ok)[0]:
+        r = x[i].astype(np.float64)
+        if names[i] == "minus_flt_max_all":
+            np.testing.assert_array_equal(y[i], np.float32(1.0 / cols))
+            continue
+        fin = np.isfinite(r)
+        e = np.exp(r[fin] - r[fin].max())
+        np.testing.assert_allclose(y[i][fin], e / e.sum(), rtol=1e-6)
+        np.testing.assert_array_equal(y[i][~fin], 0.0)
+    # a masked row ignores what lies in the padding, special values included
+    xm = base[:1].copy()
+    xm[0, 10:] = [np.nan, np.inf, -np.inf] + [np.nan] * (cols - 13)
+    ym = oracle.softmax(xm, np.array([10], np.int32), 1)
+    np.testing.assert_array_equal(ym, oracle.softmax(base[:1], np.array([10], np.int32), 1))
