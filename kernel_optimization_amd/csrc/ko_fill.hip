@@ -87,8 +87,16 @@ template <bool NT>
 __global__ __launch_bounds__(128) void copy_f32_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                        int64_t nvec, int64_t n) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
-    for (; i < nvec; i += stride) store4<NT>(out + 4 * i, load4<NT>(in + 4 * i));
+    // NT: non-temporal loads and streaming (sc1 nt) stores, addressed as the workgroup's uniform chunk base plus
+    // 16 bytes per thread
+    for (int64_t i0 = blockIdx.x * static_cast<int64_t>(blockDim.x); i0 < nvec; i0 += stride) {
+        const int64_t i = i0 + threadIdx.x;
+        if (i < nvec) {
+            const float4v v = load4<NT>(in + 4 * i);
+            if constexpr (NT) stream_store16(out + 4 * i0, threadIdx.x * 16u, v);
+            else store4<false>(out + 4 * i, v);
+        }
+    }
     // tail (n not a multiple of 4)
     const int64_t t = nvec * 4 + blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
     if (t < n) out[t] = in[t];

@@ -271,7 +271,8 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 if (erow(row) & 1) v = u32x4{v[2], v[3], v[0], v[1]};
                 const int gm = row0 + part * PROWS + row;
                 const int gn = col0 + c * 8;
-                // streaming store: D is written once and not read again by this kernel
+                // streaming store: D is written once and not read again by this kernel (`sc1 nt`, which helps the
+                // row kernels, measured no different here: 74.3 against 73.8 us)
                 __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p.D + gm * ldd + gn));
             }
         }

@@ -55,6 +55,16 @@ __device__ __forceinline__ void welford_update(wave::Welford &w, float x, float 
     w.m2 = __builtin_fmaf(d, x - w.mean, w.m2);
 }
 
+// The same update where the count is not a compile-time constant: 1/count comes from the hardware reciprocal
+// (1 ulp).  M2 is accumulated against the mean actually formed, so the triplet stays consistent and the
+// deviation is far inside the 1e-5 gate.
+__device__ __forceinline__ void welford_update_counted(wave::Welford &w, float x) {
+    w.count += 1.0f;
+    const float d = x - w.mean;
+    w.mean = __builtin_fmaf(d, __builtin_amdgcn_rcpf(w.count), w.mean);
+    w.m2 = __builtin_fmaf(d, x - w.mean, w.m2);
+}
+
 template <int IO>
 struct Args {
     const typename Io<IO>::elem *in;
@@ -157,7 +167,9 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
 
-        typename Io<IO>::elem *dst = out + row * cols;
+        // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
+        typename Io<IO>::elem *dst0 = out + (row - sub) * cols;
+        const uint32_t sub_off = static_cast<uint32_t>(sub) * static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem);
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
@@ -182,7 +194,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
                 }
 #pragma unroll
                 for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[e], b[e]);
-                Io<IO>::template store<NT>(dst + E * j, y);
+                Io<IO>::store_stream(dst0, sub_off + 16u * j, y);
             }
         }
         if (row_ok && l == 0) {
@@ -254,9 +266,13 @@ __device__ __forceinline__ void normalize_vec(const float (&x)[Io<IO>::E], float
     }
 }
 
-// One workgroup per row, the row held in registers between its single read and its single write; both are
+// One workgroup per row, the row held on chip between its single read and its single write; both are
 // nontemporal (every byte is touched once; measured faster than cached accesses on rows of 16 KB and more).
-template <int IO, int THREADS, int VPL>
+// VPL vectors per thread live in registers, LV more in LDS (vector k of thread t at tail[k][t], filled by
+// direct-to-LDS loads, which cost no registers on the way).  REST: what lies beyond those (VPL + LV) * THREADS
+// vectors is streamed - folded into the statistics as it arrives, and read a second time for the output - so a
+// row a little longer than the chip holds costs a little more traffic, not half as much again.
+template <int IO, int THREADS, int VPL, int LV = 0, bool REST = false>
 __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename Io<IO>::elem *in,
                                                                   typename Io<IO>::elem *out,
                                                                   float *__restrict__ mean_out,
@@ -266,8 +282,13 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
                                                                   int64_t rows, int cols, float eps,
                                                                   float inv_denominator) {
     constexpr int E = Io<IO>::E;
+    typedef typename Io<IO>::raw Raw;
     __shared__ float lds[48];
+    extern __shared__ __attribute__((aligned(16))) char tail_bytes[];  // Raw tail[LV][THREADS]
+    Raw *tail = reinterpret_cast<Raw *>(tail_bytes);
     constexpr Reciprocals<VPL * E> rcp;
+    constexpr int UNROLL = 2;                       // vectors per thread and trip of the streamed part
+    constexpr int kCached = (VPL + LV) * THREADS;   // vectors of a row held on chip
     const int nvec = cols / E;
     // gamma/beta of this thread's columns stay in registers across the rows the workgroup walks, when
     // row, gamma and beta fit the register budget of the workgroup size (128 per lane at 1024 threads)
@@ -303,6 +324,18 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
                 loaded[k] = typename Io<IO>::raw{};
                 if (j < nvec) loaded[k] = Io<IO>::template load_raw<true>(at_bytes(src, first + k * kStep));
             }
+            if constexpr (LV > 0) {
+                // each lane's 16 bytes land at the wave's base plus 16 x lane, i.e. at tail[k][thread]; lanes
+                // past the end of the row write nothing
+#pragma unroll
+                for (int k = 0; k < LV; ++k) {
+                    const int j = threadIdx.x + (VPL + k) * THREADS;
+                    if (j < nvec)
+                        __builtin_amdgcn_global_load_lds(
+                            (const __attribute__((address_space(1))) void *)at_bytes(src, first + (VPL + k) * kStep),
+                            (__attribute__((address_space(3))) void *)(tail + k * THREADS + (threadIdx.x & ~63u)), 16, 0, 0);
+                }
+            }
 #pragma unroll
             for (int k = 0; k < VPL; ++k) Io<IO>::unpack(loaded[k], v[k]);
         }
@@ -318,10 +351,80 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
                 for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
             }
         }
+        // (the loops over the tail are kept rolled: unrolled, the compiler fetches all of it from LDS at once and spills)
+#pragma unroll 1
+        for (int k = 0; k < LV; ++k) {
+            if (static_cast<int>(threadIdx.x) + (VPL + k) * THREADS < nvec) {
+                float x[E];
+                Io<IO>::unpack(tail[k * THREADS + threadIdx.x], x);
+#pragma unroll
+                for (int e = 0; e < E; ++e) welford_update_counted(w, x[e] - x0);
+            }
+        }
+        if constexpr (REST) {
+            // cached loads here: the second read of these vectors may still find them in L2
+            for (int j0 = kCached + threadIdx.x; j0 < nvec; j0 += THREADS * UNROLL) {
+                float x[UNROLL][E];
+                Raw loaded[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    loaded[u] = Raw{};
+                    if (j0 + u * THREADS < nvec) loaded[u] = Io<IO>::template load_raw<false>(src + E * (j0 + u * THREADS));
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    if (j0 + u * THREADS >= nvec) break;
+#pragma unroll
+                    for (int e = 0; e < E; ++e) welford_update_counted(w, x[u][e] - x0);
+                }
+            }
+        }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
         const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
         typename Io<IO>::elem *dst = out + row * cols;
+        if constexpr (REST) {
+            // the streamed part first and from the row's end backwards: what was read last is the likeliest to be
+            // in a cache still
+            const int rest = nvec - kCached;
+            const int trips = rest > 0 ? (rest + THREADS * UNROLL - 1) / (THREADS * UNROLL) : 0;
+            for (int t = trips - 1; t >= 0; --t) {
+                const int j0 = kCached + threadIdx.x + t * (THREADS * UNROLL);
+                float x[UNROLL][E];
+                Raw loaded[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    loaded[u] = Raw{};
+                    if (j0 + u * THREADS < nvec) loaded[u] = Io<IO>::template load_raw<true>(src + E * (j0 + u * THREADS));
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const int j = j0 + u * THREADS;
+                    if (j >= nvec) break;
+                    float y[E];
+#pragma unroll
+                    for (int e = 0; e < E; ++e) x[u][e] -= x0;
+                    normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
+                    Io<IO>::store_stream(dst, 16u * j, y);
+                }
+            }
+        }
+#pragma unroll 1
+        for (int k = 0; k < LV; ++k) {
+            const int j = threadIdx.x + (VPL + k) * THREADS;
+            if (j < nvec) {
+                float x[E], y[E];
+                Io<IO>::unpack(tail[k * THREADS + threadIdx.x], x);
+#pragma unroll
+                for (int e = 0; e < E; ++e) x[e] -= x0;
+                normalize_vec<IO>(x, mean, rstd, gamma, beta, E * j, y);
+                Io<IO>::store_stream(dst, first + (VPL + k) * kStep, y);
+            }
+        }
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = threadIdx.x + k * THREADS;
@@ -342,7 +445,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
                         y[e] = t;
                     }
                 }
-                Io<IO>::template store<true>(at_bytes(dst, first + k * kStep), y);
+                Io<IO>::store_stream(dst, first + k * kStep, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -424,7 +527,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] -= x0;
                 normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                Io<IO>::template store<true>(dst + E * j, y);
+                Io<IO>::store_stream(dst, 16u * j, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -504,8 +607,9 @@ int launch_wave_lpr(const Args<IO> &a, int lpr) {
 // workgroup 80 values per thread of 1024 threads (81920 columns).
 constexpr int kWaveMaxVpl = 8;
 constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
+constexpr int kTailMaxVecs = 9;  // 16-byte vectors per thread of a 1024-thread workgroup kept in LDS (9 x 16 KB)
 template <int IO>
-constexpr int kBlockMaxVecs = 1024 * (80 / Io<IO>::E);
+constexpr int kBlockMaxVecs = 1024 * (80 / Io<IO>::E);  // in registers; BLOCK takes longer rows too (LDS, then streaming)
 
 // Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
 // {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
@@ -553,12 +657,23 @@ int launch_block_threads(const Args<IO> &a) {
     else if (vpl <= 8) KO_LN_BLOCK(8);
     else if constexpr (THREADS == 1024) {
         // a single resident workgroup of 1024 threads has 128 registers per thread: up to 80 hold the row
+        constexpr int kRegs = 80 / Io<IO>::E;  // vectors per thread held in registers
         if constexpr (Io<IO>::E == 4) {
             if (vpl <= 12) KO_LN_BLOCK(12);
             else if (vpl <= 16) KO_LN_BLOCK(16);
-            else KO_LN_BLOCK(20);
-        } else {
+            else if (vpl <= 20) KO_LN_BLOCK(20);
+        } else if (vpl <= 10) {
             KO_LN_BLOCK(10);
+        }
+        if (vpl > kRegs) {
+            // longer rows: nine more vectors per thread in LDS (9 x 16 KB), the rest of the row streamed twice
+            constexpr int kRegsTail = Io<IO>::E == 4 ? 20 : 8;  // 16-bit storage: 64 values, the conversions need registers too
+            auto kernel = layernorm_block_kernel<IO, THREADS, kRegsTail, kTailMaxVecs, true>;
+            static std::atomic<uint64_t> done{0};
+            if (const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 160 * 1024 - 256, done); rc != KO_OK)
+                return rc;
+            kernel<<<g, b, static_cast<size_t>(kTailMaxVecs) * THREADS * 16, a.stream>>>(
+                a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
         }
     }
 #undef KO_LN_BLOCK
@@ -625,8 +740,7 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
-                 : nvec <= kBlockMaxVecs<IO> ? KO_POLICY_BLOCK
-                                         : KO_POLICY_BLOCK_NOCACHE;
+                                      : KO_POLICY_BLOCK;  // rows past what the chip holds stream their far end twice
     }
     switch (policy) {
         case KO_POLICY_WARP:
@@ -635,9 +749,6 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
                             "layernorm: WARP policy holds at most %d columns per row, got %d", kWaveMaxVecs * E, a.cols);
             return launch_wave_any<IO>(a);
         case KO_POLICY_BLOCK:
-            if (nvec > kBlockMaxVecs<IO>)
-                return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "layernorm: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs<IO> * E, a.cols);
             return launch_block<IO>(a);
         case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO>(a);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);

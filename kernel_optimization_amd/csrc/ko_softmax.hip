@@ -108,8 +108,8 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
             // of the row loads.
             const uint64_t r0 = static_cast<uint64_t>(row0);
             const int64_t first_row = static_cast<int64_t>(
-                (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0 >> 32))) << 32) |
-                __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0)));
+                (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0 >> 32)))) << 32) |
+                static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(r0))));
 #pragma unroll
             for (int r = 0; r < RPW; ++r) {
                 const int64_t rr = first_row + r;
@@ -165,14 +165,17 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
         s = wave::allreduce<LPR, wave::Sum>(s);
         const float inv = 1.0f / s;
 
-        typename Io<IO>::elem *dst = out + row * cols;
+        // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
+        typename Io<IO>::elem *dst0 = out + row0 * cols;
+        const uint32_t sub_off = static_cast<uint32_t>(sub) * static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem);
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
             if (row_ok && j < nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
-                Io<IO>::template store<NT>(dst + E * j, v[k]);
+                if constexpr (NT) Io<IO>::store_stream(dst0, sub_off + 16u * j, v[k]);
+                else Io<IO>::template store<false>(dst0 + static_cast<int64_t>(sub) * cols + E * j, v[k]);
             }
         }
     }
@@ -210,18 +213,28 @@ __device__ __forceinline__ float block_allreduce_slot(float v, float *slot, floa
     return r;
 }
 
-// One workgroup per row, the row held in registers between its single read and its single write.  Loads and
+// One workgroup per row, the row held on chip between its single read and its single write.  Loads and
 // stores bypass the caches' retention (nontemporal): every byte is touched once, and on rows of 16 to 128 KB
 // that measured 9 % faster than cached accesses.  Issuing the next row's loads ahead of the reductions
 // measured no different: two or more resident workgroups already cover each other's reductions.
-template <int IO, int THREADS, int VPL, bool MASKED>
+// VPL vectors per thread live in registers.  LV more live in LDS (vector k of thread t at tail[k][t], filled by
+// direct-to-LDS loads, so they cost no registers on the way): a 1024-thread workgroup alone on a CU has 128
+// registers per thread, of which 96 can hold row values, and 9 x 16 KB of the CU's 160 KB of LDS hold the rest
+// of rows up to 135168 fp32 columns, which would otherwise be read twice.  fp32 storage writes the exponentials
+// back into the tail; 16-bit storage keeps the inputs there (eight values per 16 bytes) and takes the
+// exponential again on the way out.
+template <int IO, int THREADS, int VPL, bool MASKED, int LV = 0>
 __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename Io<IO>::elem *in,
                                                                 typename Io<IO>::elem *out, int64_t rows,
                                                                 int cols,
                                                                 const int32_t *__restrict__ valid_len,
                                                                 int64_t rows_per_seq) {
     constexpr int E = Io<IO>::E;
+    static_assert(LV == 0 || !MASKED, "the LDS tail is built for rows without a mask");
+    typedef typename Io<IO>::raw Raw;
     __shared__ float lds[2][16];
+    extern __shared__ __attribute__((aligned(16))) char tail_bytes[];  // Raw tail[LV][THREADS]
+    Raw *tail = reinterpret_cast<Raw *>(tail_bytes);
     const int nvec = cols / E;
     // Byte offset of this thread's first vector in a row (vector k lies k * THREADS * 16 bytes further); passed
     // through an empty asm per row so that addresses are formed per use from the uniform row pointer and this
@@ -247,14 +260,29 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                     for (int e = 0; e < E; ++e) v[k][e] = -INFINITY;
                 }
             }
-        } else {
-            typename Io<IO>::raw loaded[VPL];
+        }
+        typename Io<IO>::raw loaded[(IO == IO_F32 && !MASKED) ? 1 : VPL];
+        if constexpr (!(IO == IO_F32 && !MASKED)) {
 #pragma unroll
             for (int k = 0; k < VPL; ++k) {
                 const int j = threadIdx.x + k * THREADS;
                 loaded[k] = typename Io<IO>::raw{};
                 if (j < nvec) loaded[k] = fetch_row_vec<IO, MASKED, true>(at_bytes(src, first + k * kStep), j, vlen);
             }
+        }
+        if constexpr (LV > 0) {
+            // the tail goes from global memory straight into LDS: each lane's 16 bytes land at the wave's base
+            // plus 16 x lane, i.e. at tail[k][thread]; lanes past the end of the row write nothing
+#pragma unroll
+            for (int k = 0; k < LV; ++k) {
+                const int j = threadIdx.x + (VPL + k) * THREADS;
+                if (j < nvec)
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void *)at_bytes(src, first + (VPL + k) * kStep),
+                        (__attribute__((address_space(3))) void *)(tail + k * THREADS + (threadIdx.x & ~63u)), 16, 0, 0);
+            }
+        }
+        if constexpr (!(IO == IO_F32 && !MASKED)) {
 #pragma unroll
             for (int k = 0; k < VPL; ++k) {
                 const int j = threadIdx.x + k * THREADS;
@@ -268,6 +296,14 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
         float m = -FLT_MAX;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) m = vec_max<E>(v[k], m);
+#pragma unroll
+        for (int k = 0; k < LV; ++k) {
+            if (static_cast<int>(threadIdx.x) + (VPL + k) * THREADS < nvec) {
+                float x[E];
+                Io<IO>::unpack(tail[k * THREADS + threadIdx.x], x);
+                m = vec_max<E>(x, m);
+            }
+        }
         m = block_allreduce_slot<THREADS, wave::Max>(m, lds[0], -FLT_MAX);
         const bool pad_is_zero = MASKED && m > kMaskValue + 128.0f;  // see the wave kernel
         float s = 0.0f;
@@ -284,6 +320,19 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                 }
             }
         }
+#pragma unroll
+        for (int k = 0; k < LV; ++k) {
+            if (static_cast<int>(threadIdx.x) + (VPL + k) * THREADS < nvec) {
+                float x[E];
+                Io<IO>::unpack(tail[k * THREADS + threadIdx.x], x);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    x[e] = exp_for_storage<IO>(x[e] - m);
+                    s += x[e];
+                }
+                if constexpr (IO == IO_F32) tail[k * THREADS + threadIdx.x] = Raw{x[0], x[1], x[2], x[3]};
+            }
+        }
         s = block_allreduce_slot<THREADS, wave::Sum>(s, lds[1], 0.0f);
         const float inv = 1.0f / s;
         typename Io<IO>::elem *dst = out + row * cols;
@@ -293,7 +342,20 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
             if (j < nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
-                Io<IO>::template store<true>(at_bytes(dst, first + k * kStep), v[k]);
+                Io<IO>::store_stream(dst, first + k * kStep, v[k]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < LV; ++k) {
+            if (static_cast<int>(threadIdx.x) + (VPL + k) * THREADS < nvec) {
+                float x[E];
+                Io<IO>::unpack(tail[k * THREADS + threadIdx.x], x);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    if constexpr (IO != IO_F32) x[e] = exp_for_storage<IO>(x[e] - m);
+                    x[e] *= inv;
+                }
+                Io<IO>::store_stream(dst, first + (VPL + k) * kStep, x);
             }
         }
     }
@@ -372,7 +434,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
                 if (j >= nvec) break;
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
-                Io<IO>::template store<true>(dst + E * j, x[u]);
+                Io<IO>::store_stream(dst, 16u * j, x[u]);
             }
         }
     }
@@ -448,10 +510,12 @@ constexpr int kWaveMaxVpl = 8;
 // Longest row per policy, in 16-byte vectors: 512 per wavefront, 8192 per workgroup
 // (fp32: 2048 and 32768 columns; 16-bit: twice that).
 constexpr int kWaveMaxVecs = 64 * kWaveMaxVpl;
-// BLOCK policy: at most 96 values per thread of a 1024-thread workgroup (98304 columns).  With a mask the
+// BLOCK policy: at most 96 values per thread of a 1024-thread workgroup in registers (98304 columns) and, without
+// a mask, nine more 16-byte vectors per thread in LDS (135168 fp32 or 172032 16-bit columns).  With a mask the
 // kernels past 64 values per thread spill registers, and AUTO leaves those rows to the re-reading policy.
+constexpr int kTailMaxVecs = 9;  // of 16 KB each per 1024-thread workgroup, in the 160 KB of LDS of a CU
 template <int IO>
-constexpr int kBlockMaxVecs = 1024 * (96 / Io<IO>::E);
+constexpr int kBlockMaxVecs = 1024 * (96 / Io<IO>::E + kTailMaxVecs);
 template <int IO>
 constexpr int kBlockMaxVecsMasked = 1024 * (64 / Io<IO>::E);
 
@@ -509,13 +573,31 @@ int launch_block_threads(const Args<IO> &a) {
     else if (vpl <= 8) KO_SM_BLOCK(8);
     else if constexpr (THREADS == 1024) {
         // a single resident workgroup of 1024 threads has 128 registers per thread: up to 96 hold the row
+        constexpr int kRegs = 96 / E;  // vectors per thread held in registers
         if constexpr (E == 4) {
             if (vpl <= 12) KO_SM_BLOCK(12);
             else if (vpl <= 16) KO_SM_BLOCK(16);
             else if (vpl <= 20) KO_SM_BLOCK(20);
-            else KO_SM_BLOCK(24);
+            else if (vpl <= 24) KO_SM_BLOCK(24);
         } else if (vpl <= 10) KO_SM_BLOCK(10);
-        else KO_SM_BLOCK(12);
+        else if (vpl <= 12) KO_SM_BLOCK(12);
+        if constexpr (!MASKED) {
+            // longer rows: the rest of the row in LDS (4 or 9 vectors of 16 KB per workgroup)
+            if (vpl > kRegs) {
+                const int lv = vpl - kRegs <= 4 ? 4 : kTailMaxVecs;
+                const void *fn = lv == 4 ? reinterpret_cast<const void *>(softmax_block_kernel<IO, THREADS, kRegs, false, 4>)
+                                         : reinterpret_cast<const void *>(softmax_block_kernel<IO, THREADS, kRegs, false, kTailMaxVecs>);
+                static std::atomic<uint64_t> done4{0}, done9{0};
+                if (const int rc = allow_dynamic_lds(fn, 160 * 1024 - 256, lv == 4 ? done4 : done9); rc != KO_OK) return rc;
+                const size_t bytes = static_cast<size_t>(lv) * THREADS * 16;
+                if (lv == 4)
+                    softmax_block_kernel<IO, THREADS, kRegs, false, 4><<<g, b, bytes, a.stream>>>(
+                        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
+                else
+                    softmax_block_kernel<IO, THREADS, kRegs, false, kTailMaxVecs><<<g, b, bytes, a.stream>>>(
+                        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
+            }
+        }
     }
 #undef KO_SM_BLOCK
     KO_CHECK_LAUNCH();
@@ -572,10 +654,11 @@ int dispatch(const Args<IO> &a, int policy) {
                             a.cols);
             return launch_wave_any<IO, MASKED>(a);
         case KO_POLICY_BLOCK:
-            if (nvec > kBlockMaxVecs<IO>)
+            // with a mask the row has to fit the registers (no LDS tail)
+            if (nvec > (MASKED ? 1024 * (96 / E) : kBlockMaxVecs<IO>))
                 return fail(KO_ERR_UNSUPPORTED_SHAPE,
-                            "softmax: BLOCK policy holds at most %d columns per row, got %d", kBlockMaxVecs<IO> * E,
-                            a.cols);
+                            "softmax: BLOCK policy holds at most %d columns per row%s, got %d",
+                            (MASKED ? 1024 * (96 / E) : kBlockMaxVecs<IO>) * E, MASKED ? " with a mask" : "", a.cols);
             return launch_block<IO, MASKED>(a);
         case KO_POLICY_BLOCK_NOCACHE: return launch_nocache<IO, MASKED>(a);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "softmax: unknown policy %d", policy);

@@ -217,16 +217,30 @@ __device__ __forceinline__ float4v load4(const float *p) {
 // The s_nop behind the store is required: a store of more than 64 bits reads its data registers over several
 // cycles, and a vector-ALU write to them within the next two wait states would change what is stored.  The
 // compiler inserts those wait states for its own stores but does not look inside inline assembly.
+// The address is a wave-uniform base (in scalar registers) plus a 32-bit byte offset per lane: with a 64-bit
+// address per lane the register allocator, which cannot move or merge inline assembly, spilled in the kernels
+// that hold 96 row values per thread.  `uniform_base` MUST have the same value in every lane of the wavefront
+// (the compiler reads it from the first active lane if it cannot prove that).
 template <class V>
-__device__ __forceinline__ void stream_store16(V *q, V v) {
+__device__ __forceinline__ void stream_store16(void *uniform_base, uint32_t byte_offset, V v) {
     static_assert(sizeof(V) == 16, "");
-    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(q), "v"(v));
+    // through readfirstlane: the "s" constraint alone does not move a value the compiler holds in vector
+    // registers (a row pointer derived from threadIdx.x >> 6, say) into scalar ones
+    const uint64_t b = reinterpret_cast<uint64_t>(uniform_base);
+    // (the builtin returns int: each half goes through uint32_t, or the low half would be sign-extended)
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32)));
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b)));
+    const uint64_t base = (static_cast<uint64_t>(hi) << 32) | lo;
+    // s_nop 4 in front: the base reaches its scalar registers through v_readfirstlane, a vector-ALU write of
+    // scalar registers, and a memory instruction may read such a register only five wait states later.  The
+    // compiler keeps that distance for its own instructions but cannot see that this assembly reads them.
+    asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 sc1 nt\n\ts_nop 1" ::"v"(byte_offset), "v"(v), "s"(base));
 }
 
 template <bool NT>
 __device__ __forceinline__ void store4(float *p, float4v v) {
     float4v *q = reinterpret_cast<float4v *>(p);
-    if constexpr (NT) stream_store16(q, v);
+    if constexpr (NT) __builtin_nontemporal_store(v, q);
     else *q = v;
 }
 
@@ -260,6 +274,10 @@ struct Io<IO_F32> {
     static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
         store4<NT>(p, float4v{v[0], v[1], v[2], v[3]});
     }
+    // streaming store of one vector at uniform_base + byte_offset (see stream_store16)
+    static __device__ __forceinline__ void store_stream(elem *uniform_base, uint32_t byte_offset, const float (&v)[E]) {
+        stream_store16(uniform_base, byte_offset, float4v{v[0], v[1], v[2], v[3]});
+    }
     static __device__ __forceinline__ float scalar(const elem *p) { return *p; }
 };
 
@@ -273,7 +291,7 @@ __device__ __forceinline__ uint4v load_bits16(const uint16_t *p) {
 template <bool NT>
 __device__ __forceinline__ void store_bits16(uint16_t *p, uint4v v) {
     uint4v *q = reinterpret_cast<uint4v *>(p);
-    if constexpr (NT) stream_store16(q, v);
+    if constexpr (NT) __builtin_nontemporal_store(v, q);
     else *q = v;
 }
 
@@ -302,6 +320,12 @@ struct Io<IO_F16> {
 #pragma unroll
         for (int e = 0; e < E; ++e) h[e] = static_cast<_Float16>(v[e]);
         store_bits16<NT>(p, __builtin_bit_cast(uint4v, h));
+    }
+    static __device__ __forceinline__ void store_stream(elem *uniform_base, uint32_t byte_offset, const float (&v)[E]) {
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < E; ++e) h[e] = static_cast<_Float16>(v[e]);
+        stream_store16(uniform_base, byte_offset, __builtin_bit_cast(uint4v, h));
     }
     static __device__ __forceinline__ float scalar(const elem *p) {
         return static_cast<float>(__builtin_bit_cast(_Float16, *p));
@@ -339,30 +363,40 @@ struct Io<IO_BF16> {
             x[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{v[2 * e], v[2 * e + 1]}, bf16x2));
         store_bits16<NT>(p, x);
     }
+    static __device__ __forceinline__ void store_stream(elem *uniform_base, uint32_t byte_offset, const float (&v)[E]) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        uint4v x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            x[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{v[2 * e], v[2 * e + 1]}, bf16x2));
+        stream_store16(uniform_base, byte_offset, x);
+    }
     static __device__ __forceinline__ float scalar(const elem *p) {
         return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
     }
 };
 
-// exp(d) for d <= 0, about 1 ulp: d*log2(e) is formed as a rounded product plus its
-// exact residual and the low part of log2(e), the integer part is split off and
-// applied with ldexp, and the hardware base-2 exponential (v_exp_f32) only sees a
-// fraction in [-0.5, 0.5].  Arguments below -128 (minus infinity included) are clamped:
-// the result is 0 either way.  A NaN argument gives NaN - the clamp is a compare and
-// select, not fmaxf, which would return the clamp value for a NaN - so that a NaN or
-// a +inf element (inf - inf) poisons its row's sum as it does with expf in the
-// reference (nn_operators/softmax/softmax.h:46).
+// exp(d) for d <= 0, within 2 ulp: 2^y (1 + r ln 2), where y = d * log2(e) is the rounded product, r its exact
+// residual plus d times the low part of log2(e) (|r| <= 2^-24 |y|, so the first-order term is all that matters),
+// and 2^y is the hardware base-2 exponential (v_exp_f32: 1 ulp over its whole range; results below 2^-126 are
+// flushed to zero, which no gate here can see: they are below FLT_MIN relative to a sum of at least 1).  Eight
+// vector-ALU operations per value; splitting off the integer part and applying it with ldexp took twelve, and on
+// rows that fill a workgroup's registers that arithmetic is time during which the compute unit requests no memory.
+// Arguments below -128 (minus infinity included) are clamped: the result is 0 either way.  A NaN argument gives
+// NaN - the clamp is a compare and select, not fmaxf, which would return the clamp value for a NaN - so that a NaN
+// or a +inf element (inf - inf) poisons its row's sum as it does with expf in the reference
+// (nn_operators/softmax/softmax.h:46).
 __device__ __forceinline__ float exp_nonpositive(float d) {
     const float kLog2eHi = 0x1.715476p+0f;
     const float kLog2eLo = 0x1.4ae0cp-26f;
+    const float kLn2 = 0x1.62e43p-1f;
     d = d < -128.0f ? -128.0f : d;
-    float y = d * kLog2eHi;
+    const float y = d * kLog2eHi;
     float r = __builtin_fmaf(d, kLog2eHi, -y);
     r = __builtin_fmaf(d, kLog2eLo, r);
-    float n = __builtin_rintf(y);
-    float f = (y - n) + r;
-    float e = __builtin_amdgcn_exp2f(f);
-    return __builtin_ldexpf(e, static_cast<int>(n));
+    const float e = __builtin_amdgcn_exp2f(y);
+    return __builtin_fmaf(e * r, kLn2, e);
 }
 
 // exp(d) for d <= 0 where the result is rounded to bfloat16 afterwards (which keeps fp32's exponent range, so

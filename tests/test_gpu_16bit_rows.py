@@ -45,7 +45,8 @@ def test_softmax16_every_lane_mapping(ko, lpr, bf16):
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("policy,rows,cols", [(2, 37, 128), (2, 19, 1024), (2, 5, 16384), (2, 3, 65536), (2, 11, 5000),
                                               (2, 2, 81920), (2, 2, 98304), (0, 2, 98304),
-                                              (3, 37, 128), (3, 4, 40000), (3, 2, 262144), (0, 3, 8192), (0, 2, 131072)])
+                                              (3, 37, 128), (3, 4, 40000), (3, 2, 262144), (0, 3, 8192), (0, 2, 131072),
+                                              (2, 2, 131072), (2, 2, 172032), (0, 2, 172040)])
 def test_softmax16_block_policies(ko, policy, rows, cols, bf16):
     xb = _bits(inputs.normal_f32((rows, cols), 70 + cols, 0.0, 4.0), bf16)
     _, ref64 = oracle.softmax16(xb, bf16=bf16)
@@ -103,7 +104,8 @@ def test_layernorm16_matches_oracle(ko, rows, cols, unbiased, bf16):
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("policy,rows,cols", [(2, 37, 128), (2, 19, 1024), (2, 5, 16384), (2, 3, 32768),
                                               (2, 2, 65536), (2, 2, 81920), (0, 2, 81920),
-                                              (3, 37, 128), (3, 4, 40000), (0, 3, 8192), (0, 2, 65536), (0, 2, 131072)])
+                                              (3, 37, 128), (3, 4, 40000), (0, 3, 8192), (0, 2, 65536), (0, 2, 131072),
+                                              (2, 2, 98304), (2, 2, 139264), (2, 2, 139272), (2, 1, 300000)])
 def test_layernorm16_block_policies(ko, policy, rows, cols, bf16):
     xb = _bits(inputs.normal_f32((rows, cols), 110 + cols, 0.5, 2.0), bf16)
     gb = _bits(inputs.normal_f32((cols,), 111, 1.0, 0.1), bf16)
@@ -124,8 +126,6 @@ def test_layernorm16_plain_in_place_and_errors(ko, bf16):
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 12, 1e-5, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 16, 1e-5, 0, 9, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 0, 16, 1e-5, 0, dt, 0, None) == ko.KO_OK
-    # the row-per-workgroup policy holds 81920 columns
-    assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 1, 98304, 1e-5, 0, dt, 2, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
 
 
 @pytest.mark.parametrize("bf16", [False, True])

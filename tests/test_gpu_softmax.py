@@ -49,7 +49,9 @@ def test_softmax_every_lane_mapping(ko, lpr, cols):
     (2, 37, 128), (2, 19, 1024), (2, 9, 4096), (2, 5, 8192), (2, 3, 32768), (2, 11, 5000),
     (2, 3, 40960), (2, 2, 49152), (2, 3, 65536), (2, 2, 81920), (2, 3, 98304), (2, 2, 70004), (2, 5000, 2052),
     (3, 5000, 2052), (3, 37, 128), (3, 19, 1024), (3, 4, 40000), (3, 2, 131072),
-    (0, 3, 4096), (0, 2, 65536), (0, 2, 98304), (0, 2, 98308)])
+    (0, 3, 4096), (0, 2, 65536), (0, 2, 98304), (0, 2, 98308),
+    # past the registers of a workgroup: up to nine more vectors per thread in LDS
+    (2, 3, 98308), (2, 2, 114688), (2, 3, 114692), (2, 2, 131072), (2, 3, 135168), (0, 2, 131072), (0, 2, 135172)])
 def test_softmax_block_policies(ko, policy, rows, cols):
     """Row-per-workgroup (BLOCK) and re-read (BLOCK_NOCACHE) policies, and AUTO on long rows."""
     x = inputs.normal_f32((rows, cols), 4321 + cols, 0.0, 4.0)
@@ -155,10 +157,14 @@ def test_softmax_errors(ko):
         ko.softmax(buf, buf, 1, 4096, policy=1)  # WARP policy holds at most 2048 columns
     assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert "WARP" in str(e.value)
-    big = ko.DeviceBuffer(131072 * 4)
+    big = ko.DeviceBuffer(135172 * 4)
     with pytest.raises(ko.KoError) as e:
-        ko.softmax(big, big, 1, 131072, policy=2)  # BLOCK policy holds at most 98304 columns
+        ko.softmax(big, big, 1, 135172, policy=2)  # BLOCK policy holds at most 135168 columns (registers + LDS)
     assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE and "BLOCK" in str(e.value)
+    vl = ko.DeviceBuffer.from_numpy(np.array([100], np.int32))
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(big, big, 1, 131072, valid_len=vl, rows_per_seq=1, policy=2)  # with a mask: registers only
+    assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE and "mask" in str(e.value)
 
 
 def test_softmax_full_size_cfg1_properties(ko):

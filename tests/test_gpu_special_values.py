@@ -26,7 +26,7 @@ def _to64(bits, bf16):
 
 # policy, cols: WARP at several lane mappings (ragged 260 and 1000 leave empty vector slots), BLOCK, re-read
 SOFTMAX_SHAPES = [(1, 128), (1, 512), (1, 260), (1, 1000), (1, 2048), (2, 128), (2, 4096), (2, 5000), (2, 40960),
-                  (3, 128), (3, 5000), (3, 40000), (0, 768)]
+                  (3, 128), (3, 5000), (3, 40000), (0, 768), (2, 131072)]
 
 
 @pytest.mark.parametrize("policy,cols", SOFTMAX_SHAPES)
@@ -78,7 +78,8 @@ def test_softmax16_special_values(ko, policy, cols, bf16):
 
 
 @pytest.mark.parametrize("policy,cols", [(1, 128), (1, 768), (1, 260), (1, 1000), (1, 2048), (2, 768), (2, 4096),
-                                         (2, 5000), (2, 40960), (3, 768), (3, 5000), (3, 40000), (0, 1024)])
+                                         (2, 5000), (2, 40960), (3, 768), (3, 5000), (3, 40000), (0, 1024),
+                                         (2, 131072)])
 @pytest.mark.parametrize("affine", [True, False])
 def test_layernorm_special_values(ko, policy, cols, affine):
     base = inputs.normal_f32((5, cols), 700 + cols, 0.5, 2.0)
