@@ -645,7 +645,9 @@ int launch_block_threads(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + THREADS - 1) / THREADS;
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
+    if (tuning(knob_rows_block_grid) == 1) grid = a.rows;  // one workgroup per row
     if (grid > a.rows) grid = a.rows;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     dim3 g(static_cast<unsigned>(grid)), b(THREADS);
 #define KO_LN_BLOCK(V)                                                                                 \
     layernorm_block_kernel<IO, THREADS, V><<<g, b, 0, a.stream>>>(a.in, a.out, a.mean, a.rstd, a.gamma, \
@@ -700,7 +702,9 @@ int launch_block(const Args<IO> &a) {
 template <int IO, int THREADS>
 int launch_nocache_threads(const Args<IO> &a) {
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
+    if (tuning(knob_rows_block_grid) == 1) grid = a.rows;  // one workgroup per row
     if (grid > a.rows) grid = a.rows;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     layernorm_nocache_kernel<IO, THREADS><<<dim3(static_cast<unsigned>(grid)), dim3(THREADS), 0, a.stream>>>(
         a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
     KO_CHECK_LAUNCH();

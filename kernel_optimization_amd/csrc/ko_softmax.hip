@@ -518,6 +518,10 @@ template <int IO>
 constexpr int kBlockMaxVecs = 1024 * (96 / Io<IO>::E + kTailMaxVecs);
 template <int IO>
 constexpr int kBlockMaxVecsMasked = 1024 * (64 / Io<IO>::E);
+// AUTO goes to the re-reading policy from five LDS vectors on: with one workgroup per CU either way, nine of them
+// cost about what the second read does ([1024, 131072]: 244 against 238 us; [1170, 114688], four: 218 against 236).
+template <int IO>
+constexpr int kBlockAutoMaxVecs = 1024 * (96 / Io<IO>::E + 4);
 
 // Lanes per row for the WARP policy.  A group of LPR lanes holds a row in VPL vectors per lane, VPL from
 // {1, 2, 3, 4, 6, 8}; the choice wastes the fewest vector slots (idle lanes still cost issue cycles
@@ -561,7 +565,11 @@ int launch_block_threads(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + THREADS - 1) / THREADS;
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
+    // one workgroup per row for rows of at most two vectors per thread (see launch_block); knob: 1 always, 2 never
+    const int grid_knob = tuning(knob_rows_block_grid);
+    if (grid_knob == 1 || (grid_knob != 2 && vpl <= 2 && THREADS >= 512)) grid = a.rows;
     if (grid > a.rows) grid = a.rows;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     dim3 g(static_cast<unsigned>(grid)), b(THREADS);
 #define KO_SM_BLOCK(V)                                                                         \
     softmax_block_kernel<IO, THREADS, V, MASKED><<<g, b, 0, a.stream>>>(                         \
@@ -609,8 +617,17 @@ int launch_block(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     int threads = tuning(knob_softmax_block_threads);
     if (threads != 256 && threads != 512 && threads != 1024) {
-        threads = 256;
-        while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;
+        // Rows of up to two vectors per thread of a big workgroup: 512 or 1024 threads and one workgroup per row,
+        // dispatched in row order (like the wave kernels and the plain copy, a one-shot launch beats a grid that
+        // walks the rows: [32768, 4096] 183 -> 164 us = 0.98 of the same-bytes copy, [16384, 8192] 188 -> 168 us).
+        // Longer rows: up to four vectors per thread before the workgroup grows, and a grid of two workgroups
+        // per resident slot walking the rows.
+        if (nvec <= 1024) threads = 512;
+        else if (nvec <= 2048) threads = 1024;
+        else {
+            threads = 256;
+            while (threads < 1024 && (nvec + threads - 1) / threads > 4) threads <<= 1;
+        }
     }
     while (threads < 1024 && (nvec + threads - 1) / threads > 8) threads <<= 1;
     if (threads == 256) return launch_block_threads<IO, 256, MASKED>(a);
@@ -621,7 +638,9 @@ int launch_block(const Args<IO> &a) {
 template <int IO, int THREADS, bool MASKED>
 int launch_nocache_threads(const Args<IO> &a) {
     int64_t grid = static_cast<int64_t>(compute_units()) * (2048 / THREADS) * 2;
+    if (tuning(knob_rows_block_grid) == 1) grid = a.rows;  // one workgroup per row
     if (grid > a.rows) grid = a.rows;
+    if (grid > 0x7fffffff) grid = 0x7fffffff;
     softmax_nocache_kernel<IO, THREADS, MASKED><<<dim3(static_cast<unsigned>(grid)), dim3(THREADS), 0, a.stream>>>(
         a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
     KO_CHECK_LAUNCH();
@@ -643,7 +662,7 @@ int dispatch(const Args<IO> &a, int policy) {
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
-                 : nvec <= (MASKED ? kBlockMaxVecsMasked<IO> : kBlockMaxVecs<IO>) ? KO_POLICY_BLOCK
+                 : nvec <= (MASKED ? kBlockMaxVecsMasked<IO> : kBlockAutoMaxVecs<IO>) ? KO_POLICY_BLOCK
                                          : KO_POLICY_BLOCK_NOCACHE;
     }
     switch (policy) {
