@@ -640,11 +640,14 @@ def main():
         del k2
         res["steps"], res["warmup"] = args.steps, args.warmup
         others.append(res)
-        for op, rows, cols, policy in (("softmax", 49152, 1024, ko.POLICY_WARP), ("softmax", 8192, 16384, ko.POLICY_BLOCK),
+        for op, rows, cols, policy in (("softmax", 49152, 1024, ko.POLICY_WARP), ("softmax", 32768, 4096, ko.POLICY_BLOCK),
+                                       ("softmax", 8192, 16384, ko.POLICY_BLOCK),
                                        ("softmax", 2048, 65536, ko.POLICY_BLOCK),
                                        ("softmax", 1024, 131072, ko.POLICY_BLOCK_NOCACHE),
+                                       ("layernorm", 32768, 4096, ko.POLICY_BLOCK),
                                        ("layernorm", 8192, 16384, ko.POLICY_BLOCK),
                                        ("layernorm", 2048, 65536, ko.POLICY_BLOCK),
+                                       ("layernorm", 1024, 131072, ko.POLICY_BLOCK),
                                        ("layernorm", 1024, 131072, ko.POLICY_BLOCK_NOCACHE)):
             res = bench_long_rows(op, rows, cols, policy, args.steps, args.warmup)
             res["steps"], res["warmup"] = args.steps, args.warmup

@@ -42,9 +42,9 @@ typedef enum ko_status {
  * BLOCK_NOCACHE = row per workgroup, row re-read from global memory
  *         (SoftMaxBlockNoCacheImpl softmax.h:116-166, LayerNormBlockNoCacheImpl layernorm.h:254-300)
  * AUTO  = chosen from the row length: the first of the three that holds the row.
- * Longest rows: WARP 2048 fp32 / 4096 16-bit columns; BLOCK 98304 columns for softmax, 81920 for
- * LayerNorm; BLOCK_NOCACHE any length.  A policy asked for explicitly on a longer row returns
- * KO_ERR_UNSUPPORTED_SHAPE. */
+ * Longest rows: WARP 2048 fp32 / 4096 16-bit columns; BLOCK softmax 135168 fp32 / 172032 16-bit columns
+ * (98304 columns with a padding mask), LayerNorm any length (what the chip does not hold is read twice);
+ * BLOCK_NOCACHE any length.  A policy asked for explicitly on a longer row returns KO_ERR_UNSUPPORTED_SHAPE. */
 typedef enum ko_policy {
     KO_POLICY_AUTO = 0,
     KO_POLICY_WARP = 1,
