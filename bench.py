@@ -660,6 +660,10 @@ def main():
         res, _ = bench_sgemm(3, args.steps, args.warmup, vendor, shape=(4000, 4000, 4000))
         res["steps"], res["warmup"] = args.steps, args.warmup
         others.append(res)
+        # a deep K on few tiles: K cut into slices that run side by side, partial products summed by a second kernel
+        res, _ = bench_sgemm(3, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(256, 256, 2048))
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16000, 3072, 768))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)

@@ -155,7 +155,14 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * C may be NULL (then beta is ignored); the reference's epilogue is alpha = beta = 1
  * with C given, or D = A*B with C null (simt_gemm.h:325-373).
  * m, n multiples of 4 are not required; any positive sizes are accepted.  m == 0 or n == 0 is a no-op;
- * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries. */
+ * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries.
+ * Workspace: a problem with few output tiles and a deep K (tiles for at most half of the compute units,
+ * k >= 768, operand rows on 16-byte boundaries) is cut into slices of K that run side by side; their partial
+ * products go through 8 MiB of device memory that the library allocates at the first such call on a
+ * (device, stream) pair and keeps until the process ends.  Calls on different streams therefore never share
+ * it.  A first such call made while the stream is being captured into a graph allocates nothing and takes
+ * the unsliced kernels; so does every call once 64 pairs hold a workspace.  Results do not depend on the
+ * timing of the slices (summed in slice order), but the sliced and the unsliced path round differently. */
 int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
                  float beta, const float *C, float *D, ko_stream_t stream);
 

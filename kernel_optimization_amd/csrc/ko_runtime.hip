@@ -4,6 +4,7 @@
 #include "ko_internal.h"
 
 #include <cstring>
+#include <mutex>
 
 namespace ko {
 
@@ -63,6 +64,35 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
     if (bit && (done.load(std::memory_order_acquire) & bit)) return KO_OK;
     KO_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
     if (bit) done.fetch_or(bit, std::memory_order_release);
+    return KO_OK;
+}
+
+int stream_workspace(hipStream_t stream, void **workspace) {
+    struct Entry { int device; hipStream_t stream; void *memory; };
+    constexpr int kMaxEntries = 64;
+    static Entry entries[kMaxEntries];
+    static int used = 0;
+    static std::mutex lock;
+    *workspace = nullptr;
+    int dev = 0;
+    KO_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> guard(lock);
+    for (int i = 0; i < used; ++i)
+        if (entries[i].device == dev && entries[i].stream == stream) {
+            *workspace = entries[i].memory;
+            return KO_OK;
+        }
+    if (used == kMaxEntries) return KO_OK;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        return KO_OK;
+    }
+    if (capture != hipStreamCaptureStatusNone) return KO_OK;
+    void *memory = nullptr;
+    KO_HIP(hipMalloc(&memory, kStreamWorkspaceBytes));
+    entries[used++] = Entry{dev, stream, memory};
+    *workspace = memory;
     return KO_OK;
 }
 

@@ -60,7 +60,22 @@ struct Params {
     int tiles_n;
     int blocked;  // 1: the tile grid is cut into 4 x 8 blocks, one per XCD and round (see tile_of)
     int lda;      // floats between rows of A (K, or more when A is a column range of a wider matrix)
+    int k_slice;  // 0, or: workgroups with blockIdx.y = s multiply columns [s * k_slice, (s + 1) * k_slice) of A by
+                  // the same rows of B and write their M x N partial product (alpha 1, no C) behind D + s * M * N
 };
+
+// The problem a workgroup of a K-sliced launch works on: its slice of A and B and its own partial product.
+__device__ __forceinline__ Params slice_of(Params p) {
+    if (p.k_slice > 0) {
+        const int s = static_cast<int>(blockIdx.y);
+        const int k0 = s * p.k_slice;
+        p.A += k0;
+        p.B += static_cast<int64_t>(k0) * p.N;
+        p.D += static_cast<int64_t>(s) * p.M * p.N;
+        p.K = p.K - k0 < p.k_slice ? p.K - k0 : p.k_slice;
+    }
+    return p;
+}
 
 // Workgroup -> output tile.  Workgroups go to the 8 XCDs round-robin by index, each XCD has its own
 // L2 and runs 32 workgroups at a time (one per compute unit).  In the blocked order workgroups
@@ -409,7 +424,8 @@ __device__ __attribute__((aligned(16))) const float zero_chunk[4] = {0.0f, 0.0f,
 // waits are inline assembly.  Registers filled by such a read pass through an empty assembly statement
 // behind the wait before the MFMAs use them, which keeps every use (and every copy) behind the wait.
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, bool EDGE>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_kernel(const Params p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_kernel(const Params whole) {
+    const Params p = slice_of(whole);
     constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -617,6 +633,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, bool PIPE = false>
 int launch(Params p, hipStream_t stream) {
     constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
+    if (p.k_slice > 0) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: this tiling takes no K slices");
     const int tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
@@ -649,8 +666,13 @@ int launch_direct(Params p, hipStream_t stream) {
     // Operand rows have to start on 16-byte boundaries and K must not end inside a 16-byte chunk.
     const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                          p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
+    if (!aligned && p.k_slice > 0) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: K slices need 16-byte aligned operand rows");
     if (!aligned) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
-    const bool edge = p.M % BM != 0 || p.N % BN != 0 || p.K % (2 * BK) != 0;
+    // K-sliced launches: every slice but the last is k_slice deep (a multiple of 4), the last takes the rest.
+    const int slices = p.k_slice > 0 ? (p.K + p.k_slice - 1) / p.k_slice : 1;
+    const int k_last = p.K - (slices - 1) * (p.k_slice > 0 ? p.k_slice : 0);
+    const int k_each = slices > 1 ? p.k_slice : p.K;
+    const bool edge = p.M % BM != 0 || p.N % BN != 0 || k_each % (2 * BK) != 0 || k_last % (2 * BK) != 0;
     const int tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t nblocks = static_cast<int64_t>(tiles_m) * p.tiles_n;
@@ -662,14 +684,54 @@ int launch_direct(Params p, hipStream_t stream) {
     static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge]); st != KO_OK)
         return st;
-    kernel<<<dim3(static_cast<unsigned>(nblocks)), dim3(THREADS), lds_bytes, stream>>>(p);
+    kernel<<<dim3(static_cast<unsigned>(nblocks), static_cast<unsigned>(slices)), dim3(THREADS), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
+// D = alpha * (P_0 + P_1 + ... + P_{slices-1}) + beta * C over the M x N partial products a K-sliced launch
+// left behind `partials`, summed in slice order whatever order the slices finished in.
+// One 64-lane workgroup per 256 (VEC) or 64 outputs: the problems that are sliced have few outputs, and small
+// workgroups spread them over more compute units.  The partial products of eight slices are fetched together
+// (they come from memory behind the L2s: another XCD wrote them) and added one after the other.
+template <bool VEC>
+__global__ __launch_bounds__(64) void sgemm_slices_sum_kernel(const float *__restrict__ partials, int slices,
+                                                              int64_t count, float alpha, float beta,
+                                                              const float *__restrict__ C, float *__restrict__ D) {
+    constexpr int W = VEC ? 4 : 1;
+    typedef float vec_t __attribute__((ext_vector_type(W)));
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x) * W;
+    if (i >= count) return;
+    const float *src = partials + i;
+    vec_t acc = *reinterpret_cast<const vec_t *>(src);
+    int s = 1;
+    for (; s + 8 <= slices; s += 8) {
+        vec_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const vec_t *>(src + (s + j) * count);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += v[j];
+    }
+    for (; s < slices; ++s) acc += *reinterpret_cast<const vec_t *>(src + s * count);
+    acc *= alpha;
+    if (C != nullptr && beta != 0.0f) acc += beta * *reinterpret_cast<const vec_t *>(C + i);
+    __builtin_nontemporal_store(acc, reinterpret_cast<vec_t *>(D + i));
+}
+
+int sum_slices(const float *partials, int slices, const Params &p, hipStream_t stream) {
+    const int64_t count = static_cast<int64_t>(p.M) * p.N;
+    const bool vec = count % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.C) | reinterpret_cast<uintptr_t>(p.D)) & 15) == 0;
+    const int64_t threads = vec ? count / 4 : count;
+    const dim3 grid(static_cast<unsigned>((threads + 63) / 64));
+    if (vec) sgemm_slices_sum_kernel<true><<<grid, 64, 0, stream>>>(partials, slices, count, p.alpha, p.beta, p.C, p.D);
+    else sgemm_slices_sum_kernel<false><<<grid, 64, 0, stream>>>(partials, slices, count, p.alpha, p.beta, p.C, p.D);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
 
 // One launch: the tiling by shape (variant <= 0) or the one asked for.
 int run(Params p, hipStream_t s, int variant) {
-    const int64_t m = p.M, n = p.N, k = p.K;
+    const int64_t m = p.M, n = p.N, k = p.k_slice > 0 ? p.k_slice : p.K;
     if (variant <= 0) {
         // Few tiles (fewer 128 x 128 tiles than compute units): 64 x 64 tiles with K split four ways inside
         // the workgroup; otherwise 128 x 128 tiles with K split two ways (2048^3, one tile per compute unit:
@@ -708,6 +770,49 @@ int run(Params p, hipStream_t s, int variant) {
     }
 }
 
+// K slices for problems that are deep and have few output tiles (256 x 256 x 2048: 32 tiles of 32 x 64 on 256
+// compute units).  The slices are workgroups of one launch (blockIdx.y); their partial products go to
+// `workspace_bytes` of device memory and a second kernel sums them in slice order, so the result does not
+// depend on which slice finished first.  Returns the slice count (1: do not slice) and the slice depth.
+//   - operands as the direct-to-LDS kernels want them (rows on 16-byte boundaries);
+//   - tiles for at most half of the compute units, and as many slices as bring the launch up to one
+//     workgroup per compute unit, each at least 256 deep and a multiple of 128 (whole pairs of K tiles).
+int plan_k_slices(const Params &p, size_t workspace_bytes, int *k_slice) {
+    *k_slice = 0;
+    const int forced = tuning(knob_sgemm_k_slices);
+    if (forced == 1) return 1;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
+                         p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
+    if (!aligned) return 1;
+    const int64_t cu = compute_units();
+    const int64_t t64 = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+    const int64_t tiles = 2 * t64 <= cu ? ((p.M + 31) / 32) * ((p.N + 63) / 64) : t64;  // as run() picks the tiling
+    // The second launch costs 2-3 us: below K = 768 the slices do not win them back (256 x 256 x 512: 7.0 us
+    // whole, 7.5 us in two slices; K = 768: 9.2 against 8.3; K = 2048: 19.8 against 11.1).
+    if (forced < 2 && p.K < 768) return 1;
+    int64_t slices = forced >= 2 ? forced : cu / tiles;
+    if (forced < 2 && slices > p.K / 256) slices = p.K / 256;
+    if (slices < 2) return 1;
+    const int64_t depth = ((p.K + slices - 1) / slices + 127) / 128 * 128;
+    slices = (p.K + depth - 1) / depth;
+    if (slices < 2 || slices > 65535) return 1;
+    if (static_cast<uint64_t>(slices) * p.M * p.N * sizeof(float) > workspace_bytes) return 1;
+    *k_slice = static_cast<int>(depth);
+    return static_cast<int>(slices);
+}
+
+// The K-sliced form of one problem: partial products into `workspace`, then their sum and the epilogue.
+int run_sliced(const Params &p, int slices, int k_slice, float *workspace, hipStream_t s) {
+    Params part = p;
+    part.C = nullptr;
+    part.D = workspace;
+    part.alpha = 1.0f;
+    part.beta = 0.0f;
+    part.k_slice = k_slice;
+    if (const int st = run(part, s, 0); st != KO_OK) return st;
+    return sum_slices(workspace, slices, p, s);
+}
+
 }  // namespace
 }  // namespace ko
 
@@ -721,9 +826,17 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     if (k == 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: k must be positive");
     if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: dimension too large");
     if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
-    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, static_cast<int>(k)};
+    Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, static_cast<int>(k), 0};
     hipStream_t s = as_stream(stream);
     const int variant = tuning(knob_sgemm_variant);
+    if (variant <= 0) {
+        int k_slice = 0;
+        if (const int slices = plan_k_slices(p, kStreamWorkspaceBytes, &k_slice); slices > 1) {
+            void *workspace = nullptr;
+            if (const int st = stream_workspace(s, &workspace); st != KO_OK) return st;
+            if (workspace != nullptr) return run_sliced(p, slices, k_slice, static_cast<float *>(workspace), s);
+        }
+    }
     if (variant <= 0 && tuning(knob_sgemm_split_rows) != 1 && k >= 512) {
         // A last round of 128 x 128 tiles that fills at most half of the compute units costs a whole round:
         // the tile rows that fill whole rounds go out as one launch, the rows below them as a second one

@@ -76,6 +76,50 @@ def test_sgemm_uneven_last_round_goes_out_as_two_launches(ko, m, n, k):
         ko.set_tuning("sgemm.split_rows", 0)
 
 
+@pytest.fixture
+def sgemm_k_slices(ko):
+    """Sets the slice count (0: by shape, 1: never, n: n slices) and puts the default back afterwards."""
+    yield lambda value: ko.set_tuning("sgemm.k_slices", value)
+    ko.set_tuning("sgemm.k_slices", 0)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 2048), (128, 64, 4096), (100, 200, 3000), (33, 68, 1300), (512, 512, 8192),
+                                   (64, 64, 516), (1, 4, 16384), (320, 192, 1024)])
+def test_sgemm_deep_k_on_few_tiles_is_cut_into_slices(ko, sgemm_k_slices, m, n, k):
+    """Few output tiles and a deep K: the default dispatch cuts K into slices that run as workgroups of one
+    launch and sums their partial products in a second kernel.  Small integers make every product and sum
+    exact, so a slice that starts at the wrong k, overlaps its neighbour, pads with anything but zeros or
+    lands at the wrong place of the partial products shows as a wrong integer.  The unsliced path and forced
+    slice counts (ragged last slices among them) must give the same matrix."""
+    rng = np.random.default_rng(m + n + k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    for slices in (0, 1, 2, 3, 7):
+        sgemm_k_slices(slices)
+        np.testing.assert_array_equal(ko.sgemm_host(A, B), ref, err_msg=f"k_slices={slices}")
+        np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=f"k_slices={slices}")
+
+
+def test_sgemm_k_slices_against_oracle_and_repeatable(ko, sgemm_k_slices):
+    """Uniform inputs through the sliced path: within the fp32 summation bound of the oracle, bit-identical
+    from call to call (the partial products are summed in slice order, not in order of arrival), and the
+    epilogue (alpha, beta, C) is applied once, to the sum."""
+    m, n, k = 256, 256, 2048
+    A, B = inputs.uniform_f32((m, k), 21), inputs.uniform_f32((k, n), 22)
+    C = inputs.normal_f32((m, n), 23)
+    ref, ap = oracle.sgemm(A, B, want_absprod=True)
+    first = ko.sgemm_host(A, B)
+    assert_sgemm_close(first, ref, ap, k)
+    for _ in range(3):
+        np.testing.assert_array_equal(ko.sgemm_host(A, B), first)
+    ref2, ap2 = oracle.sgemm(A, B, C, 0.5, -2.0, want_absprod=True)
+    assert_sgemm_close(ko.sgemm_host(A, B, C, 0.5, -2.0), ref2, 0.5 * ap2 + 2.0 * np.abs(C) + 1e-6, k)
+    sgemm_k_slices(1)
+    assert_sgemm_close(ko.sgemm_host(A, B), ref, ap, k)
+
+
 def test_sgemm_cfg3_full(ko):
     """1024^3, U(-1,1), alpha=1, beta=0, C null: the whole output against the oracle, with the
     reference's own abs <= 1e-3 gate (nn_operators/gemm/main.cu:169-170) as well."""

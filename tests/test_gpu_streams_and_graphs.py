@@ -1,6 +1,6 @@
 """The operators are plain kernel launches on the caller's stream, so a caller can capture them into a HIP graph
 (the reference's drivers launch on one non-blocking stream as well, softmax/main.cu:28-29).  This test captures a
-softmax -> LayerNorm -> 16-bit GEMM -> SGEMM -> 16-bit GEMM (persistent kernel) sequence with the HIP runtime that libko.so itself is linked against,
+softmax -> LayerNorm -> 16-bit GEMM -> SGEMM -> 16-bit GEMM (persistent kernel) -> K-sliced SGEMM sequence with the HIP runtime that libko.so itself is linked against,
 replays the graph several times with eager work and synchronisations in between, and compares every replay bit
 for bit with the eager results.  One eager pass comes first: the library's one-time set-up (device properties,
 kernel attributes) is not stream work and belongs in front of a capture."""
@@ -49,6 +49,10 @@ def test_operators_replay_from_a_hip_graph(ko):
     a2, b2, d2 = ko.DeviceBuffer(m2 * k2 * 2), ko.DeviceBuffer(n2 * k2 * 2), ko.DeviceBuffer(m2 * n2 * 2)
     m3, n3, k3 = 8000, 2312, 256  # cut along columns and twice along rows: the most launches behind one call
     a3, b3, d3 = ko.DeviceBuffer(m3 * k3 * 2), ko.DeviceBuffer(n3 * k3 * 2), ko.DeviceBuffer(m3 * n3 * 2)
+    m4, n4, k4 = 256, 256, 2048  # few tiles, deep K: slices of K into the stream's workspace, then their sum
+    a4, b4, d4 = ko.DeviceBuffer(m4 * k4 * 4), ko.DeviceBuffer(k4 * n4 * 4), ko.DeviceBuffer(m4 * n4 * 4)
+    ko.fill_uniform_f32(a4, m4 * k4, 511)
+    ko.fill_uniform_f32(b4, k4 * n4, 512)
     ko.fill_uniform_16(a3, m3 * k3, 509)
     ko.fill_uniform_16(b3, n3 * k3, 510)
     ko.fill_uniform_16(a2, m2 * k2, 507)
@@ -66,21 +70,22 @@ def test_operators_replay_from_a_hip_graph(ko):
         ko.sgemm(m, n, k, a32, b32, d32, stream=stream)
         ko.gemm16(m2, n2, k2, a2, b2, d2, stream=stream)
         ko.gemm16(m3, n3, k3, a3, b3, d3, stream=stream)
+        ko.sgemm(m4, n4, k4, a4, b4, d4, stream=stream)
 
     def outputs():
         return (dl.download(np.uint32, (rows, cols)), dmean.download(np.uint32, (rows,)),
                 d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)),
-                d3.download(np.uint16, (m3, n3)))
+                d3.download(np.uint16, (m3, n3)), d4.download(np.uint32, (m4, n4)))
 
     def clear():
         for buf, nbytes in ((ds, rows * cols * 4), (dl, rows * cols * 4), (dmean, rows * 4), (d16, m * n * 2), (d32, m * n * 4),
-                            (d2, m2 * n2 * 2), (d3, m3 * n3 * 2)):
+                            (d2, m2 * n2 * 2), (d3, m3 * n3 * 2), (d4, m4 * n4 * 4)):
             buf.upload(np.zeros(nbytes, np.uint8))
 
     chain()
     stream.synchronize()
     want = outputs()
-    assert want[0].any() and want[2].any() and want[3].any()
+    assert want[0].any() and want[2].any() and want[3].any() and want[6].any()
 
     graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
     assert hip.hipStreamBeginCapture(stream.handle, 0) == 0  # hipStreamCaptureModeGlobal
@@ -109,6 +114,47 @@ def test_operators_replay_from_a_hip_graph(ko):
         hip.hipGraphDestroy(graph)
 
 
+def test_sgemm_whose_first_sliced_call_is_captured_allocates_nothing(ko):
+    """The workspace of the K-sliced SGEMM belongs to a stream and is allocated by the first sliced call on it.
+    Inside a capture nothing may be allocated: a stream that has no workspace yet takes the unsliced kernels
+    there.  Small integers make both paths exact, so the replayed result is checked against the exact product."""
+    ko.lib()
+    hip = _hip_runtime()
+    stream = ko.Stream()
+    m, n, k = 128, 192, 3072
+    rng = np.random.default_rng(77)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    dA, dB, dD = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B), ko.DeviceBuffer(m * n * 4)
+    ko.set_tuning("sgemm.k_slices", 1)  # one-time set-up of the unsliced kernel in front of the capture, no workspace yet
+    try:
+        ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
+    finally:
+        ko.set_tuning("sgemm.k_slices", 0)
+    stream.synchronize()
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 0) == 0
+    try:
+        ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
+    finally:
+        rc = hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
+    try:
+        for replay in range(2):
+            dD.upload(np.zeros(m * n * 4, np.uint8))
+            assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+            stream.synchronize()
+            np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+    # the same call outside a capture gets the stream its workspace and slices K
+    ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
+    stream.synchronize()
+    np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))
+
+
 def test_operators_from_two_threads_on_two_streams(ko):
     """Thread-compatible entry points: two host threads, each with its own stream and buffers, run the row
     operators and the GEMMs at the same time; every result equals the single-threaded one bit for bit."""
@@ -122,6 +168,10 @@ def test_operators_from_two_threads_on_two_streams(ko):
         dx, dy, dl = ko.DeviceBuffer.from_numpy(x), ko.DeviceBuffer(rows * cols * 4), ko.DeviceBuffer(rows * cols * 4)
         a, b, d = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
         a16, b16, d16 = ko.DeviceBuffer(m * k * 2), ko.DeviceBuffer(n * k * 2), ko.DeviceBuffer(m * n * 2)
+        ms, ns, ks = 128, 128, 2048  # K-sliced: each stream sums its partial products in a workspace of its own
+        a_s, b_s, d_s = ko.DeviceBuffer(ms * ks * 4), ko.DeviceBuffer(ks * ns * 4), ko.DeviceBuffer(ms * ns * 4)
+        ko.fill_uniform_f32(a_s, ms * ks, seed + 5, stream=stream)
+        ko.fill_uniform_f32(b_s, ks * ns, seed + 6, stream=stream)
         ko.fill_uniform_f32(a, m * k, seed + 1, stream=stream)
         ko.fill_uniform_f32(b, k * n, seed + 2, stream=stream)
         ko.fill_uniform_16(a16, m * k, seed + 3, stream=stream)
@@ -131,12 +181,13 @@ def test_operators_from_two_threads_on_two_streams(ko):
             ko.layernorm(dy, dl, rows, cols, stream=stream)
             ko.sgemm(m, n, k, a, b, d, stream=stream)
             ko.gemm16(m, n, k, a16, b16, d16, stream=stream)
+            ko.sgemm(ms, ns, ks, a_s, b_s, d_s, stream=stream)
         if stream is not None:
             stream.synchronize()
         else:
             ko.synchronize()
         out[seed] = (dy.download(np.uint32, (rows, cols)), dl.download(np.uint32, (rows, cols)),
-                     d.download(np.uint32, (m, n)), d16.download(np.uint16, (m, n)))
+                     d.download(np.uint32, (m, n)), d16.download(np.uint16, (m, n)), d_s.download(np.uint32, (ms, ns)))
 
     want = {}
     for seed in (610, 620):
