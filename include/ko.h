@@ -166,6 +166,21 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
 int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
                  float beta, const float *C, float *D, ko_stream_t stream);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
+ * same kernels and the same bits as ko_sgemm_f32, but the partial products of a K-sliced problem go to an
+ * 8 MiB array that is part of the library's device code (one copy per GPU, held until the process ends)
+ * instead of a workspace allocated for the stream: the call makes no hipMalloc or hipFree, also not the
+ * first one on a stream.  A slice plan whose partial products exceed the array is refused with
+ * KO_ERR_UNSUPPORTED_SHAPE (plans chosen by shape need at most 64 x 64 floats per compute unit, 4 MiB on 256
+ * of them, and always fit; only a slice count forced through ko_set_tuning("sgemm.k_slices") can exceed it).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams, different
+ * threads) race on it and must be serialised by the caller.  Nothing in it has to start at zero: every
+ * element the summing kernel reads was written by the same call.  The first call on a device looks up the
+ * array's address (no stream work; make it outside a capture). */
+int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
+                                float beta, const float *C, float *D, ko_stream_t stream);
+
 /* ---- tensor-core-path GEMM: replaces
  *      gemm<GemmKernelTensorCore<half, half, half, ...>><<<...>>>(problem_size, A, B, C, D)
  *      (nn_operators/gemm/tensor_core_gemm.h:341-399; its launch is commented out at gemm/main.cu:344).

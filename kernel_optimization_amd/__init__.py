@@ -69,6 +69,7 @@ SIGNATURES = {
     "ko_softmax_16": (_int, [_vp, _vp, _i64, _i64, _vp, _i64, _int, _int, _vp]),
     "ko_layernorm_16": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _int, _int, _vp]),
     "ko_sgemm_f32": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _f, _vp, _vp, _vp]),
+    "ko_sgemm_f32_static_scratch": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _f, _vp, _vp, _vp]),
     "ko_gemm_f16f32acc": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp]),
     "ko_gemm_f16f32acc_bias_act": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp, _int, _vp]),
     "ko_fill_normal_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
@@ -275,6 +276,11 @@ def layernorm16(inp, out, rows, cols, mean=None, rstd=None, gamma=None, beta=Non
 
 def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
     check(lib().ko_sgemm_f32(m, n, k, alpha, _p(A), _p(B), beta, _p(C), _p(D), _h(stream)))
+
+
+def sgemm_static_scratch(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
+    """ko_sgemm_f32 for callers that cannot allocate: partial products in the library's static device array."""
+    check(lib().ko_sgemm_f32_static_scratch(m, n, k, alpha, _p(A), _p(B), beta, _p(C), _p(D), _h(stream)))
 
 
 def gemm16(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, b_layout=COL_MAJOR, dtype=F16,

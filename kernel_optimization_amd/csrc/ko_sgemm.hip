@@ -31,6 +31,12 @@
 #include <type_traits>
 #include <utility>
 
+// Partial products of the entry point that allocates nothing (ko_sgemm_f32_static_scratch): as large as the
+// workspace the allocating entry point gives a stream.  Every device the library runs on holds its own copy
+// until the process ends.  In host code the name is a stand-in, not a device address: host code uses the
+// address that ko::static_scratch() asks the runtime for, once per device.
+static __device__ __align__(256) unsigned char scratch[ko::kStreamWorkspaceBytes];
+
 namespace ko {
 namespace {
 
@@ -773,11 +779,13 @@ int run(Params p, hipStream_t s, int variant) {
 // K slices for problems that are deep and have few output tiles (256 x 256 x 2048: 32 tiles of 32 x 64 on 256
 // compute units).  The slices are workgroups of one launch (blockIdx.y); their partial products go to
 // `workspace_bytes` of device memory and a second kernel sums them in slice order, so the result does not
-// depend on which slice finished first.  Returns the slice count (1: do not slice) and the slice depth.
+// depend on which slice finished first.  Returns the slice count (1: do not slice) and the slice depth; the
+// caller checks that slices x M x N floats fit its workspace (chosen by shape they are at most 64 x 64 floats
+// per compute unit).
 //   - operands as the direct-to-LDS kernels want them (rows on 16-byte boundaries);
 //   - tiles for at most half of the compute units, and as many slices as bring the launch up to one
 //     workgroup per compute unit, each at least 256 deep and a multiple of 128 (whole pairs of K tiles).
-int plan_k_slices(const Params &p, size_t workspace_bytes, int *k_slice) {
+int plan_k_slices(const Params &p, int *k_slice) {
     *k_slice = 0;
     const int forced = tuning(knob_sgemm_k_slices);
     if (forced == 1) return 1;
@@ -796,7 +804,6 @@ int plan_k_slices(const Params &p, size_t workspace_bytes, int *k_slice) {
     const int64_t depth = ((p.K + slices - 1) / slices + 127) / 128 * 128;
     slices = (p.K + depth - 1) / depth;
     if (slices < 2 || slices > 65535) return 1;
-    if (static_cast<uint64_t>(slices) * p.M * p.N * sizeof(float) > workspace_bytes) return 1;
     *k_slice = static_cast<int>(depth);
     return static_cast<int>(slices);
 }
@@ -813,13 +820,30 @@ int run_sliced(const Params &p, int slices, int k_slice, float *workspace, hipSt
     return sum_slices(workspace, slices, p, s);
 }
 
-}  // namespace
-}  // namespace ko
+// The address of `scratch` on the current device (looked up once per device).
+int static_scratch(void **address) {
+    constexpr int kCached = 64;
+    static std::atomic<void *> known[kCached];  // zero-initialised
+    int dev = 0;
+    KO_HIP(hipGetDevice(&dev));
+    if (dev >= 0 && dev < kCached) {
+        if (void *a = known[dev].load(std::memory_order_acquire)) {
+            *address = a;
+            return KO_OK;
+        }
+    }
+    void *a = nullptr;
+    KO_HIP(hipGetSymbolAddress(&a, HIP_SYMBOL(scratch)));
+    if (a == nullptr) return fail(KO_ERR_RUNTIME, "sgemm: the static scratch array has no address on device %d", dev);
+    if (dev >= 0 && dev < kCached) known[dev].store(a, std::memory_order_release);
+    *address = a;
+    return KO_OK;
+}
 
-KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A,
-                           const float *B, float beta, const float *C, float *D,
-                           ko_stream_t stream) {
-    using namespace ko;
+// Both SGEMM entry points.  `own_scratch`: partial products of a K-sliced problem go to the static array of the
+// device instead of the stream's allocated workspace, and a slice plan that does not fit is an error.
+int sgemm(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B, float beta, const float *C,
+          float *D, ko_stream_t stream, bool own_scratch) {
     if (m < 0 || n < 0 || k < 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
     if (m == 0 || n == 0) return KO_OK;
@@ -831,9 +855,18 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
     const int variant = tuning(knob_sgemm_variant);
     if (variant <= 0) {
         int k_slice = 0;
-        if (const int slices = plan_k_slices(p, kStreamWorkspaceBytes, &k_slice); slices > 1) {
+        if (const int slices = plan_k_slices(p, &k_slice); slices > 1) {
+            const uint64_t need = static_cast<uint64_t>(slices) * m * n * sizeof(float);
             void *workspace = nullptr;
-            if (const int st = stream_workspace(s, &workspace); st != KO_OK) return st;
+            if (own_scratch) {
+                if (need > sizeof(scratch))
+                    return fail(KO_ERR_UNSUPPORTED_SHAPE,
+                                "sgemm: the partial products of %d slices of K (%llu bytes) do not fit the static scratch array (%zu bytes)",
+                                slices, (unsigned long long)need, sizeof(scratch));
+                if (const int st = static_scratch(&workspace); st != KO_OK) return st;
+            } else if (need <= kStreamWorkspaceBytes) {
+                if (const int st = stream_workspace(s, &workspace); st != KO_OK) return st;
+            }
             if (workspace != nullptr) return run_sliced(p, slices, k_slice, static_cast<float *>(workspace), s);
         }
     }
@@ -860,4 +893,17 @@ KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const f
         }
     }
     return run(p, s, variant);
+}
+
+}  // namespace
+}  // namespace ko
+
+KO_EXPORT int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B, float beta,
+                           const float *C, float *D, ko_stream_t stream) {
+    return ko::sgemm(m, n, k, alpha, A, B, beta, C, D, stream, false);
+}
+
+KO_EXPORT int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
+                                          float beta, const float *C, float *D, ko_stream_t stream) {
+    return ko::sgemm(m, n, k, alpha, A, B, beta, C, D, stream, true);
 }
