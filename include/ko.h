@@ -154,7 +154,9 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * D[m,n] = alpha * A[m,k] * B[k,n] + beta * C[m,n], all row-major fp32.
  * C may be NULL (then beta is ignored); the reference's epilogue is alpha = beta = 1
  * with C given, or D = A*B with C null (simt_gemm.h:325-373).
- * m, n multiples of 4 are not required; any positive sizes are accepted.  m == 0 or n == 0 is a no-op;
+ * m, n, k multiples of 4 and 16-byte aligned pointers are not required (operand rows that do not start on
+ * 16-byte boundaries are loaded four bytes at a time: about 0.7 of the aligned rate); any positive sizes are
+ * accepted.  m == 0 or n == 0 is a no-op;
  * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries.
  * Workspace: a problem with few output tiles and a deep K (tiles for at most half of the compute units,
  * k >= 768, operand rows on 16-byte boundaries) is cut into slices of K that run side by side; their partial

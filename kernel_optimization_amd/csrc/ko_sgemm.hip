@@ -416,6 +416,15 @@ __device__ __forceinline__ void static_for(F &&f) {
 // What lanes fetch in place of operand elements past the end of K.
 __device__ __attribute__((aligned(16))) const float zero_chunk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 
+// One direct-to-LDS load: LB (16 or 4) bytes per lane from `from` (per lane) to `to` + LB * lane (`to` wave-uniform).
+template <int LB>
+__device__ __forceinline__ void load_to_lds(const char *from, char *to) {
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    if constexpr (LB == 16) __builtin_amdgcn_global_load_lds((gptr_t)from, (lptr_t)to, 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)from, (lptr_t)to, 4, 0, 0);
+}
+
 // Direct-to-LDS kernel (EDGE false: full tiles and an even number of K tiles): the same tiles, LDS layout, fragment
 // order and epilogue as the PIPE form of sgemm_kernel, but global_load_lds_dwordx4 moves 16 bytes per
 // lane from global memory straight into LDS (lane l of a wave-level load fills the l-th 16-byte slot
@@ -429,7 +438,12 @@ __device__ __attribute__((aligned(16))) const float zero_chunk[4] = {0.0f, 0.0f,
 // for all of them (vmcnt(0)) before every fragment read it knows of; so the fragment reads and their
 // waits are inline assembly.  Registers filled by such a read pass through an empty assembly statement
 // behind the wait before the MFMAs use them, which keeps every use (and every copy) behind the wait.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, bool EDGE>
+//
+// LB = 4 (with EDGE): operand rows that do not start on 16-byte boundaries (N, K or the row stride of A not a
+// multiple of 4, or unaligned base pointers).  The same LDS layout is filled four bytes per lane instead of
+// sixteen (global_load_lds_dword: lane l fills the l-th dword behind the wave-uniform base), four times as
+// many loads; each lane fetches the element that belongs in its dword, a zero where k is past the end.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int KSPLIT, int NSTAGE, bool EDGE, int LB = 16>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_kernel(const Params whole) {
     const Params p = slice_of(whole);
     constexpr int THREADS = 64 * WAVES_M * WAVES_N * KSPLIT;
@@ -440,11 +454,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
     constexpr int B_CHUNKS = BK * BN / 4;
     constexpr int BNC = BN / 4;
     constexpr int CHUNKS = A_CHUNKS + B_CHUNKS;
-    constexpr int LOADS = CHUNKS / THREADS;      // wave-level loads per wave and K tile
-    constexpr int A_LOADS = A_CHUNKS / THREADS;  // the first A_LOADS of them fetch A
+    constexpr int PER_CHUNK = 16 / LB;                       // loads that fill one 16-byte chunk
+    constexpr int LOADS = CHUNKS * PER_CHUNK / THREADS;      // wave-level loads per wave and K tile
+    constexpr int A_LOADS = A_CHUNKS * PER_CHUNK / THREADS;  // the first A_LOADS of them fetch A
     constexpr int KGROUPS = BK / 8;
     constexpr int GROUPS = KGROUPS / KSPLIT;
     constexpr int STAGE_BYTES = CHUNKS * 16;
+    static_assert(LB == 16 || (LB == 4 && EDGE), "the dword form is an edge form");
     static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "a wave-level load stays inside A or B");
     static_assert(KGROUPS % KSPLIT == 0 && (BK == 32 || BK == 64 || BK == 128) && BN % 64 == 0 && NSTAGE >= 2, "");
     static_assert((NSTAGE - 1) * LOADS < 64 && BK * BN * 4 < 65536 && TM * 32 * A_ROW_CHUNKS * 16 < 65536, "");
@@ -463,7 +479,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
     const int N = p.N, K = p.K;
-    // EDGE: K (a multiple of 4) is padded with zeros up to the next pair of K tiles.
+    // EDGE: K (a multiple of 4 unless LB = 4) is padded with zeros up to the next pair of K tiles.
     const int KT = EDGE ? 2 * ((K + 2 * BK - 1) / (2 * BK)) : K / BK;
 
     // A rows of 256 bytes or more fill lines of the 64 banks; of 128 bytes two rows share one, and the
@@ -471,24 +487,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
     auto swz_a = [](int row) { return BK == 32 ? (row >> 1) & 7 : row & 15; };
     auto swz_b = [](int k) { return ((k >> 2) & 1) << 3; };
 
-    // What this thread fetches with each of its loads: LDS slot tid + i * THREADS of the stage, K tile 0.
+    // What this thread fetches with each of its loads: LDS slot (of LB bytes) tid + i * THREADS of the stage, K tile 0.
     const char *src[LOADS];
-    int koff[EDGE ? LOADS : 1];  // EDGE: the k, within a K tile, of the chunk (A) or row (B) this lane fetches
+    int koff[EDGE ? LOADS : 1];  // EDGE: the k, within a K tile, of the chunk or element (A) or row (B) this lane fetches
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-        const int idx = tid + i * THREADS;
+        const int slot = tid + i * THREADS;
+        const int idx = slot / PER_CHUNK, d = slot % PER_CHUNK;  // 16-byte chunk of the stage, element within it (LB = 4)
         if (i < A_LOADS) {
             const int row = idx / A_ROW_CHUNKS, c = idx % A_ROW_CHUNKS;
-            if constexpr (EDGE) koff[i] = 4 * (c ^ swz_a(row));
+            const int k = 4 * (c ^ swz_a(row)) + d;
+            if constexpr (EDGE) koff[i] = k;
             int gr = m0 + row;
             if constexpr (EDGE) gr = gr < p.M ? gr : p.M - 1;  // rows past M fetch the last row again; never stored
-            src[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(gr) * p.lda + 4 * (c ^ swz_a(row)));
+            src[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(gr) * p.lda + k);
         } else {
             const int b = idx - A_CHUNKS;
             const int kr = b / BNC, c = b % BNC;
             if constexpr (EDGE) koff[i] = kr;
-            int gn = n0 + 4 * (c ^ swz_b(kr));
-            if constexpr (EDGE) gn = gn < N ? gn : N - 4;  // columns past N (a multiple of 4) fetch the last chunk again
+            int gn = n0 + 4 * (c ^ swz_b(kr)) + d;
+            // columns past N fetch the last chunk (N a multiple of 4) or element again: they only feed columns never stored
+            if constexpr (EDGE) gn = gn < N ? gn : N - (LB == 16 ? 4 : 1);
             src[i] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(kr) * N + gn);
         }
     }
@@ -511,10 +530,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
         if constexpr (EDGE) k_left = K - ld_kt * BK;
     };
     auto issue = [&](int stage) {
-        char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * 1024;
+        char *dst = reinterpret_cast<char *>(lds) + stage * STAGE_BYTES + wave * (64 * LB);
 #pragma unroll
         for (int i = 0; i < LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)source(i), (lptr_t)(dst + i * THREADS * 16), 16, 0, 0);
+            load_to_lds<LB>(source(i), dst + i * THREADS * LB);
         advance();
     };
 
@@ -601,7 +620,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
         constexpr int A_READS = GROUPS * TM, B_READS = TN * GROUPS * 4;
         constexpr int PIECES = LOADS + A_READS + B_READS;
         constexpr int PER = (PIECES + NMFMA - 1) / NMFMA;
-        char *dst = reinterpret_cast<char *>(lds) + wr * STAGE_BYTES + wave * 1024;
+        char *dst = reinterpret_cast<char *>(lds) + wr * STAGE_BYTES + wave * (64 * LB);
         const uint32_t off = static_cast<uint32_t>(rd) * STAGE_BYTES;
         static_for<NMFMA>([&](auto q_c) {
             constexpr int q = decltype(q_c)::value;
@@ -610,7 +629,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void sgemm_direct_
             static_for<PER>([&](auto r_c) {
                 constexpr int pc = q * PER + decltype(r_c)::value;
                 if constexpr (pc < LOADS) {
-                    __builtin_amdgcn_global_load_lds((gptr_t)source(pc), (lptr_t)(dst + pc * THREADS * 16), 16, 0, 0);
+                    load_to_lds<LB>(source(pc), dst + pc * THREADS * LB);
                     if constexpr (pc == LOADS - 1) advance();
                 } else if constexpr (pc < LOADS + A_READS) {
                     constexpr int u = pc - LOADS, g2 = u / TM, i2 = u % TM;
@@ -673,7 +692,7 @@ int launch_direct(Params p, hipStream_t stream) {
     const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                          p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
     if (!aligned && p.k_slice > 0) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: K slices need 16-byte aligned operand rows");
-    if (!aligned) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
+    if (!aligned && tuning(knob_sgemm_unaligned) == 1) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
     // K-sliced launches: every slice but the last is k_slice deep (a multiple of 4), the last takes the rest.
     const int slices = p.k_slice > 0 ? (p.K + p.k_slice - 1) / p.k_slice : 1;
     const int k_last = p.K - (slices - 1) * (p.k_slice > 0 ? p.k_slice : 0);
@@ -685,10 +704,12 @@ int launch_direct(Params p, hipStream_t stream) {
     if (nblocks > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: too many tiles");
     p.blocked = tuning(knob_sgemm_mapping) != 1 && tiles_m % 4 == 0 && p.tiles_n % 8 == 0 &&
                 ((tiles_m / 4) * (p.tiles_n / 8)) % 8 == 0;
-    auto kernel = edge ? sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, true>
-                       : sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, false>;
-    static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
-    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge]); st != KO_OK)
+    // Operand rows off 16-byte boundaries: the edge form that fills LDS four bytes per lane.
+    auto kernel = !aligned ? sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, true, 4>
+                  : edge   ? sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, true>
+                           : sgemm_direct_kernel<BM, BN, BK, WAVES_M, WAVES_N, KSPLIT, NSTAGE, false>;
+    static std::atomic<uint64_t> configured[3] = {{0}, {0}, {0}};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[!aligned ? 2 : edge]); st != KO_OK)
         return st;
     kernel<<<dim3(static_cast<unsigned>(nblocks), static_cast<unsigned>(slices)), dim3(THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
@@ -761,6 +782,11 @@ int run(Params p, hipStream_t s, int variant) {
         const bool big = t128 >= cu && 97 * ((t128 + cu - 1) / cu) <= 31 * ((t64 + cu - 1) / cu);
         variant = big ? (k >= 2048 ? 40 : 36)
                       : (2 * t64 <= cu ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
+        // Operand rows off 16-byte boundaries are loaded four bytes per lane, four times as many loads with an
+        // address each: the 128 x 128 x 64 form would spill registers there.
+        const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
+                             p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
+        if (!aligned && variant == 40) variant = 36;
     }
     switch (variant) {
         case 13: return launch<64, 64, 64, 2, 2, 4, true>(p, s);

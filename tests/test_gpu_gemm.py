@@ -511,6 +511,49 @@ def test_sgemm_ragged_shapes_are_exact_on_small_integers(ko):
         np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=str((m, n, k)))
 
 
+def test_sgemm_rows_off_16_byte_boundaries_are_exact_on_small_integers(ko):
+    """N, K or a base pointer that is not a multiple of four floats: operand rows do not start on 16-byte
+    boundaries and the direct-to-LDS kernels fill their stages four bytes per lane.  Every lane then fetches one
+    element of its own (clamped at M and N, a zero past K), so a wrong element, a missing zero or a swizzle
+    applied at the wrong granularity shows as a wrong integer.  The register pipeline (knob sgemm.unaligned = 1)
+    must give the same matrix."""
+    rng = np.random.default_rng(11)
+    shapes = [(int(rng.integers(1, 1500)), int(rng.integers(1, 1500)), int(rng.integers(1, 1500))) for _ in range(10)]
+    shapes += [(1023, 1025, 1027), (129, 2, 1), (64, 64, 65), (2500, 2302, 130), (3, 1001, 2050), (2049, 2047, 3000)]
+    try:
+        for m, n, k in shapes:
+            A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+            B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+            C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+            ref = A.astype(np.float64) @ B.astype(np.float64)
+            for knob in (0, 1):
+                ko.set_tuning("sgemm.unaligned", knob)
+                np.testing.assert_array_equal(ko.sgemm_host(A, B), ref, err_msg=str((m, n, k, knob)))
+                np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=str((m, n, k, knob)))
+    finally:
+        ko.set_tuning("sgemm.unaligned", 0)
+    # aligned sizes behind base pointers that are one float off a 16-byte boundary
+    m, n, k = 200, 136, 264
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    dA, dB, dD = ko.DeviceBuffer(m * k * 4 + 16), ko.DeviceBuffer(k * n * 4 + 16), ko.DeviceBuffer(m * n * 4)
+    for offset_a, offset_b in ((4, 0), (0, 4), (12, 8)):
+        dA.upload(np.concatenate([np.zeros(offset_a // 4, np.float32), A.ravel(), np.zeros(4 - offset_a // 4, np.float32)]))
+        dB.upload(np.concatenate([np.zeros(offset_b // 4, np.float32), B.ravel(), np.zeros(4 - offset_b // 4, np.float32)]))
+        ko.sgemm(m, n, k, dA.ptr + offset_a, dB.ptr + offset_b, dD)
+        ko.synchronize()
+        np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))
+
+
+@pytest.mark.parametrize("sgemm_variant", [33, 35, 36, 37, 41], indirect=True)
+def test_sgemm_unaligned_rows_against_oracle(ko, sgemm_variant):
+    """Uniform inputs through the four-byte form of every direct-to-LDS tiling, within the fp32 summation bound."""
+    m, n, k = 261, 203, 777
+    A, B = inputs.uniform_f32((m, k), 31), inputs.uniform_f32((k, n), 32)
+    ref, ap = oracle.sgemm(A, B, want_absprod=True)
+    assert_sgemm_close(ko.sgemm_host(A, B), ref, ap, k)
+
+
 @pytest.mark.parametrize("m,n,k", [(4136, 2048, 256), (8000, 2304, 768), (4353, 4096, 128)])
 def test_gemm16_ragged_row_counts_whole_output(ko, m, n, k):
     """Row counts that do not fill the last row of 256 x 256 tiles: the full tile rows run on the pinned kernel,
