@@ -667,6 +667,10 @@ def main():
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16000, 3072, 768))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
+        # K off the K tile: padded with zeros inside the pinned kernel
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16384, 3072, 760))
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)

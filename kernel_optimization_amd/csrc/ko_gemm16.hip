@@ -767,7 +767,12 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
     else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
-template <class T, bool BF16, bool B_ROW>
+__device__ __attribute__((aligned(16))) const uint32_t zero_chunk16[4] = {0u, 0u, 0u, 0u};
+
+// EDGE_K: K is any multiple of 8 and is padded with zeros up to the next multiple of 128 - a lane whose
+// 16-byte chunk (or, for a row-major B, whose row) lies at or past K fetches 16 zero bytes instead, chosen per
+// load with a compare and two selects, so nothing is read past the end of a row or of the matrix.
+template <class T, bool BF16, bool B_ROW, bool EDGE_K = false>
 __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -791,15 +796,16 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets address math run on the scalar unit
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int K = p.K;
-    const int KT = K / kBK;
+    const int KT = EDGE_K ? 2 * ((K + 2 * kBK - 1) / (2 * kBK)) : K / kBK;
     const int grid = gridDim.x;
     const int my_tiles = (p.nblocks - static_cast<int>(blockIdx.x) + grid - 1) / grid;
     const int total = my_tiles * KT;
     if (total == 0) return;
 
     const int row_in = lane >> 3;
-    const uint32_t lane_off =
-        static_cast<uint32_t>(row_in * K + (((lane & 7) ^ swz<1>(8 * wave + row_in)) << 3)) * 2u;
+    const int lane_k = ((lane & 7) ^ swz<1>(8 * wave + row_in)) << 3;  // first k, within a K tile, of this lane's chunk
+    const uint32_t lane_off = static_cast<uint32_t>(row_in * K + lane_k) * 2u;
+    const char *const zeros = reinterpret_cast<const char *>(&zero_chunk16);
 
     // Row-major B ([K][N]): the K tile of B is 64 rows of BN values and stays row-major in LDS.  A load
     // instruction of a wave covers two rows (k = 2 * (wave + WAVES * J) + r, r = lane / 32); the 16-byte chunk a
@@ -851,15 +857,30 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         }
     };
     // load number I of the cursor's K tile (the A loads first, then the B loads); the last one moves the cursor
+    // EDGE_K: where load I of the cursor's K tile reads from - its place in A or B, or the zero chunk when the
+    // lane's k lies at or past K (for a row-major B the k is the row the load fetches)
+    auto source_a = [&](int i) {
+        const char *at = cur_a + i * group_stride + lane_off;
+        if constexpr (EDGE_K) at = ld_kt * kBK + lane_k < K ? at : zeros;
+        return at;
+    };
+    auto source_b = [&](int j) {
+        const char *at = cur_b + j * group_stride_b + lane_off_b;
+        if constexpr (EDGE_K) {
+            const int k = B_ROW ? 2 * (wave + WAVES * j) + (lane >> 5) : lane_k;
+            at = ld_kt * kBK + k < K ? at : zeros;
+        }
+        return at;
+    };
     auto issue_one = [&](int stage, auto i_c) {
         constexpr int I = decltype(i_c)::value;
         if constexpr (I < A_LOADS) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(cur_a + I * group_stride + lane_off),
+            __builtin_amdgcn_global_load_lds((gptr_t)source_a(I),
                                              (lptr_t)(lds_bytes + stage * A_BYTES + 1024 * (wave + WAVES * I)), 16, 0, 0);
         } else {
             constexpr int J = I - A_LOADS;
             __builtin_amdgcn_global_load_lds(
-                (gptr_t)(cur_b + J * group_stride_b + lane_off_b),
+                (gptr_t)source_b(J),
                 (lptr_t)(lds_bytes + 2 * A_BYTES + stage * B_BYTES + 1024 * (wave + WAVES * J)), 16, 0, 0);
             if constexpr (J == B_LOADS - 1) advance_cursor();
         }
@@ -869,12 +890,10 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         char *dst_b = lds_bytes + 2 * A_BYTES + stage * B_BYTES;
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(cur_a + i * group_stride + lane_off),
-                                             (lptr_t)(dst_a + 1024 * (wave + WAVES * i)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)source_a(i), (lptr_t)(dst_a + 1024 * (wave + WAVES * i)), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(cur_b + i * group_stride_b + lane_off_b),
-                                             (lptr_t)(dst_b + 1024 * (wave + WAVES * i)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)source_b(i), (lptr_t)(dst_b + 1024 * (wave + WAVES * i)), 16, 0, 0);
         if (ld_kt + 1 < KT) {
             ++ld_kt;
             cur_a += kBK * 2;
@@ -1084,11 +1103,12 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
 template <class T, bool BF16, bool B_ROW = false>
 int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
-    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % (2 * kBK)) != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 128 == 0");
-    auto kernel = gemm16_pinned_kernel<T, BF16, B_ROW>;
-    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
-    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
+    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % 8) != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 8 == 0");
+    const bool edge_k = p.K % (2 * kBK) != 0;  // padded with zeros up to a pair of K tiles inside the kernel
+    auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true> : gemm16_pinned_kernel<T, BF16, B_ROW, false>;
+    static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge_k]); st != KO_OK)
         return st;
     p.tiles_n = p.N / T::BN;
     const int tiles_m = p.M / T::BM;
@@ -1186,8 +1206,8 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
     }
     if (variant <= 0) {
         // Enough 256x256 tiles to fill the chip: the big tiling - as a persistent direct-to-LDS kernel
-        // when the tiles are full and both operands are K-contiguous (the pinned one when K is a
-        // multiple of 128), else as the register pipeline.
+        // when the tiles are full (the pinned one from K = 128 on; a K that is not a multiple of 128 is padded
+        // with zeros inside the kernel), else as the register pipeline.
         // Fewer: smaller tiles so that the grid still covers the compute units.
         const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
         // Two reasons to send the last rows out as a launch of their own, with the tiling their size asks for:
@@ -1201,7 +1221,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // to the pinned kernel when the rest of the shape allows - and the remaining columns (fewer than 256)
         // as a launch of their own; C, D and a row-major B keep their row strides.
         if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.ldb % 8 == 0 &&
-            p.K % (2 * kBK) == 0 && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
+            p.K >= 2 * kBK && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
             const int n1 = p.N - p.N % 256;
             Params left = p, right = p;
             left.N = n1;
@@ -1217,7 +1237,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         if (row_cuts > 0 && split_knob != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
             const int64_t tn = (p.N + 255) / 256;
-            const bool pinned_ok = p.N % 256 == 0 && p.K % (2 * kBK) == 0;
+            const bool pinned_ok = p.N % 256 == 0 && p.K >= 2 * kBK;
             int64_t rows_top = p.M % 256 != 0 && pinned_ok ? p.M / 256 : (p.M + 255) / 256;  // in tile rows
             const int64_t tiles = rows_top * tn, rounds = tiles / cu;
             if (rounds >= 1 && tiles % cu != 0) {
@@ -1241,7 +1261,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // The pinned kernel is so much faster per tile that it wins from half a chip's worth of full tiles on
         // (192 tiles on 256 CUs: 16384 x 768 x 3072 takes 69 us against 103 us with 128 x 128 tiles; at 96 tiles
         // the two are level).
-        if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K % (2 * kBK) == 0)
+        if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K >= 2 * kBK)
             return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
         if (big_tiles < compute_units()) {
             // Fewer big tiles than that: the largest of the small tilings that still gives every compute unit one

@@ -249,6 +249,31 @@ def test_gemm16_variants_agree_bitwise(ko, m, n, k):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k", [(4096, 2048, 760), (2048, 4096, 200), (4352, 2304, 136), (2048, 4096, 1032)])
+def test_gemm16_k_off_the_k_tile_is_padded_with_zeros(ko, m, n, k, b_col_major, bf16):
+    """K a multiple of 8 but not of 128 on shapes of full 256 x 256 tiles: the pinned kernel pads K with zeros
+    up to the next pair of K tiles (lanes whose chunk or row lies past K fetch a zero chunk).  A zero that is
+    missing, a chunk fetched from the next row instead, or padding applied to the wrong K tile changes the
+    sums: the whole output must equal the register pipeline's (variant 9, which bounds-checks K) bit for bit,
+    and sampled rows must agree with the oracle."""
+    A = _bits16((m, k), 61, bf16)
+    B = _bits16((n, k), 62, bf16)
+    Bdev = B if b_col_major else np.ascontiguousarray(B.T)
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
+    got = ko.gemm16_host(A, Bdev, m, n, k, **kw)
+    ko.set_tuning("gemm16.variant", 9)
+    try:
+        want = ko.gemm16_host(A, Bdev, m, n, k, **kw)
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+    np.testing.assert_array_equal(got, want)
+    idx = np.sort(np.random.default_rng(5).choice(m, 48, replace=False))
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, bf16=bf16)
+    assert_gemm16_close(_to_f64(got[idx], bf16), ref64, ap, k, bf16=bf16)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("k", [320, 384])
 def test_gemm16_default_path_big(ko, bf16, k):
     """Large enough for the default dispatch to take a persistent direct-to-LDS kernel (512 tiles of
