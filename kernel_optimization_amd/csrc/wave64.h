@@ -107,10 +107,12 @@ struct Welford {
 __device__ __forceinline__ Welford welford_merge(const Welford &a, const Welford &b) {
     Welford r;
     r.count = a.count + b.count;
-    const float n = r.count > 0.0f ? r.count : 1.0f;  // both sides empty: 0/1 keeps the triplet at zero
-    r.mean = (a.count * a.mean + b.count * b.mean) / n;
+    // 1/n from the hardware reciprocal (1 ulp; two correctly rounded divisions cost ten instructions each, and
+    // a workgroup-wide all-reduce makes ten merges per row).  Both sides empty: n = 1 keeps the triplet at zero.
+    const float inv_n = __builtin_amdgcn_rcpf(r.count > 0.0f ? r.count : 1.0f);
+    r.mean = (a.count * a.mean + b.count * b.mean) * inv_n;
     const float d = b.mean - a.mean;
-    r.m2 = (a.m2 + b.m2) + d * d * (a.count * b.count / n);
+    r.m2 = (a.m2 + b.m2) + d * d * (a.count * b.count * inv_n);
     return r;
 }
 
