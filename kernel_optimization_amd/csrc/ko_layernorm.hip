@@ -48,6 +48,11 @@ struct Reciprocals {
     }
 };
 
+// 1 / sqrt(x) from the hardware instruction (1 ulp; the gate on rstd is 1e-5 relative).  A correctly rounded
+// square root followed by a correctly rounded division is some 25 instructions that every lane of a row runs.
+// Special values as with the division: +inf -> 0, 0 -> +inf, NaN and negative -> NaN.
+__device__ __forceinline__ float rsqrt_1ulp(float x) { return __builtin_amdgcn_rsqf(x); }
+
 __device__ __forceinline__ void welford_update(wave::Welford &w, float x, float inv_count) {
     w.count += 1.0f;
     const float d = x - w.mean;
@@ -151,21 +156,56 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         const bool row_ok = row < rows;
         const float x0 = wave::broadcast_group_first<LPR>(v[0][0]);
         wave::Welford w{0.0f, 0.0f, 0.0f};
+        if constexpr (FULL) {
+            // Every lane holds VPL * E values in registers: its triplet (count, mean, M2) is formed in two passes
+            // over them - sums of independent pairs instead of VPL * E dependent Welford updates.
+            float s[E], q[E];
 #pragma unroll
-        for (int k = 0; k < VPL; ++k) {
-            const int j = l + k * LPR;
+            for (int e = 0; e < E; ++e) {
+                v[0][e] -= x0;
+                s[e] = v[0][e];
+            }
 #pragma unroll
-            for (int e = 0; e < E; ++e) v[k][e] -= x0;
-            if (FULL || j < nvec) {
+            for (int k = 1; k < VPL; ++k)
 #pragma unroll
-                for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
+                for (int e = 0; e < E; ++e) {
+                    v[k][e] -= x0;
+                    s[e] += v[k][e];
+                }
+            float sum = s[0];
+#pragma unroll
+            for (int e = 1; e < E; ++e) sum += s[e];
+            const float lane_mean = sum * (1.0f / (VPL * E));
+#pragma unroll
+            for (int e = 0; e < E; ++e) q[e] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < VPL; ++k)
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const float d = v[k][e] - lane_mean;
+                    q[e] = __builtin_fmaf(d, d, q[e]);
+                }
+            float m2 = q[0];
+#pragma unroll
+            for (int e = 1; e < E; ++e) m2 += q[e];
+            w = wave::Welford{static_cast<float>(VPL * E), lane_mean, m2};
+        } else {
+#pragma unroll
+            for (int k = 0; k < VPL; ++k) {
+                const int j = l + k * LPR;
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[k][e] -= x0;
+                if (FULL || j < nvec) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
+                }
             }
         }
         if constexpr (FULL) w = wave::welford_allreduce_equal<LPR>(w);
         else w = wave::welford_allreduce<LPR>(w);
 
         const float mean = w.mean;  // of the shifted row
-        const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
+        const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
 
         // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
         typename Io<IO>::elem *dst0 = out + (row - sub) * cols;
@@ -383,7 +423,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
         }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
-        const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
+        const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
         typename Io<IO>::elem *dst = out + row * cols;
         if constexpr (REST) {
             // the streamed part first and from the row's end backwards: what was read last is the likeliest to be
@@ -503,7 +543,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
         }
         w = block_welford_allreduce<THREADS>(w, lds);
         const float mean = w.mean;  // of the shifted row
-        const float rstd = 1.0f / sqrtf(w.m2 * inv_denominator + eps);
+        const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
         typename Io<IO>::elem *dst = out + row * cols;
         // Second pass from the row's end backwards (what the first pass read last is the likeliest to be in a
         // cache still), with nontemporal accesses: nothing is touched again.
