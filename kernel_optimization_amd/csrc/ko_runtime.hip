@@ -74,6 +74,8 @@ int stream_workspace(hipStream_t stream, void **workspace) {
     static int used = 0;
     static std::mutex lock;
     *workspace = nullptr;
+    // one handle value stands for a different stream in every host thread: no workspace can belong to it
+    if (stream == hipStreamPerThread) return KO_OK;
     int dev = 0;
     KO_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> guard(lock);
