@@ -158,24 +158,25 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * 16-byte boundaries are loaded four bytes at a time: about 0.7 of the aligned rate); any positive sizes are
  * accepted.  m == 0 or n == 0 is a no-op;
  * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries.
- * Workspace: a problem with few output tiles and a deep K (tiles for at most half of the compute units,
- * k >= 768, operand rows on 16-byte boundaries) is cut into slices of K that run side by side; their partial
- * products go through 8 MiB of device memory that the library allocates at the first such call on a
- * (device, stream) pair and keeps until the process ends.  Calls on different streams therefore never share
- * it.  A first such call made while the stream is being captured into a graph allocates nothing and takes
- * the unsliced kernels; so does every call once 64 pairs hold a workspace.  Results do not depend on the
- * timing of the slices (summed in slice order), but the sliced and the unsliced path round differently. */
+ * Workspace: a problem with a deep K whose output tiles do not fill the chip (tiles for at most half of the
+ * compute units and k >= 768, or rounds of tiles that leave many compute units idle and k >= 2048; operand
+ * rows on 16-byte boundaries) is cut into slices of K that run side by side; their partial products go
+ * through 32 MiB of device memory that the library allocates at the first such call on a (device, stream)
+ * pair and keeps until the process ends.  Calls on different streams therefore never share it.  A first
+ * such call made while the stream is being captured into a graph allocates nothing and takes the unsliced
+ * kernels; so does every call once 64 pairs hold a workspace.  Results do not depend on the timing of the
+ * slices (summed in slice order), but the sliced and the unsliced path round differently. */
 int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
                  float beta, const float *C, float *D, ko_stream_t stream);
 
 /* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
  * same kernels and the same bits as ko_sgemm_f32, but the partial products of a K-sliced problem go to an
- * 8 MiB array that is part of the library's device code (one copy per GPU, held until the process ends)
+ * 32 MiB array that is part of the library's device code (one copy per GPU, held until the process ends)
  * instead of a workspace allocated for the stream: the call makes no hipMalloc or hipFree, also not the
  * first one on a stream.  A slice plan whose partial products exceed the array is refused with
- * KO_ERR_UNSUPPORTED_SHAPE (plans chosen by shape need at most 64 x 64 floats per compute unit, 4 MiB on 256
- * of them, and always fit; only a slice count forced through ko_set_tuning("sgemm.k_slices") can exceed it).
+ * KO_ERR_UNSUPPORTED_SHAPE (plans chosen by shape are chosen to fit; only a slice count forced through
+ * ko_set_tuning("sgemm.k_slices") can exceed it).
  * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams, different
  * threads) race on it and must be serialised by the caller.  Nothing in it has to start at zero: every
  * element the summing kernel reads was written by the same call.  The first call on a device looks up the

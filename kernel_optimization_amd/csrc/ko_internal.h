@@ -30,7 +30,7 @@ int hip_fail(hipError_t err, const char *expr, const char *file, int line);
     X(layernorm_blocks_per_cu, "layernorm.blocks_per_cu") X(layernorm_block_threads, "layernorm.block_threads") \
     X(layernorm_wave_threads, "layernorm.wave_threads") X(softmax_wave_lds, "softmax.wave_lds") X(rows_block_grid, "rows.block_grid") X(layernorm_wave_lds, "layernorm.wave_lds")           \
     X(sgemm_variant, "sgemm.variant") X(sgemm_mapping, "sgemm.mapping") X(sgemm_split_rows, "sgemm.split_rows") \
-    X(sgemm_k_slices, "sgemm.k_slices") X(sgemm_unaligned, "sgemm.unaligned")                                                                     \
+    X(sgemm_k_slices, "sgemm.k_slices") X(sgemm_slice_variant, "sgemm.slice_variant") X(sgemm_unaligned, "sgemm.unaligned")                                                                     \
     X(gemm16_variant, "gemm16.variant") X(gemm16_mapping, "gemm16.mapping")                                 \
     X(gemm16_split_rows, "gemm16.split_rows") X(copy_blocks_per_cu, "copy.blocks_per_cu")                   \
     X(copy_nontemporal, "copy.nontemporal")
@@ -73,7 +73,7 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
 // with KO_OK, where nothing may be allocated (the stream is being captured into a graph and has no workspace
 // yet, 64 pairs already hold one, or the stream is hipStreamPerThread): the caller then takes its path without a
 // workspace.
-constexpr size_t kStreamWorkspaceBytes = size_t{8} << 20;
+constexpr size_t kStreamWorkspaceBytes = size_t{32} << 20;
 int stream_workspace(hipStream_t stream, void **workspace);
 
 }  // namespace ko

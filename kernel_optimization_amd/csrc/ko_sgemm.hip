@@ -802,48 +802,100 @@ int run(Params p, hipStream_t s, int variant) {
     }
 }
 
-// K slices for problems that are deep and have few output tiles (256 x 256 x 2048: 32 tiles of 32 x 64 on 256
-// compute units).  The slices are workgroups of one launch (blockIdx.y); their partial products go to
-// `workspace_bytes` of device memory and a second kernel sums them in slice order, so the result does not
-// depend on which slice finished first.  Returns the slice count (1: do not slice) and the slice depth; the
-// caller checks that slices x M x N floats fit its workspace (chosen by shape they are at most 64 x 64 floats
-// per compute unit).
-//   - operands as the direct-to-LDS kernels want them (rows on 16-byte boundaries);
-//   - tiles for at most half of the compute units, and as many slices as bring the launch up to one
-//     workgroup per compute unit, each at least 256 deep and a multiple of 128 (whole pairs of K tiles).
-int plan_k_slices(const Params &p, int *k_slice) {
-    *k_slice = 0;
+// K slices.  The slices are workgroups of one launch (blockIdx.y); their partial products go to a workspace and
+// a second kernel sums them in slice order, so the result does not depend on which slice finished first.
+// Operands must be as the direct-to-LDS kernels want them (rows on 16-byte boundaries).  Two cases:
+//   - few output tiles (tiles for at most half of the compute units, 256 x 256 x 2048: 32 tiles of 32 x 64 on 256
+//     CUs) and K >= 768: as many slices as bring the launch up to one workgroup per compute unit, each at
+//     least 256 deep and a multiple of 128 (whole pairs of K tiles); the tiling as for the unsliced problem;
+//   - more tiles, but rounds that do not fill the chip, and K >= 2048 (768 x 768 x 16384: 144 tiles of 64 x 64 on
+//     256 CUs, a round of K = 16384 at 56 % of the chip): the tiling and slice count that a cost model of the
+//     three tilings puts lowest - rounds x (fixed + per-64-k x depth / 64) + the summing kernel, the constants
+//     from K sweeps on this device - when that is at least a tenth below the best unsliced estimate (36 tiles
+//     of 128 x 128 in 7 slices: 252 workgroups, 253 -> 153 us; hipBLASLt 159 us).
+struct SlicePlan {
+    int slices = 1;   // 1: do not slice
+    int k_slice = 0;  // depth of every slice but the last
+    int variant = 0;  // tiling of the sliced launch (0: as run() picks it)
+};
+
+SlicePlan plan_k_slices(const Params &p, size_t workspace_bytes) {
+    SlicePlan plan;
     const int forced = tuning(knob_sgemm_k_slices);
-    if (forced == 1) return 1;
+    if (forced == 1) return plan;
     const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                          p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
-    if (!aligned) return 1;
+    if (!aligned) return plan;
     const int64_t cu = compute_units();
     const int64_t t64 = ((p.M + 63) / 64) * ((p.N + 63) / 64);
-    const int64_t tiles = 2 * t64 <= cu ? ((p.M + 31) / 32) * ((p.N + 63) / 64) : t64;  // as run() picks the tiling
-    // The second launch costs 2-3 us: below K = 768 the slices do not win them back (256 x 256 x 512: 7.0 us
-    // whole, 7.5 us in two slices; K = 768: 9.2 against 8.3; K = 2048: 19.8 against 11.1).
-    if (forced < 2 && p.K < 768) return 1;
-    int64_t slices = forced >= 2 ? forced : cu / tiles;
-    if (forced < 2 && slices > p.K / 256) slices = p.K / 256;
-    if (slices < 2) return 1;
-    const int64_t depth = ((p.K + slices - 1) / slices + 127) / 128 * 128;
-    slices = (p.K + depth - 1) / depth;
-    if (slices < 2 || slices > 65535) return 1;
-    *k_slice = static_cast<int>(depth);
-    return static_cast<int>(slices);
+    auto set = [&](int64_t slices, int variant) {
+        if (slices < 2) return;
+        const int64_t depth = ((p.K + slices - 1) / slices + 127) / 128 * 128;
+        slices = (p.K + depth - 1) / depth;
+        if (slices < 2 || slices > 65535) return;
+        plan.slices = static_cast<int>(slices);
+        plan.k_slice = static_cast<int>(depth);
+        plan.variant = variant;
+    };
+    if (forced >= 2) {
+        set(forced, tuning(knob_sgemm_slice_variant));
+        return plan;
+    }
+    if (2 * t64 <= cu) {
+        // The second launch costs 2-3 us: below K = 768 the slices do not win them back (256 x 256 x 512: 7.0 us
+        // whole, 7.5 us in two slices; K = 768: 9.2 against 8.3; K = 2048: 19.8 against 11.1).
+        if (p.K < 768) return plan;
+        const int64_t tiles = ((p.M + 31) / 32) * ((p.N + 63) / 64);  // run() takes 32 x 64 tiles here
+        int64_t slices = cu / tiles;
+        if (slices > p.K / 256) slices = p.K / 256;
+        set(slices, 0);
+        return plan;
+    }
+    if (p.K < 2048) return plan;
+    // us of one round of workgroups that are `depth` deep: {fixed, per 64 k}; rounds of one workgroup per
+    // compute unit (32 x 64 tiles: of two, which then take 1.2 us per 64 k instead of 0.5)
+    struct Tiling { int bm, bn, variant; double fixed, per64; int per_cu; };
+    const Tiling tilings[3] = {{128, 128, 0, 6.0, 3.67, 1}, {64, 64, 0, 5.2, 0.95, 1}, {32, 64, 41, 4.2, 1.2, 2}};
+    const double out_bytes = 4.0 * p.M * p.N;
+    double best_whole = 1e30, best_sliced = 1e30;
+    int64_t best_slices = 1;
+    int best_variant = 0;
+    for (const Tiling &t : tilings) {
+        const int64_t tiles = static_cast<int64_t>((p.M + t.bm - 1) / t.bm) * ((p.N + t.bn - 1) / t.bn);
+        const int64_t slots = cu * t.per_cu;
+        for (int64_t slices = 1; slices <= 64 && p.K / slices >= 512; ++slices) {
+            if (slices > 1 && slices * out_bytes > static_cast<double>(workspace_bytes)) break;
+            const int64_t depth = slices == 1 ? p.K : ((p.K + slices - 1) / slices + 127) / 128 * 128;
+            const int64_t groups = tiles * ((p.K + depth - 1) / depth);
+            const int64_t rounds = (groups + slots - 1) / slots;
+            const double per64 = t.per_cu == 2 && groups <= cu ? 0.5 : t.per64;
+            double us = rounds * (t.fixed + per64 * depth / 64.0);
+            if (slices == 1) {
+                if (us < best_whole) best_whole = us;
+                continue;
+            }
+            us += 2.5 + (slices + 1) * out_bytes / 5e6;  // the summing kernel: its launch, partial products in, D out
+            if (us < best_sliced) {
+                best_sliced = us;
+                best_slices = slices;
+                best_variant = t.variant != 0 ? t.variant : t.bm == 128 ? (depth >= 2048 ? 40 : 36) : (depth % 256 == 0 ? 35 : 33);
+            }
+        }
+    }
+    if (best_sliced < 0.9 * best_whole) set(best_slices, best_variant);
+    return plan;
 }
 
 // The K-sliced form of one problem: partial products into `workspace`, then their sum and the epilogue.
-int run_sliced(const Params &p, int slices, int k_slice, float *workspace, hipStream_t s) {
+int run_sliced(const Params &p, const SlicePlan &plan, float *workspace, hipStream_t s) {
     Params part = p;
     part.C = nullptr;
     part.D = workspace;
     part.alpha = 1.0f;
     part.beta = 0.0f;
-    part.k_slice = k_slice;
-    if (const int st = run(part, s, 0); st != KO_OK) return st;
-    return sum_slices(workspace, slices, p, s);
+    part.k_slice = plan.k_slice;
+    if (const int st = run(part, s, plan.variant); st != KO_OK) return st;
+    return sum_slices(workspace, plan.slices, p, s);
 }
 
 // The address of `scratch` on the current device (looked up once per device).
@@ -880,8 +932,8 @@ int sgemm(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const fl
     hipStream_t s = as_stream(stream);
     const int variant = tuning(knob_sgemm_variant);
     if (variant <= 0) {
-        int k_slice = 0;
-        if (const int slices = plan_k_slices(p, &k_slice); slices > 1) {
+        if (const SlicePlan plan = plan_k_slices(p, sizeof(scratch)); plan.slices > 1) {
+            const int slices = plan.slices;
             const uint64_t need = static_cast<uint64_t>(slices) * m * n * sizeof(float);
             void *workspace = nullptr;
             if (own_scratch) {
@@ -893,7 +945,7 @@ int sgemm(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const fl
             } else if (need <= kStreamWorkspaceBytes) {
                 if (const int st = stream_workspace(s, &workspace); st != KO_OK) return st;
             }
-            if (workspace != nullptr) return run_sliced(p, slices, k_slice, static_cast<float *>(workspace), s);
+            if (workspace != nullptr) return run_sliced(p, plan, static_cast<float *>(workspace), s);
         }
     }
     if (variant <= 0 && tuning(knob_sgemm_split_rows) != 1 && k >= 512) {

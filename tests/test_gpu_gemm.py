@@ -102,6 +102,31 @@ def test_sgemm_deep_k_on_few_tiles_is_cut_into_slices(ko, sgemm_k_slices, m, n, 
         np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=f"k_slices={slices}")
 
 
+@pytest.mark.parametrize("m,n,k", [(768, 768, 4096), (1280, 1280, 4096), (700, 836, 2052), (1536, 640, 8192)])
+def test_sgemm_rounds_that_do_not_fill_the_chip_are_sliced(ko, sgemm_k_slices, m, n, k):
+    """More tiles than half the compute units but rounds that leave many of them idle, and a deep K: the
+    planner's cost model picks a tiling and a slice count (128 x 128 tiles in seven slices for the first shape).
+    Exact on small integers, whichever plan it takes, and equal to the unsliced result."""
+    rng = np.random.default_rng(m + n + k)
+    A = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    B = rng.integers(-3, 4, (k, n)).astype(np.float32)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    for slices in (0, 1):
+        sgemm_k_slices(slices)
+        np.testing.assert_array_equal(ko.sgemm_host(A, B), ref, err_msg=f"k_slices={slices}")
+        np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=f"k_slices={slices}")
+    for variant in (36, 40, 35, 41):  # forced plans on every tiling the planner can choose
+        ko.set_tuning("sgemm.slice_variant", variant)
+        try:
+            for slices in (3, 7):
+                sgemm_k_slices(slices)
+                np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C,
+                                              err_msg=f"variant={variant} k_slices={slices}")
+        finally:
+            ko.set_tuning("sgemm.slice_variant", 0)
+
+
 def test_sgemm_k_slices_against_oracle_and_repeatable(ko, sgemm_k_slices):
     """Uniform inputs through the sliced path: within the fp32 summation bound of the oracle, bit-identical
     from call to call (the partial products are summed in slice order, not in order of arrival), and the

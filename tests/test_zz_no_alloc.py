@@ -28,9 +28,11 @@ def _both(ko, m, n, k, seed, with_c):
 def test_static_scratch_sgemm_gives_the_bits_of_the_allocating_entry_point(ko):
     import oracle
     from tolerances import assert_sgemm_close
-    # sliced (32 tiles, 8 slices), then a smaller sliced problem with ragged tiles and a ragged last slice, then
-    # one that is not sliced at all
-    for (m, n, k), with_c in (((256, 256, 2048), False), ((100, 72, 1300), True), ((512, 384, 256), True)):
+    # sliced by the cost model (36 tiles of 128 x 128 in seven slices: 16.5 MiB of partial products), then by the
+    # few-tiles rule (32 tiles, 8 slices), then a smaller sliced problem with ragged tiles and a ragged last
+    # slice, then one that is not sliced at all
+    for (m, n, k), with_c in (((768, 768, 4096), True), ((256, 256, 2048), False), ((100, 72, 1300), True),
+                              ((512, 384, 256), True)):
         A, B, C, alpha, beta, want, got = _both(ko, m, n, k, 900 + m, with_c)
         np.testing.assert_array_equal(got, want, err_msg=str((m, n, k)))
         ref, ap = oracle.sgemm(A, B, C, alpha, beta, want_absprod=True)
@@ -39,7 +41,7 @@ def test_static_scratch_sgemm_gives_the_bits_of_the_allocating_entry_point(ko):
 
 
 def test_static_scratch_sgemm_refuses_what_does_not_fit(ko):
-    m, n, k = 1024, 1024, 4096  # 16 forced slices of 4 MiB each against an array of 8 MiB
+    m, n, k = 1024, 1024, 4096  # 16 forced slices of 4 MiB each against an array of 32 MiB
     buf = ko.DeviceBuffer(m * k * 4)
     out = ko.DeviceBuffer(m * n * 4)
     ko.set_tuning("sgemm.k_slices", 16)
