@@ -577,6 +577,120 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
     }
 }
 
+// Rows of a few vectors per thread (up to 2048 vectors: 8192 fp32 columns): one workgroup per group of R rows,
+// dispatched in row order and gone when its rows are written (a one-shot launch keeps the memory system busier
+// than a grid that walks the rows in step: [32768, 4096] without gamma and beta 181 -> 165 us, the time of the
+// softmax on the same rows).  gamma and beta have to be fetched by every workgroup, from L2: with R rows held in
+// registers at once they are fetched once per R rows, and the R triplets share the barrier of the
+// workgroup-wide all-reduce ([52428, 2560]: walking grid 194 us, one row per workgroup 189 us, two 174 us).
+template <int IO, int THREADS, int VPL, int R>
+__global__ __launch_bounds__(THREADS) void layernorm_block_batch_kernel(const typename Io<IO>::elem *in,
+                                                                        typename Io<IO>::elem *out,
+                                                                        float *__restrict__ mean_out,
+                                                                        float *__restrict__ rstd_out,
+                                                                        const typename Io<IO>::elem *__restrict__ gamma,
+                                                                        const typename Io<IO>::elem *__restrict__ beta,
+                                                                        int64_t rows, int cols, float eps,
+                                                                        float inv_denominator) {
+    constexpr int E = Io<IO>::E;
+    constexpr int WAVES = THREADS / 64;
+    typedef typename Io<IO>::raw Raw;
+    __shared__ float lds[R * 3 * 16];
+    constexpr Reciprocals<VPL * E> rcp;
+    const int nvec = cols / E;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+    const uint32_t first = threadIdx.x * 16u;
+    constexpr uint32_t kStep = THREADS * 16u;
+
+    Raw loaded[R][VPL];  // all loads first, conversions afterwards
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const typename Io<IO>::elem *src = in + (row0 + r) * cols;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            loaded[r][k] = Raw{};
+            if (row0 + r < rows && j < nvec) loaded[r][k] = Io<IO>::template load_raw<true>(at_bytes(src, first + k * kStep));
+        }
+    }
+    float x0[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) x0[r] = row0 + r < rows ? Io<IO>::scalar(in + (row0 + r) * cols) : 0.0f;
+    // gamma and beta behind the rows: memory returns in order, and the statistics do not need them
+    float g[VPL][E], b[VPL][E];
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+        const int j = threadIdx.x + k * THREADS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            g[k][e] = 1.0f;
+            b[k][e] = 0.0f;
+        }
+        if (j < nvec) {
+            if (gamma) Io<IO>::template load<false>(gamma + E * j, g[k]);
+            if (beta) Io<IO>::template load<false>(beta + E * j, b[k]);
+        }
+    }
+
+    float v[R][VPL][E];
+    wave::Welford w[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        w[r] = wave::Welford{0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            Io<IO>::unpack(loaded[r][k], v[r][k]);
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[r][k][e] -= x0[r];
+            if (j < nvec) {  // a thread's valid vectors are its first ones, so the n-th element it folds has count n
+#pragma unroll
+                for (int e = 0; e < E; ++e) welford_update(w[r], v[r][k][e], rcp.v[E * k + e + 1]);
+            }
+        }
+        w[r] = wave::welford_allreduce<64>(w[r]);
+    }
+    if constexpr (WAVES > 1) {
+        if ((threadIdx.x & 63) == 0) {
+            const int wv = threadIdx.x >> 6;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                lds[(3 * r + 0) * 16 + wv] = w[r].count;
+                lds[(3 * r + 1) * 16 + wv] = w[r].mean;
+                lds[(3 * r + 2) * 16 + wv] = w[r].m2;
+            }
+        }
+        __syncthreads();
+        const int i = threadIdx.x & (WAVES - 1);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            w[r] = wave::welford_allreduce<WAVES>(
+                wave::Welford{lds[(3 * r + 0) * 16 + i], lds[(3 * r + 1) * 16 + i], lds[(3 * r + 2) * 16 + i]});
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t row = row0 + r;
+        if (row >= rows) break;
+        const float mean = w[r].mean;  // of the shifted row
+        const float rstd = rsqrt_1ulp(w[r].m2 * inv_denominator + eps);
+        typename Io<IO>::elem *dst = out + row * cols;
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
+            if (j < nvec) {
+                float y[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[r][k][e] - mean) * rstd, g[k][e], b[k][e]);
+                Io<IO>::store_stream(dst, first + k * kStep, y);
+            }
+        }
+        if (threadIdx.x == 0) {
+            if (mean_out) mean_out[row] = rstd != rstd ? rstd : x0[r] + mean;  // no statistics for a row with NaN or inf
+            if (rstd_out) rstd_out[row] = rstd;
+        }
+    }
+}
+
 // ------------------------------------------------------------------ dispatch
 template <int IO, int LPR, int VPL, bool FULL>
 int launch_wave_full(const Args<IO> &a) {
@@ -723,10 +837,52 @@ int launch_block_threads(const Args<IO> &a) {
     return KO_OK;
 }
 
+// Rows of 513 to 2048 vectors: layernorm_block_batch_kernel with 512 threads, one row per workgroup without
+// gamma and beta, two rows with them.
+template <int IO>
+int launch_block_batch(const Args<IO> &a) {
+    const int nvec = a.cols / Io<IO>::E;
+    const int vpl = (nvec + 511) / 512;
+    int r = tuning(knob_layernorm_block_rows);
+    if (r != 1 && r != 2) r = a.gamma != nullptr || a.beta != nullptr ? 2 : 1;
+    const int64_t grid = (a.rows + r - 1) / r;
+    if (grid > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: too many rows");
+    const dim3 g(static_cast<unsigned>(grid)), b(512);
+#define KO_LN_BATCH(V)                                                                                          \
+    do {                                                                                                        \
+        if (r == 1)                                                                                             \
+            layernorm_block_batch_kernel<IO, 512, V, 1><<<g, b, 0, a.stream>>>(a.in, a.out, a.mean, a.rstd, a.gamma, \
+                                                                              a.beta, a.rows, a.cols, a.eps,   \
+                                                                              a.inv_denominator);              \
+        else                                                                                                    \
+            layernorm_block_batch_kernel<IO, 512, V, 2><<<g, b, 0, a.stream>>>(a.in, a.out, a.mean, a.rstd, a.gamma, \
+                                                                              a.beta, a.rows, a.cols, a.eps,   \
+                                                                              a.inv_denominator);              \
+    } while (0)
+    if (vpl <= 2) KO_LN_BATCH(2);
+    else if (vpl <= 3) KO_LN_BATCH(3);
+    else KO_LN_BATCH(4);
+#undef KO_LN_BATCH
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 template <int IO>
 int launch_block(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     int threads = tuning(knob_layernorm_block_threads);
+    // Rows of 513 to 2048 vectors (2052 to 8192 fp32 columns) as a one-shot launch: without gamma and beta one row
+    // per workgroup; with them two rows per workgroup, which share their fetch - unless rows lie a multiple of
+    // 8 KB apart: two rows, gamma and beta then fall on the same memory channels at the same moment, and the
+    // walking grid below, which keeps gamma and beta in registers, is the faster one ([32768, 4096]: 181 us
+    // walking, 188 us two rows per workgroup; [43690, 3072]: 192 and 175 us; without gamma and beta 181 -> 165 us
+    // and 191 -> 162 us).  Knob layernorm.block_rows: -1 walking grid always, 1 or 2 rows per workgroup.
+    if (nvec > 512 && nvec <= 2048 && threads == 0 && tuning(knob_rows_block_grid) == 0) {
+        const int forced = tuning(knob_layernorm_block_rows);
+        const bool affine = a.gamma != nullptr || a.beta != nullptr;
+        const bool rows_on_one_channel = (static_cast<int64_t>(a.cols) * sizeof(typename Io<IO>::elem)) % 8192 == 0;
+        if (forced == 1 || forced == 2 || (forced == 0 && (!affine || !rows_on_one_channel))) return launch_block_batch<IO>(a);
+    }
     if (threads != 256 && threads != 512 && threads != 1024) {
         // up to eight vectors per thread before the workgroup grows: gamma and beta then still fit the registers
         // next to the row at 256 and 512 threads ([8192, 16384]: 512 threads 181 us, 1024 threads 186 us)

@@ -115,6 +115,26 @@ def test_layernorm16_block_policies(ko, policy, rows, cols, bf16):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,cols", [(7, 4104), (5, 5120), (9, 8192), (3, 12296), (4, 16384)])
+def test_layernorm16_rows_of_a_few_vectors_per_thread(ko, rows, cols, bf16):
+    """16-bit storage through the one-shot BLOCK kernel (513 to 2048 vectors of eight values), one and two rows per
+    workgroup, with and without gamma and beta, and through the walking grid."""
+    dt = ko.BF16 if bf16 else ko.F16
+    xb = _bits(inputs.normal_f32((rows, cols), 130 + cols, 0.5, 2.0), bf16)
+    gb = _bits(inputs.normal_f32((cols,), 131, 1.0, 0.1), bf16)
+    bb = _bits(inputs.normal_f32((cols,), 132, 0.0, 0.1), bf16)
+    try:
+        for g_, b_ in ((gb, bb), (None, None)):
+            _, ref64, rmean, rrstd = oracle.layernorm16(xb, g_, b_, 1e-5, False, bf16)
+            for block_rows in (0, 1, 2, -1):
+                ko.set_tuning("layernorm.block_rows", block_rows)
+                y, mean, rstd = ko.layernorm16_host(xb, g_, b_, 1e-5, False, dtype=dt, policy=2)
+                assert_layernorm16_close((_to64(y, bf16), mean, rstd), (ref64, rmean, rrstd), bf16)
+    finally:
+        ko.set_tuning("layernorm.block_rows", 0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
 def test_layernorm16_plain_in_place_and_errors(ko, bf16):
     dt = ko.BF16 if bf16 else ko.F16
     xb = _bits(inputs.normal_f32((60, 768), 120, 0.5, 2.0), bf16)

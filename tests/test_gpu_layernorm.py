@@ -52,6 +52,28 @@ def test_layernorm_block_policies(ko, policy, rows, cols):
     assert_layernorm_close(ko.layernorm_host(x, g, b, policy=policy), oracle.layernorm(x, g, b))
 
 
+@pytest.mark.parametrize("affine", [True, False])
+@pytest.mark.parametrize("rows,cols", [(7, 2052), (33, 2560), (9, 3072), (5, 4096), (11, 5000), (3, 6148), (6, 7168), (4, 8192)])
+def test_layernorm_rows_of_a_few_vectors_per_thread(ko, rows, cols, affine):
+    """2052 to 8192 columns through the default dispatch and through each form it chooses between: the one-shot
+    kernel with one and with two rows per workgroup (odd row counts leave the last workgroup a single row; row
+    lengths that do not fill the last vector of every thread; gamma and beta present or absent) and the walking
+    grid.  Every form against the oracle, in place as well."""
+    x, g, b = _case(rows, cols, 1300 + cols)
+    if not affine:
+        g = b = None
+    ref = oracle.layernorm(x, g, b)
+    try:
+        for block_rows in (0, 1, 2, -1):
+            ko.set_tuning("layernorm.block_rows", block_rows)
+            for policy in (0, 2):
+                assert_layernorm_close(ko.layernorm_host(x, g, b, policy=policy), ref)
+            assert_layernorm_close(ko.layernorm_host(x, g, b, policy=2, in_place=True), ref)
+            assert_layernorm_close(ko.layernorm_host(x, g, b, unbiased=True, policy=2), oracle.layernorm(x, g, b, unbiased=True))
+    finally:
+        ko.set_tuning("layernorm.block_rows", 0)
+
+
 def test_layernorm_optional_arguments(ko):
     """gamma, beta, mean and rstd are independently optional (the reference runs with affine off,
     nn_operators/layernorm/main.cu:22)."""
