@@ -664,6 +664,11 @@ def main():
         res, _ = bench_sgemm(3, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(256, 256, 2048))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
+        # a weight-gradient shape: 144 tiles of 64 x 64 would leave 112 compute units idle; the planner takes
+        # 36 tiles of 128 x 128 in seven slices of K
+        res, _ = bench_sgemm(3, args.steps, args.warmup, vendor, shape=(768, 768, 16384))
+        res["steps"], res["warmup"] = args.steps, args.warmup
+        others.append(res)
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16000, 3072, 768))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)

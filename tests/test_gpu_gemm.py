@@ -127,6 +127,20 @@ def test_sgemm_rounds_that_do_not_fill_the_chip_are_sliced(ko, sgemm_k_slices, m
             ko.set_tuning("sgemm.slice_variant", 0)
 
 
+def test_sgemm_random_deep_shapes_are_exact_on_small_integers(ko):
+    """Random shapes with K of 2048 and more, through the default dispatch: whatever the planner decides (whole,
+    few-tiles slices, or a tiling and slice count from its cost model), small integers must come out exact."""
+    rng = np.random.default_rng(23)
+    for _ in range(10):
+        m, n = int(rng.integers(20, 400)) * 4, int(rng.integers(20, 400)) * 4
+        k = int(rng.integers(512, 1500)) * 4
+        A = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        B = rng.integers(-3, 4, (k, n)).astype(np.float32)
+        C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+        ref = A.astype(np.float64) @ B.astype(np.float64)
+        np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C, err_msg=str((m, n, k)))
+
+
 def test_sgemm_k_slices_against_oracle_and_repeatable(ko, sgemm_k_slices):
     """Uniform inputs through the sliced path: within the fp32 summation bound of the oracle, bit-identical
     from call to call (the partial products are summed in slice order, not in order of arrival), and the
