@@ -724,7 +724,7 @@ int launch_direct(Params p, hipStream_t stream) {
 template <bool VEC>
 __global__ __launch_bounds__(64) void sgemm_slices_sum_kernel(const float *__restrict__ partials, int slices,
                                                               int64_t count, float alpha, float beta,
-                                                              const float *__restrict__ C, float *__restrict__ D) {
+                                                              const float *C, float *D) {  // C may be D
     constexpr int W = VEC ? 4 : 1;
     typedef float vec_t __attribute__((ext_vector_type(W)));
     const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x) * W;
