@@ -155,6 +155,11 @@ def test_sgemm_k_slices_against_oracle_and_repeatable(ko, sgemm_k_slices):
         np.testing.assert_array_equal(ko.sgemm_host(A, B), first)
     ref2, ap2 = oracle.sgemm(A, B, C, 0.5, -2.0, want_absprod=True)
     assert_sgemm_close(ko.sgemm_host(A, B, C, 0.5, -2.0), ref2, 0.5 * ap2 + 2.0 * np.abs(C) + 1e-6, k)
+    # C and D the same buffer (D = alpha A B + beta D): the summing kernel reads C where it writes D
+    dA, dB, dD = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B), ko.DeviceBuffer.from_numpy(C)
+    ko.sgemm(m, n, k, dA, dB, dD, dD, 0.5, -2.0)
+    ko.synchronize()
+    assert_sgemm_close(dD.download(np.float32, (m, n)), ref2, 0.5 * ap2 + 2.0 * np.abs(C) + 1e-6, k)
     sgemm_k_slices(1)
     assert_sgemm_close(ko.sgemm_host(A, B), ref, ap, k)
 
