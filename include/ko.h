@@ -191,7 +191,10 @@ int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, co
  * the reference's layout, tensor_core_gemm.h:178) or column-major (KO_COL_MAJOR:
  * memory [n][k]); C, D [m,n] row-major.  Elements are binary16 or bfloat16
  * (in_dtype); products accumulate in fp32 on the matrix cores; D is rounded once
- * to the 16-bit type.  C may be NULL.  k must be a multiple of 8; A, B, C, D 16-byte aligned. */
+ * to the 16-bit type.  C may be NULL.  k must be a multiple of 8; A, B, C, D 16-byte aligned.
+ * Workspace: like ko_sgemm_f32, a deep K (k >= 2048) on few output tiles is cut into slices of K whose fp32
+ * partial products go through the 32 MiB workspace of the (device, stream) pair, allocated at the first such
+ * call on the stream; a first such call inside a graph capture allocates nothing and runs unsliced. */
 int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A, const void *B,
                       int b_layout, float beta, const void *C, void *D, int in_dtype,
                       ko_stream_t stream);

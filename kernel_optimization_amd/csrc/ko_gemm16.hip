@@ -123,6 +123,11 @@ struct Params {
     int act;                    // KO_ACT_*
     int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
     int ldb;                    // row-major B: elements between its rows (N, or more likewise)
+    // K slices (gemm16_kernel only): workgroups with blockIdx.y = s multiply k in [s * k_slice, (s + 1) * k_slice) and
+    // write their M x N partial product as fp32 (no alpha, C, bias or activation) behind partial + s * M * N
+    int k_slice;                // 0: no slices
+    float *partial;
+    int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
 };
 
 // x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
@@ -364,8 +369,46 @@ __device__ __forceinline__ u32x4 read_b_transposed(const u32x4 *sb, int k0, int 
     return __builtin_bit_cast(u32x4, static_cast<short8v>(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7)));
 }
 
+// The problem a workgroup of a K-sliced launch works on: its K range of A and B, its own partial product.
+template <bool B_ROW_MAJOR>
+__device__ __forceinline__ Params slice_of(Params p) {
+    if (p.k_slice > 0) {
+        const int s = static_cast<int>(blockIdx.y);
+        const int k0 = s * p.k_slice;
+        p.A += k0;
+        p.B += B_ROW_MAJOR ? static_cast<int64_t>(k0) * p.ldb : static_cast<int64_t>(k0);
+        p.partial += static_cast<int64_t>(s) * p.M * p.N;
+        p.K = p.K - k0 < p.k_slice ? p.K - k0 : p.k_slice;
+    }
+    return p;
+}
+
+// One wave's accumulator tile as fp32 into a partial product (rows of N floats; N a multiple of 4, so a lane's four
+// consecutive columns are inside the matrix together or not at all).
+template <int WTM, int WTN>
+__device__ __forceinline__ void store_partial(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], int lane, int row0,
+                                              int col0) {
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < WTM / 32; ++i) {
+        const int m = row0 + i * 32 + frow;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < WTN / 32; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = col0 + j * 32 + 8 * q + 4 * fhalf;
+                if (n >= p.N) continue;
+                const float4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                *reinterpret_cast<float4v *>(p.partial + static_cast<int64_t>(m) * p.N + n) = v;
+            }
+    }
+}
+
 template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
-__global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
+__global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params whole) {
+    const Params p = slice_of<B_ROW_MAJOR>(whole);
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N, REG_STAGES = T::REG_STAGES;
     constexpr bool FRAG_DB = T::FRAG_DB;
     constexpr int SWIZZLE = T::SWIZZLE;
@@ -389,6 +432,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
     const int m0 = (tile / p.tiles_n) * BM;
     const int n0 = (tile % p.tiles_n) * BN;
     const int M = p.M, N = p.N, K = p.K;
+    const int ldk = p.ldk;
 
     const int KT = (K + kBK - 1) / kBK;
 
@@ -400,7 +444,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
     // and K tile: scalar registers) plus a per-lane byte offset that never changes, so the
     // loads need one offset register instead of a 64-bit pointer each.
     constexpr int ROWS_PER_ITER = THREADS / kChunks;  // rows covered by one load instruction of the workgroup
-    const uint32_t lane_off_a = static_cast<uint32_t>((tid / kChunks) * K + (tid % kChunks) * 8) * 2u;
+    const uint32_t lane_off_a = static_cast<uint32_t>((tid / kChunks) * ldk + (tid % kChunks) * 8) * 2u;
 
     auto load_global = [&](int kt, auto slot) {
         constexpr int S = decltype(slot)::value;
@@ -414,10 +458,10 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
             if constexpr (EDGE) {
                 gr = gr < M ? gr : M - 1;  // rows past the edge re-read the last row; their results are never stored
                 u32x4 v = {0u, 0u, 0u, 0u};
-                if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.A + static_cast<int64_t>(gr) * K + kc);
+                if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.A + static_cast<int64_t>(gr) * ldk + kc);
                 ra[S][i] = v;
             } else {
-                const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + i * ROWS_PER_ITER) * K + k0);
+                const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + i * ROWS_PER_ITER) * ldk + k0);
                 ra[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
             }
         }
@@ -431,10 +475,10 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
                 if constexpr (EDGE) {
                     gr = gr < N ? gr : N - 1;
                     u32x4 v = {0u, 0u, 0u, 0u};
-                    if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.B + static_cast<int64_t>(gr) * K + kc);
+                    if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.B + static_cast<int64_t>(gr) * ldk + kc);
                     rb[S][i] = v;
                 } else {
-                    const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + i * ROWS_PER_ITER) * K + k0);
+                    const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + i * ROWS_PER_ITER) * ldk + k0);
                     rb[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
                 }
             }
@@ -570,7 +614,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params p) {
         if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
     }
 
-    store_tile<WTM, WTN, SWIZZLE, BF16, EDGE>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+    if (p.partial != nullptr) store_partial<WTM, WTN>(p, acc, lane, m0 + wm * WTM, n0 + wn * WTN);
+    else store_tile<WTM, WTN, SWIZZLE, BF16, EDGE>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
 }
 
 // Direct-to-LDS kernels for full tiles with K-contiguous operands (column-major B):
@@ -1157,7 +1202,8 @@ int launch_edge(const Params &p, hipStream_t stream) {
     static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK)
         return st;
-    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(THREADS), lds_bytes, stream>>>(p);
+    const int slices = p.k_slice > 0 ? (p.K + p.k_slice - 1) / p.k_slice : 1;
+    kernel<<<dim3(static_cast<unsigned>(p.nblocks), static_cast<unsigned>(slices)), dim3(THREADS), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
@@ -1167,7 +1213,8 @@ int launch(Params p, hipStream_t stream) {
     const int tiles_m = (p.M + T::BM - 1) / T::BM;
     p.tiles_n = (p.N + T::BN - 1) / T::BN;
     p.nblocks = tiles_m * p.tiles_n;
-    const bool edge = (p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0;
+    // K slices are a multiple of the K tile deep; only the last one can end inside a K tile
+    const bool edge = (p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % kBK) != 0 || (p.k_slice % kBK) != 0;
     if (edge) return launch_edge<T, BF16, B_ROW_MAJOR, true>(p, stream);
     return launch_edge<T, BF16, B_ROW_MAJOR, false>(p, stream);
 }
@@ -1193,6 +1240,106 @@ int launch_direct(const Params &p, hipStream_t stream) {
     }
 }
 
+// D = act(alpha * (P_0 + ... + P_{slices-1}) + beta * C + bias), rounded once, from the fp32 partial products of a
+// K-sliced launch, summed in slice order.  One thread per four consecutive columns.
+template <bool BF16>
+__global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, int slices) {
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    const int groups_per_row = p.N / 4;
+    const int64_t g = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
+    if (g >= static_cast<int64_t>(p.M) * groups_per_row) return;
+    const int m = static_cast<int>(g / groups_per_row), n = static_cast<int>(g % groups_per_row) * 4;
+    const int64_t count = static_cast<int64_t>(p.M) * p.N;
+    const float *src = p.partial + static_cast<int64_t>(m) * p.N + n;
+    float4v acc = *reinterpret_cast<const float4v *>(src);
+    int s = 1;
+    for (; s + 8 <= slices; s += 8) {
+        float4v t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = *reinterpret_cast<const float4v *>(src + (s + j) * count);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += t[j];
+    }
+    for (; s < slices; ++s) acc += *reinterpret_cast<const float4v *>(src + s * count);
+    const bool use_c = p.C != nullptr && p.beta != 0.0f;
+    const int64_t off = static_cast<int64_t>(m) * p.ldd + n;
+    u32x2 c2 = {0, 0}, b2 = {0, 0};
+    if (use_c) c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+    if (p.bias) b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
+    float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+    finish4<BF16>(p, v, c2, b2, use_c);
+    u32x2 o;
+    o[0] = pack2<BF16>(v[0], v[1]);
+    o[1] = pack2<BF16>(v[2], v[3]);
+    *reinterpret_cast<u32x2 *>(p.D + off) = o;
+}
+
+// K slices for a deep K on few output tiles (weight-gradient shapes: 768 x 768 x 16384 is 36 tiles of 128 x 128).
+// As in the SGEMM: the slices are workgroups of one launch of the register pipeline (blockIdx.y), their fp32 partial
+// products go to the stream's workspace, a second kernel sums them in slice order and applies the whole epilogue
+// once.  From K = 2048 on, by tile count (measured against the whole problem, us):
+//   - at most a quarter of the compute units' worth of 128 x 128 tiles: slices at least 512 deep up to one
+//     workgroup per compute unit, of 128 x 128 or 64 x 64 tiles, whichever comes closer to that (64 x 64 on a tie):
+//     768 x 768 x 16384 82 -> 40 (7 slices of 36 tiles), 512 x 512 x 8192 43 -> 18, 256 x 256 x 16384 81 -> 15,
+//     1024 x 1024 x 8192 46 -> 34;
+//   - up to one such tile per compute unit: slices at least 2048 deep up to two workgroups per compute unit:
+//     768 x 2304 x 16384 130 -> 97 (4 slices of 108 tiles), 768 x 3072 x 16384 172 -> 121; shallower slices lose
+//     (2048 x 768 x 3072: 25.5 whole, 27 in four slices).
+struct SlicePlan16 {
+    int slices = 1, k_slice = 0;
+    bool tiles_128 = false;  // 128 x 128 tiles (else 64 x 64)
+};
+
+SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
+    SlicePlan16 plan;
+    const int forced = tuning(knob_gemm16_k_slices);
+    if (forced == 1 || p.N % 8 != 0 || p.ldd % 4 != 0) return plan;
+    const int64_t cu = compute_units();
+    const double out_bytes = 4.0 * p.M * p.N;
+    auto set = [&](int64_t slices, bool tiles_128) {
+        if (slices < 2) return;
+        const int64_t depth = ((p.K + slices - 1) / slices + kBK - 1) / kBK * kBK;
+        slices = (p.K + depth - 1) / depth;
+        if (slices < 2 || slices > 65535 || slices * out_bytes > static_cast<double>(workspace_bytes)) return;
+        plan.slices = static_cast<int>(slices);
+        plan.k_slice = static_cast<int>(depth);
+        plan.tiles_128 = tiles_128;
+    };
+    const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
+    const int64_t t64 = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64);
+    if (forced >= 2) {
+        set(forced, t128 * forced >= cu / 2);
+        return plan;
+    }
+    if (p.K < 2048) return plan;
+    const int64_t fit = static_cast<int64_t>(static_cast<double>(workspace_bytes) / out_bytes);  // slices the workspace holds
+    auto capped = [&](int64_t slices, int64_t min_depth) {
+        if (slices > p.K / min_depth) slices = p.K / min_depth;
+        return slices < fit ? slices : fit;
+    };
+    if (4 * t128 <= cu) {
+        const int64_t s128 = capped(cu / t128, 512), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
+        if (s64 >= 2 && s64 * t64 >= s128 * t128) set(s64, false);
+        else set(s128, true);
+    } else if (t128 <= cu) {
+        set(capped(2 * cu / t128, 2048), true);
+    }
+    return plan;
+}
+
+template <bool BF16, bool B_ROW_MAJOR>
+int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hipStream_t stream) {
+    Params part = p;
+    part.k_slice = plan.k_slice;
+    part.partial = workspace;
+    int st = plan.tiles_128 ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream) : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
+    if (st != KO_OK) return st;
+    const int64_t groups = static_cast<int64_t>(p.M) * (p.N / 4);
+    gemm16_slices_sum_kernel<BF16><<<dim3(static_cast<unsigned>((groups + 63) / 64)), dim3(64), 0, stream>>>(part, plan.slices);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 // One call becomes at most five launches: one column cut (left, right), then at most two row cuts in the left
 // part (the rows below the last full round, and of those the rows below the last full tile row) and one in the
 // right part.  col_cut / row_cuts are what a (sub-)problem may still spend; the knobs are read once per call.
@@ -1203,6 +1350,17 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         variant = tuning(knob_gemm16_variant);
         split_knob = tuning(knob_gemm16_split_rows);
         if (variant < 0) variant = 0;
+    }
+    if (variant <= 0 && col_cut && row_cuts == 2 && p.k_slice == 0) {
+        // the whole problem, before any cut: few tiles and a deep K go out as K slices
+        const int64_t big = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
+        if (2 * big < compute_units()) {
+            if (const SlicePlan16 plan = plan_k_slices16(p, kStreamWorkspaceBytes); plan.slices > 1) {
+                void *workspace = nullptr;
+                if (const int st = stream_workspace(stream, &workspace); st != KO_OK) return st;
+                if (workspace != nullptr) return run_sliced16<BF16, B_ROW_MAJOR>(p, plan, static_cast<float *>(workspace), stream);
+            }
+        }
     }
     if (variant <= 0) {
         // Enough 256x256 tiles to fill the chip: the big tiling - as a persistent direct-to-LDS kernel
@@ -1323,7 +1481,8 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
     Params p{static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B),
              static_cast<const uint16_t *>(C), static_cast<uint16_t *>(D),
              static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, 0, 0,
-             static_cast<const uint16_t *>(bias), activation, static_cast<int>(n), static_cast<int>(n)};
+             static_cast<const uint16_t *>(bias), activation, static_cast<int>(n), static_cast<int>(n),
+             0, nullptr, static_cast<int>(k)};
     hipStream_t s = as_stream(stream);
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);

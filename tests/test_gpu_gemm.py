@@ -532,6 +532,33 @@ def test_gemm16_bias_activation(ko, act, bf16, b_col_major, m, n, k):
         assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k,slices", [(512, 512, 8192, 0), (256, 384, 2048, 3), (300, 520, 1096, 2), (768, 768, 4096, 7),
+                                          (130, 72, 4104, 5)])
+def test_gemm16_k_slices(ko, m, n, k, slices, b_col_major, bf16):
+    """A deep K on few tiles goes out as K slices of the register pipeline (fp32 partial products into the stream's
+    workspace) and a kernel that sums them in slice order and applies alpha, beta C, bias and the activation once.
+    slices = 0: the planner's own choice; otherwise a forced count (ragged tiles, a last slice that ends inside
+    a K tile).  Against the oracle, plain and with the whole epilogue, and bit-stable from call to call."""
+    A = _bits16((m, k), 71 + m, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 73 + n, bf16)
+    C = _bits16((m, n), 75, bf16)
+    bias = _bits16((n,), 77, bf16)
+    kw = dict(b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR, dtype=ko.BF16 if bf16 else ko.F16)
+    ko.set_tuning("gemm16.k_slices", slices)
+    try:
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16)
+        got = ko.gemm16_host(A, B, m, n, k, **kw)
+        assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+        np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, **kw), got)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16, C_bits=C, beta=0.5, bias_bits=bias, act=2)
+        got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
+        assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap + 2.0, k, bf16=bf16)
+    finally:
+        ko.set_tuning("gemm16.k_slices", 0)
+
+
 @pytest.mark.parametrize("variant", [0, 9, 30, 50])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_gemm16_bias_gelu_big(ko, variant, bf16):
