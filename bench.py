@@ -676,6 +676,10 @@ def main():
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16384, 3072, 760))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
+        # a 16-bit weight-gradient shape: 36 tiles of 128 x 128 in seven slices of K
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(768, 768, 16384))
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         res = bench_gemm16_bias_gelu(args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor)
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
