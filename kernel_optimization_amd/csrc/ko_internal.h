@@ -71,8 +71,8 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
 // allocated at the first request for that (device, stream) pair and kept until the process ends, so calls on
 // different streams never share it and calls on one stream use it in stream order.  `*workspace` stays null,
 // with KO_OK, where nothing may be allocated (the stream is being captured into a graph and has no workspace
-// yet, 64 pairs already hold one, or the stream is hipStreamPerThread): the caller then takes its path without a
-// workspace.
+// yet, 64 pairs already hold one, the stream is hipStreamPerThread, or the allocation fails): the caller then
+// takes its path without a workspace.
 constexpr size_t kStreamWorkspaceBytes = size_t{32} << 20;
 int stream_workspace(hipStream_t stream, void **workspace);
 

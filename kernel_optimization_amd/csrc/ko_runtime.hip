@@ -92,7 +92,12 @@ int stream_workspace(hipStream_t stream, void **workspace) {
     }
     if (capture != hipStreamCaptureStatusNone) return KO_OK;
     void *memory = nullptr;
-    KO_HIP(hipMalloc(&memory, kStreamWorkspaceBytes));
+    // no memory, or an allocation is not allowed right now (another stream of the process is being captured):
+    // the caller goes without a workspace this time
+    if (hipMalloc(&memory, kStreamWorkspaceBytes) != hipSuccess || memory == nullptr) {
+        (void)hipGetLastError();
+        return KO_OK;
+    }
     entries[used++] = Entry{dev, stream, memory};
     *workspace = memory;
     return KO_OK;
