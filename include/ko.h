@@ -249,6 +249,12 @@ int ko_get_tuning(const char *name, int *value);
  * in[lane]; out[lane] receives the all-reduce over its group of `group` lanes
  * (group in {2,4,8,16,32,64}; op 0 = max, 1 = sum). */
 int ko_debug_wave_allreduce(const float *in, float *out, int group, int op, ko_stream_t stream);
+/* What the GEMMs' host-side planners decide for a shape (16-byte aligned operands, 256 compute units when no
+ * device is visible): the number of K slices (1 = the problem goes out whole), the depth of every slice but the
+ * last, and the tiling of the sliced launch (SGEMM: the kernel variant number, 0 = chosen as for the whole
+ * problem; 16-bit GEMM: 128 or 64, the tile edge).  Touches no device memory and launches nothing. */
+int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
+int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
 
 #ifdef __cplusplus
 }

@@ -81,6 +81,10 @@ SIGNATURES = {
     "ko_set_tuning": (_int, [ctypes.c_char_p, _int]),
     "ko_get_tuning": (_int, [ctypes.c_char_p, ctypes.POINTER(_int)]),
     "ko_debug_wave_allreduce": (_int, [_vp, _vp, _int, _int, _vp]),
+    "ko_debug_sgemm_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                   ctypes.POINTER(ctypes.c_int)]),
+    "ko_debug_gemm16_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                    ctypes.POINTER(ctypes.c_int)]),
 }
 
 _lib = None
@@ -276,6 +280,14 @@ def layernorm16(inp, out, rows, cols, mean=None, rstd=None, gamma=None, beta=Non
 
 def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
     check(lib().ko_sgemm_f32(m, n, k, alpha, _p(A), _p(B), beta, _p(C), _p(D), _h(stream)))
+
+
+def gemm_plan(m, n, k, sixteen_bit=False):
+    """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM decides for a shape."""
+    a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    fn = lib().ko_debug_gemm16_plan if sixteen_bit else lib().ko_debug_sgemm_plan
+    check(fn(m, n, k, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    return a.value, b.value, c.value
 
 
 def sgemm_static_scratch(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):

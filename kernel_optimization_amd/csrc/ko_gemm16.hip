@@ -1495,3 +1495,22 @@ KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, co
     return ko_gemm_f16f32acc_bias_act(m, n, k, alpha, A, B, b_layout, beta, C, nullptr, KO_ACT_NONE, D, in_dtype,
                                       stream);
 }
+
+KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile) {
+    using namespace ko;
+    if (!slices || !k_slice || !tile || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
+        return fail(KO_ERR_INVALID_ARGUMENT, "ko_debug_gemm16_plan: bad argument");
+    Params p{};
+    p.M = static_cast<int>(m);
+    p.N = static_cast<int>(n);
+    p.K = static_cast<int>(k);
+    p.ldd = p.ldb = p.N;
+    p.ldk = p.K;
+    const int64_t big = ((m + 255) / 256) * ((n + 255) / 256);
+    SlicePlan16 plan;
+    if (2 * big < compute_units()) plan = plan_k_slices16(p, kStreamWorkspaceBytes);  // as launch_variant asks
+    *slices = plan.slices;
+    *k_slice = plan.k_slice;
+    *tile = plan.slices > 1 ? (plan.tiles_128 ? 128 : 64) : 0;
+    return KO_OK;
+}

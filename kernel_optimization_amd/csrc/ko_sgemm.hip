@@ -985,3 +985,18 @@ KO_EXPORT int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float
                                           float beta, const float *C, float *D, ko_stream_t stream) {
     return ko::sgemm(m, n, k, alpha, A, B, beta, C, D, stream, true);
 }
+
+KO_EXPORT int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant) {
+    using namespace ko;
+    if (!slices || !k_slice || !variant || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
+        return fail(KO_ERR_INVALID_ARGUMENT, "ko_debug_sgemm_plan: bad argument");
+    // operands that the planner takes for 16-byte aligned; nothing is read through them
+    const float *aligned = reinterpret_cast<const float *>(uintptr_t{256});
+    const Params p{aligned, aligned, nullptr, nullptr, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),
+                   1.0f, 0.0f, 0, 0, static_cast<int>(k), 0};
+    const SlicePlan plan = plan_k_slices(p, kStreamWorkspaceBytes);
+    *slices = plan.slices;
+    *k_slice = plan.k_slice;
+    *variant = plan.variant;
+    return KO_OK;
+}

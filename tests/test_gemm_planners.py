@@ -1,0 +1,68 @@
+"""The GEMMs' host-side K-slice planners, asked without a GPU.
+
+A plan is arithmetic on the shape and the number of compute units (256 when no device is visible, which is also what
+gfx950 has), so its invariants can be checked on the CPU: every slice but the last is a whole number of K tiles, the
+slices cover K exactly once, the fp32 partial products fit the 32 MiB workspace, and shapes that fill the chip whole
+are left whole.
+"""
+import itertools
+
+import pytest
+
+import kernel_optimization_amd as ko
+
+WORKSPACE = 32 << 20
+SIZES = [64, 100, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
+DEPTHS = [64, 512, 767, 768, 1300, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
+
+
+def _check(m, n, k, plan, k_tile, min_k):
+    slices, k_slice, _ = plan
+    assert slices >= 1
+    if slices == 1:
+        return
+    assert k >= min_k, (m, n, k, plan)
+    assert k_slice > 0 and k_slice % k_tile == 0, (m, n, k, plan)
+    assert (slices - 1) * k_slice < k <= slices * k_slice, (m, n, k, plan)   # no empty slice, none missing
+    assert slices * m * n * 4 <= WORKSPACE, (m, n, k, plan)
+
+
+@pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
+def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
+    for k in DEPTHS:
+        plan = ko.gemm_plan(m, n, k)
+        _check(m, n, k, plan, k_tile=128, min_k=768)
+        if plan[0] > 1 and plan[2]:
+            assert plan[2] in (33, 35, 36, 40), plan       # the direct-to-LDS tilings
+
+
+@pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
+def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
+    for k in DEPTHS:
+        plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
+        _check(m, n, k, plan, k_tile=64, min_k=2048)
+        if n % 8:
+            assert plan[0] == 1, (m, n, k, plan)           # partial products are written four columns at a time
+        assert plan[2] in ((128, 64) if plan[0] > 1 else (0,))
+
+
+def test_measured_decisions_stay_put():
+    """Shapes whose plans were chosen from timings: a change of the planner that moves them should be deliberate."""
+    assert ko.gemm_plan(256, 256, 2048)[:2] == (8, 256)
+    assert ko.gemm_plan(768, 768, 16384)[0] == 7
+    assert ko.gemm_plan(1024, 1024, 8192)[0] == 1
+    assert ko.gemm_plan(4096, 4096, 4096)[0] == 1
+    assert ko.gemm_plan(256, 256, 512)[0] == 1
+    assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (7, 2368, 128)
+    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (4, 2048, 64)
+    assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
+    assert ko.gemm_plan(16384, 3072, 768, sixteen_bit=True)[0] == 1
+
+
+def test_bad_arguments_are_refused():
+    with pytest.raises(ko.KoError):
+        ko.gemm_plan(0, 16, 16)
+    with pytest.raises(ko.KoError):
+        ko.gemm_plan(16, 16, -1, sixteen_bit=True)
+    with pytest.raises(ko.KoError):
+        ko.gemm_plan(1 << 31, 16, 16)
