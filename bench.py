@@ -17,6 +17,7 @@ import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -589,7 +590,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches before the timed ones; the device takes a few hundred short launches "
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
-    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"], choices=sorted(WORKLOADS) + ["copy_f32", "hbm_ceilings", "softmax_f32_786432x512_unmasked"])
+    ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"],
+                    help="one of %s, copy_f32, hbm_ceilings, softmax_f32_786432x512_unmasked, or a long-row line by name: "
+                         "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache)" % ", ".join(sorted(WORKLOADS)))
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
     ap.add_argument("--no-all", dest="all", action="store_false")
@@ -612,6 +615,15 @@ def main():
         res, _ = bench_softmax(5, args.steps, args.warmup, unmasked=True)
         print(json.dumps(res))
         return
+    row_line = re.fullmatch(r"(softmax|layernorm)_f32_(\d+)x(\d+)_(auto|warp|block|nocache)", args.workload)
+    if row_line and args.workload not in WORKLOADS:  # one of the long-row lines alone, for counters and traces
+        policy = {"auto": ko.POLICY_AUTO, "warp": ko.POLICY_WARP, "block": ko.POLICY_BLOCK,
+                  "nocache": ko.POLICY_BLOCK_NOCACHE}[row_line.group(4)]
+        print(json.dumps(bench_long_rows(row_line.group(1), int(row_line.group(2)), int(row_line.group(3)), policy,
+                                         args.steps, args.warmup)))
+        return
+    if args.workload not in WORKLOADS:
+        sys.exit("bench.py: unknown workload %r (see --help)" % args.workload)
     cfg = WORKLOADS[args.workload]
     head, keep = run_workload(cfg, args.steps, args.warmup, vendor)
     cpu, parity = (None, None)
