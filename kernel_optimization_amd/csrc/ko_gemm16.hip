@@ -42,6 +42,11 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// The same vectors where only the element's own alignment is known: rows of C and D start on 2-byte boundaries when
+// the row stride is not a multiple of 8.  Global memory takes 8- and 16-byte accesses at any element boundary (the
+// compiler emits the same one instruction for them), so such rows keep the coalesced epilogue.
+typedef u32x4 u32x4_rows __attribute__((aligned(2)));
+typedef u32x2 u32x2_rows __attribute__((aligned(2)));
 
 constexpr int kBK = 64;          // K extent of a stage
 constexpr int kChunks = kBK / 8; // 16-byte chunks per LDS row
@@ -244,7 +249,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) c_q[j][q] = *reinterpret_cast<const u32x2 *>(crow + j * 32 + 8 * q);
+                        for (int q = 0; q < 4; ++q) c_q[j][q] = *reinterpret_cast<const u32x2_rows *>(crow + j * 32 + 8 * q);
                 }
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
@@ -278,13 +283,12 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int gn = col0 + c * 8;
                 // streaming store: D is written once and not read again by this kernel (`sc1 nt`, which helps the
                 // row kernels, measured no different here: 74.3 against 73.8 us)
-                __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p.D + gm * ldd + gn));
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
             }
         }
         return;
     }
 
-    const bool vec_ok = (N & 3) == 0 && (ldd & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = row0 + i * 32 + frow;
@@ -297,15 +301,15 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 if (EDGE && n >= N) continue;
                 const int64_t off = m * ldd + n;
                 float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                if (!EDGE || vec_ok) {  // n is a multiple of 4 and n + 3 < N
+                if (!EDGE || n + 3 < N) {  // the group's four columns are inside the matrix (n is a multiple of 4)
                     u32x2 c2 = {0, 0}, b2 = {0, 0};
-                    if (use_c) c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
+                    if (use_c) c2 = *reinterpret_cast<const u32x2_rows *>(p.C + off);
                     if (p.bias) b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
                     finish4<BF16>(p, v, c2, b2, use_c);
                     u32x2 o;
                     o[0] = pack2<BF16>(v[0], v[1]);
                     o[1] = pack2<BF16>(v[2], v[3]);
-                    *reinterpret_cast<u32x2 *>(p.D + off) = o;
+                    *reinterpret_cast<u32x2_rows *>(p.D + off) = o;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -1378,7 +1382,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // Columns that do not fill the last column of big tiles: the full tile columns go out on their own -
         // to the pinned kernel when the rest of the shape allows - and the remaining columns (fewer than 256)
         // as a launch of their own; C, D and a row-major B keep their row strides.
-        if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && p.ldd % 8 == 0 && p.ldb % 8 == 0 &&
+        if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && (!B_ROW_MAJOR || (p.ldd % 8 == 0 && p.ldb % 8 == 0)) &&
             p.K >= 2 * kBK && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
             const int n1 = p.N - p.N % 256;
             Params left = p, right = p;

@@ -684,3 +684,36 @@ def test_gemm16_ragged_column_counts_whole_output(ko, m, n, k, b_col_major):
     got = ko.gemm16_host(A.view(np.uint16), Bm.view(np.uint16), m, n, k, C_bits=C.view(np.uint16), alpha=1.0, beta=2.0,
                          b_layout=layout, bias_bits=bias.view(np.uint16)).view(np.float16)
     np.testing.assert_array_equal(got, (exact + 2.0 * C.astype(np.float64) + bias.astype(np.float64)).astype(np.float16))
+
+
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("m,n,k", [(4096, 2202, 256), (4096, 2203, 128), (4136, 2317, 128), (8192, 1290, 384),
+                                   (300, 523, 72), (256, 262, 64), (513, 259, 136)])
+def test_gemm16_rows_of_c_and_d_off_16_byte_boundaries_whole_output(ko, m, n, k, b_col_major, bf16):
+    """Column counts that are not a multiple of 8 (vocabulary sizes: 30522, 50257): rows of C and D then start on 4- or
+    2-byte boundaries.  With a K-contiguous B the full tile columns still run on the pinned kernel and the rest as a
+    launch of its own, the coalesced epilogue writing its 16-byte pieces at element alignment; a row-major B (whose
+    own rows are off 16-byte boundaries then) keeps the register pipeline.  Small integers, so the whole output
+    equals the rounded exact result; D sits in front of a guard area that must come back untouched."""
+    rng = np.random.default_rng(n + k)
+    f16 = lambda x: oracle.f64_to_bf16(x) if bf16 else oracle.f64_to_f16(x)  # one rounding to the storage type
+    A = rng.integers(-4, 5, (m, k)).astype(np.float64)
+    B = rng.integers(-4, 5, (n, k)).astype(np.float64)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float64)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float64)
+    exact = A @ B.T
+    Bm = B if b_col_major else np.ascontiguousarray(B.T)
+    kw = dict(b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR, dtype=ko.BF16 if bf16 else ko.F16)
+    dA, dB = ko.DeviceBuffer.from_numpy(f16(A)), ko.DeviceBuffer.from_numpy(f16(Bm))
+    dC, dbias = ko.DeviceBuffer.from_numpy(f16(C)), ko.DeviceBuffer.from_numpy(f16(bias))
+    guard = 64
+    dD = ko.DeviceBuffer((m * n + guard) * 2)
+    for c, beta, b in ((None, 0.0, None), (dC, 2.0, dbias)):
+        dD.upload(np.full(m * n + guard, 0x7e7e, np.uint16))
+        ko.gemm16(m, n, k, dA, dB, dD, c, 1.0, beta, bias=b, **kw)
+        ko.synchronize()
+        out = dD.download(np.uint16, (m * n + guard,))
+        want = exact if c is None else exact + 2.0 * C + bias
+        np.testing.assert_array_equal(out[:m * n].reshape(m, n), f16(want))
+        assert np.all(out[m * n:] == 0x7e7e)
