@@ -688,6 +688,11 @@ def main():
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(16384, 3072, 760))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
+        # a vocabulary projection: 30522 columns put the rows of D off 16-byte boundaries (full tile columns on the
+        # pinned kernel, the last 58 columns as a launch of their own)
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(4096, 30522, 768))
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         # a 16-bit weight-gradient shape: 36 tiles of 128 x 128 in seven slices of K
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(768, 768, 16384))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
