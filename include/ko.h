@@ -193,7 +193,8 @@ int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, co
  * (in_dtype); products accumulate in fp32 on the matrix cores; D is rounded once
  * to the 16-bit type.  C may be NULL.  k must be a multiple of 8; A, B, C, D 16-byte aligned.
  * m and n are free: an n that is not a multiple of 8 (rows of C and D off 16-byte boundaries) keeps the fast
- * kernels with a column-major B and costs about a tenth; with a row-major B it runs at less than half the rate.
+ * kernels with a column-major B and costs about a tenth; with a row-major B (whose own rows are off 16-byte
+ * boundaries then) it runs at about 0.6 of the rate.
  * Workspace: like ko_sgemm_f32, a deep K (k >= 2048) on few output tiles is cut into slices of K whose fp32
  * partial products go through the 32 MiB workspace of the (device, stream) pair, allocated at the first such
  * call on the stream; a first such call inside a graph capture allocates nothing and runs unsliced. */

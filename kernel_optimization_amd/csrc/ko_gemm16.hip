@@ -498,8 +498,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params whole) 
                 u32x4 v = {0u, 0u, 0u, 0u};
                 if (!EDGE || gk < K) {
                     const uint16_t *src = p.B + static_cast<int64_t>(gk) * p.ldb + gn;
-                    if (!EDGE || (gn + 8 <= N && (p.ldb & 7) == 0)) {
-                        v = *reinterpret_cast<const u32x4 *>(src);
+                    if (!EDGE || gn + 8 <= N) {  // rows of B may start at any element (ldb not a multiple of 8)
+                        v = *reinterpret_cast<const u32x4_rows *>(src);
                     } else {
                         uint16_t t[8];
 #pragma unroll
