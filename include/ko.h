@@ -28,7 +28,7 @@ typedef void *ko_event_t;
 typedef enum ko_status {
     KO_OK = 0,
     KO_ERR_INVALID_ARGUMENT = 1,  /* null pointer, negative size, bad enum */
-    KO_ERR_UNSUPPORTED_SHAPE = 2, /* e.g. cols not a multiple of the vector width */
+    KO_ERR_UNSUPPORTED_SHAPE = 2, /* e.g. a row longer than the chosen policy holds */
     KO_ERR_RUNTIME = 3,           /* a HIP runtime call or a kernel launch failed */
     KO_ERR_OUT_OF_MEMORY = 4,
     KO_ERR_NO_DEVICE = 5
@@ -103,7 +103,9 @@ int ko_event_destroy(ko_event_t event);
  *      softmax<K><<<grid, block, K::smem_in_bytes, stream>>>(T *in, T *out)
  *      (nn_operators/softmax/softmax.h:168-174, launched at softmax/main.cu:58-60).
  * in, out: row-major [rows, cols] fp32, contiguous; in == out is allowed.
- * cols must be a multiple of 4 (the reference's static_assert, softmax.h:21).
+ * Any cols: a multiple of 4 (one 16-byte vector: the reference's vec_len = 4, softmax.h:21) is the fast case;
+ * other row lengths start their rows off 16-byte boundaries and are walked element by element (what the
+ * reference's descriptors do with vec_len = 1 or 2), at 0.6-0.9 of the rate.
  * valid_len: NULL for no mask, else device int32[ceil(rows / rows_per_seq)];
  * row r belongs to sequence r / rows_per_seq and every column
  * j >= valid_len[seq] takes the value -10000 before the softmax. */
@@ -116,8 +118,8 @@ int ko_softmax_f32_policy(const float *in, float *out, int64_t rows, int64_t col
                           ko_stream_t stream);
 
 /* Same operator on 16-bit storage: in, out are binary16 (KO_F16) or bfloat16 (KO_BF16) bit
- * patterns, the arithmetic is fp32, the result is rounded once to the storage type.  cols must be
- * a multiple of 8 (one 16-byte vector).  Stands in for the reference's T = half instantiation
+ * patterns, the arithmetic is fp32, the result is rounded once to the storage type.  cols that are
+ * a multiple of 8 (one 16-byte vector) are the fast case, other lengths as for fp32.  Stands in for the reference's T = half instantiation
  * of the same template (softmax.h:11, with the half functors of common/functors.h:71-77 and
  * limits of common/common.h:171-177).  policy: a ko_policy value. */
 int ko_softmax_16(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *valid_len,
@@ -130,7 +132,7 @@ int ko_softmax_16(const void *in, void *out, int64_t rows, int64_t cols, const i
  * in, out: row-major [rows, cols] fp32 (in == out allowed); gamma, beta: [cols]
  * or NULL (each independently); mean, rstd: [rows] outputs or NULL.
  * var divides by cols (unbiased == 0) or cols - 1 (unbiased != 0, the
- * reference's intent at layernorm.h:48).  cols must be a multiple of 4. */
+ * reference's intent at layernorm.h:48).  Any cols; multiples of 4 are the fast case (see ko_softmax_f32). */
 int ko_layernorm_f32(const float *in, float *out, float *mean, float *rstd, const float *gamma,
                      const float *beta, int64_t rows, int64_t cols, float eps, int unbiased,
                      ko_stream_t stream);
@@ -140,8 +142,8 @@ int ko_layernorm_f32_policy(const float *in, float *out, float *mean, float *rst
                             float eps, int unbiased, int policy, ko_stream_t stream);
 
 /* Same operator on 16-bit storage: in, out, gamma, beta are binary16 or bfloat16 bit patterns
- * (all of the one dtype), mean and rstd stay fp32, the arithmetic is fp32.  cols must be a
- * multiple of 8.  Stands in for Element = half in LayerNormWarpImpl and its siblings
+ * (all of the one dtype), mean and rstd stay fp32, the arithmetic is fp32.  Any cols; multiples
+ * of 8 are the fast case.  Stands in for Element = half in LayerNormWarpImpl and its siblings
  * (layernorm.h:145, with Rsqrt<half> of common/functors.h:105-111). */
 int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const void *gamma,
                     const void *beta, int64_t rows, int64_t cols, float eps, int unbiased, int dtype,

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
                 }
 #pragma unroll
                 for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[e], b[e]);
-                Io<IO>::store_stream(dst0, sub_off + 16u * j, y);
+                Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, y);
             }
         }
         if (row_ok && l == 0) {
@@ -567,7 +567,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] -= x0;
                 normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                Io<IO>::store_stream(dst, 16u * j, y);
+                Io<IO>::store_stream(dst, Io<IO>::kBytes * j, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -916,6 +916,23 @@ int launch_nocache(const Args<IO> &a) {
     return launch_nocache_threads<IO, 1024>(a);
 }
 
+// Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
+// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes) and is read once; longer rows are read twice.
+template <int IO>
+int launch_by_element(const Args<IO> &a) {
+    static_assert(Io<IO>::E == 1, "");
+    const int cols = a.cols;
+    if (cols <= 16) return launch_wave_full<IO, 16, 1, false>(a);
+    if (cols <= 32) return launch_wave_full<IO, 16, 2, false>(a);
+    if (cols <= 64) return launch_wave_full<IO, 16, 4, false>(a);
+    if (cols <= 128) return launch_wave_full<IO, 64, 2, false>(a);
+    if (cols <= 256) return launch_wave_full<IO, 64, 4, false>(a);
+    if (cols <= 512) return launch_wave_full<IO, 64, 8, false>(a);
+    if (cols <= 1024) return launch_wave_full<IO, 64, 16, false>(a);
+    if (cols <= 2048) return launch_wave_full<IO, 64, 32, false>(a);
+    return launch_nocache<IO>(a);
+}
+
 template <int IO>
 int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma, const void *beta, int64_t rows,
           int64_t cols, float eps, int unbiased, int policy, ko_stream_t stream) {
@@ -923,9 +940,6 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
     typedef typename Io<IO>::elem elem;
     if (rows < 0 || cols <= 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: rows=%lld cols=%lld", (long long)rows, (long long)cols);
-    if (cols % E != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld is not a multiple of the vector width %d",
-                    (long long)cols, E);
     if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld too large", (long long)cols);
     if (rows == 0) return KO_OK;
     if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: null in/out pointer");
@@ -934,6 +948,20 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
     if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: in/out/gamma/beta must be 16-byte aligned");
     if (!(eps >= 0.0f)) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: eps must be >= 0");
     const double denom = unbiased ? static_cast<double>(cols - 1) : static_cast<double>(cols);
+    if (cols % E != 0) {
+        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2): every
+        // policy walks such a row element by element (launch_by_element); the WARP policy's row limit stays.
+        constexpr int BY_ELEMENT = io_by_element(IO);
+        if (policy != KO_POLICY_AUTO && policy != KO_POLICY_WARP && policy != KO_POLICY_BLOCK && policy != KO_POLICY_BLOCK_NOCACHE)
+            return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);
+        if (policy == KO_POLICY_WARP && (cols + E - 1) / E > kWaveMaxVecs)
+            return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: WARP policy holds at most %d columns per row, got %lld",
+                        kWaveMaxVecs * E, (long long)cols);
+        Args<BY_ELEMENT> a1{static_cast<const elem *>(in), static_cast<elem *>(out), mean, rstd,
+                            static_cast<const elem *>(gamma), static_cast<const elem *>(beta), rows,
+                            static_cast<int>(cols), eps, static_cast<float>(1.0 / denom), as_stream(stream)};
+        return launch_by_element<BY_ELEMENT>(a1);
+    }
     Args<IO> a{static_cast<const elem *>(in), static_cast<elem *>(out), mean, rstd, static_cast<const elem *>(gamma),
                static_cast<const elem *>(beta), rows, static_cast<int>(cols), eps, static_cast<float>(1.0 / denom),
                as_stream(stream)};

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
             if (row_ok && j < nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
-                if constexpr (NT) Io<IO>::store_stream(dst0, sub_off + 16u * j, v[k]);
+                if constexpr (NT) Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, v[k]);
                 else Io<IO>::template store<false>(dst0 + static_cast<int64_t>(sub) * cols + E * j, v[k]);
             }
         }
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
                 if (j >= nvec) break;
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
-                Io<IO>::store_stream(dst, 16u * j, x[u]);
+                Io<IO>::store_stream(dst, Io<IO>::kBytes * j, x[u]);
             }
         }
     }
@@ -656,6 +656,23 @@ int launch_nocache(const Args<IO> &a) {
     return launch_nocache_threads<IO, 1024, MASKED>(a);
 }
 
+// Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
+// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes) and is read once; longer rows are read twice.
+template <int IO, bool MASKED>
+int launch_by_element(const Args<IO> &a) {
+    static_assert(Io<IO>::E == 1, "");
+    const int cols = a.cols;
+    if (cols <= 16) return launch_wave<IO, 16, 1, MASKED, true>(a);
+    if (cols <= 32) return launch_wave<IO, 16, 2, MASKED, true>(a);
+    if (cols <= 64) return launch_wave<IO, 16, 4, MASKED, true>(a);
+    if (cols <= 128) return launch_wave<IO, 64, 2, MASKED, true>(a);
+    if (cols <= 256) return launch_wave<IO, 64, 4, MASKED, true>(a);
+    if (cols <= 512) return launch_wave<IO, 64, 8, MASKED, true>(a);
+    if (cols <= 1024) return launch_wave<IO, 64, 16, MASKED, true>(a);
+    if (cols <= 2048) return launch_wave<IO, 64, 32, MASKED, true>(a);
+    return launch_nocache<IO, MASKED>(a);
+}
+
 template <int IO, bool MASKED>
 int dispatch(const Args<IO> &a, int policy) {
     constexpr int E = Io<IO>::E;
@@ -690,9 +707,6 @@ int entry(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *
     constexpr int E = Io<IO>::E;
     if (rows < 0 || cols <= 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "softmax: rows=%lld cols=%lld", (long long)rows, (long long)cols);
-    if (cols % E != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld is not a multiple of the vector width %d",
-                    (long long)cols, E);
     if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld too large", (long long)cols);
     if (rows == 0) return KO_OK;
     if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "softmax: null in/out pointer");
@@ -700,6 +714,23 @@ int entry(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *
         return fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be 16-byte aligned");
     if (valid_len && rows_per_seq <= 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "softmax: valid_len given but rows_per_seq=%lld", (long long)rows_per_seq);
+    if (cols % E != 0) {
+        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2): every
+        // policy walks such a row element by element (launch_by_element); the policies' row limits stay.
+        constexpr int BY_ELEMENT = io_by_element(IO);
+        const int64_t nvec = (cols + E - 1) / E;
+        if (policy != KO_POLICY_AUTO && policy != KO_POLICY_WARP && policy != KO_POLICY_BLOCK && policy != KO_POLICY_BLOCK_NOCACHE)
+            return fail(KO_ERR_INVALID_ARGUMENT, "softmax: unknown policy %d", policy);
+        if (policy == KO_POLICY_WARP && nvec > kWaveMaxVecs)
+            return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: WARP policy holds at most %d columns per row, got %lld",
+                        kWaveMaxVecs * E, (long long)cols);
+        if (policy == KO_POLICY_BLOCK && nvec > (valid_len ? 1024 * (96 / E) : kBlockMaxVecs<IO>))
+            return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: BLOCK policy holds at most %d columns per row%s, got %lld",
+                        (valid_len ? 1024 * (96 / E) : kBlockMaxVecs<IO>) * E, valid_len ? " with a mask" : "", (long long)cols);
+        Args<BY_ELEMENT> a{static_cast<const typename Io<IO>::elem *>(in), static_cast<typename Io<IO>::elem *>(out), rows,
+                           static_cast<int>(cols), valid_len, rows_per_seq, as_stream(stream)};
+        return valid_len ? launch_by_element<BY_ELEMENT, true>(a) : launch_by_element<BY_ELEMENT, false>(a);
+    }
     Args<IO> a{static_cast<const typename Io<IO>::elem *>(in), static_cast<typename Io<IO>::elem *>(out), rows,
                static_cast<int>(cols), valid_len, rows_per_seq, as_stream(stream)};
     return valid_len ? dispatch<IO, true>(a, policy) : dispatch<IO, false>(a, policy);

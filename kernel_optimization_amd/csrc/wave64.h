@@ -250,7 +250,13 @@ __device__ __forceinline__ void store4(float *p, float4v v) {
 // E = 4 floats or E = 8 binary16 / bfloat16 values, converted on load and rounded (to nearest
 // even) once on store.  The reference carries half specialisations of its functors for the same
 // purpose (common/functors.h:71-77,105-111, common/common.h:171-177).
-enum { IO_F32 = 0, IO_F16 = 1, IO_BF16 = 2 };
+// The *_1 kinds move one element per access (E = 1): rows whose length is not a multiple of the 16-byte vector
+// start at element alignment, and the kernels that walk a row vector by vector (the re-reading ones) walk it
+// element by element instead - what the reference's descriptors do with vec_len = 1.
+enum { IO_F32 = 0, IO_F16 = 1, IO_BF16 = 2, IO_F32_1 = 3, IO_F16_1 = 4, IO_BF16_1 = 5 };
+// the one-element kind of a storage type, and the storage type of any kind
+constexpr int io_by_element(int io) { return io % 3 + 3; }
+constexpr int io_storage(int io) { return io % 3; }
 
 template <int IO>
 struct Io;
@@ -260,6 +266,7 @@ struct Io<IO_F32> {
     typedef float elem;
     static constexpr int E = 4;
     typedef float4v raw;  // one 16-byte vector as loaded, before conversion
+    static constexpr uint32_t kBytes = sizeof(raw);  // between consecutive vectors of a row
     template <bool NT>
     static __device__ __forceinline__ raw load_raw(const elem *p) {
         return load4<NT>(p);
@@ -303,6 +310,7 @@ struct Io<IO_F16> {
     static constexpr int E = 8;
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
     typedef uint4v raw;
+    static constexpr uint32_t kBytes = sizeof(raw);
     template <bool NT>
     static __device__ __forceinline__ raw load_raw(const elem *p) {
         return load_bits16<NT>(p);
@@ -339,6 +347,7 @@ struct Io<IO_BF16> {
     typedef uint16_t elem;
     static constexpr int E = 8;
     typedef uint4v raw;
+    static constexpr uint32_t kBytes = sizeof(raw);
     template <bool NT>
     static __device__ __forceinline__ raw load_raw(const elem *p) {
         return load_bits16<NT>(p);
@@ -378,6 +387,59 @@ struct Io<IO_BF16> {
         return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
     }
 };
+
+// One element per access.  CONVERT supplies the storage type's conversions (float <-> bits).
+template <class Elem, class Convert>
+struct IoByElement {
+    typedef Elem elem;
+    static constexpr int E = 1;
+    typedef Elem raw;
+    static constexpr uint32_t kBytes = sizeof(raw);
+    template <bool NT>
+    static __device__ __forceinline__ raw load_raw(const elem *p) {
+        if constexpr (NT) return __builtin_nontemporal_load(p);
+        return *p;
+    }
+    static __device__ __forceinline__ void unpack(raw x, float (&v)[E]) { v[0] = Convert::to_float(x); }
+    template <bool NT>
+    static __device__ __forceinline__ void load(const elem *p, float (&v)[E]) {
+        unpack(load_raw<NT>(p), v);
+    }
+    template <bool NT>
+    static __device__ __forceinline__ void store(elem *p, const float (&v)[E]) {
+        if constexpr (NT) __builtin_nontemporal_store(Convert::from_float(v[0]), p);
+        else *p = Convert::from_float(v[0]);
+    }
+    static __device__ __forceinline__ void store_stream(elem *base, uint32_t byte_offset, const float (&v)[E]) {
+        __builtin_nontemporal_store(Convert::from_float(v[0]),
+                                    reinterpret_cast<elem *>(reinterpret_cast<char *>(base) + byte_offset));
+    }
+    static __device__ __forceinline__ float scalar(const elem *p) { return Convert::to_float(*p); }
+};
+struct ConvertF32 {
+    static __device__ __forceinline__ float to_float(float x) { return x; }
+    static __device__ __forceinline__ float from_float(float x) { return x; }
+};
+struct ConvertF16 {
+    static __device__ __forceinline__ float to_float(uint16_t x) { return static_cast<float>(__builtin_bit_cast(_Float16, x)); }
+    static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even
+        return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+    }
+};
+struct ConvertBF16 {
+    static __device__ __forceinline__ float to_float(uint16_t x) { return __builtin_bit_cast(float, static_cast<uint32_t>(x) << 16); }
+    static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even, as the vector kind does
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        return static_cast<uint16_t>(__builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{x, 0.0f}, bf16x2)));
+    }
+};
+template <>
+struct Io<IO_F32_1> : IoByElement<float, ConvertF32> {};
+template <>
+struct Io<IO_F16_1> : IoByElement<uint16_t, ConvertF16> {};
+template <>
+struct Io<IO_BF16_1> : IoByElement<uint16_t, ConvertBF16> {};
 
 // exp(d) for d <= 0, within 2 ulp: 2^y (1 + r ln 2), where y = d * log2(e) is the rounded product, r its exact
 // residual plus d times the low part of log2(e) (|r| <= 2^-24 |y|, so the first-order term is all that matters),
@@ -420,8 +482,8 @@ __device__ __forceinline__ float exp_nonpositive_f16(float d) {
 
 template <int IO>
 __device__ __forceinline__ float exp_for_storage(float d) {
-    if constexpr (IO == IO_F32) return exp_nonpositive(d);
-    else if constexpr (IO == IO_F16) return exp_nonpositive_f16(d);
+    if constexpr (io_storage(IO) == IO_F32) return exp_nonpositive(d);
+    else if constexpr (io_storage(IO) == IO_F16) return exp_nonpositive_f16(d);
     else return exp_nonpositive_fast(d);
 }
 

@@ -123,6 +123,30 @@ static int gpu_part() {
         for (int i = 0; i < R * C; ++i) REQUIRE(float(outb.host_ref<ko_bfloat16>()[i]) == 1.0f / C);
     }
     {
+        // vec_len = 1: the reference's descriptors take any row length that way (softmax.h:72, layernorm.h:215);
+        // 197 columns put every row but the first off a 16-byte boundary
+        constexpr int R = 6, C = 197;
+        Tensor in(R * C * 4), out(R * C * 4), mean(R * 4), rstd(R * 4);
+        for (int i = 0; i < R * C; ++i) in.host_ref<float>()[i] = (i % C == i / C) ? 3.0f : 3.0f - 100.0f;
+        in.host_to_device();
+        softmax<SoftMaxBlockImpl<float, 1, R, C>>(R, 128, SoftMaxBlockImpl<float, 1, R, C>::smem_in_bytes, stream,
+                                                  in.device_ref<float>(), out.device_ref<float>());
+        checkKoErrors(ko_stream_synchronize(stream));
+        out.device_to_host();
+        for (int i = 0; i < R * C; ++i)  // exp(-100) is below half an ulp of 1: the row's own column gets all of it
+            REQUIRE(std::fabs(out.host_ref<float>()[i] - ((i % C == i / C) ? 1.0f : 3.72e-44f)) < 1e-6f);
+        for (int i = 0; i < R * C; ++i) in.host_ref<float>()[i] = float(i % C);
+        in.host_to_device();
+        layer_normalization<LayerNormBlockImpl<float, 1, R, C, false>>(R, 128, 0, stream, in.device_ref<float>(),
+                                                                        out.device_ref<float>(), 0.0f, nullptr, nullptr,
+                                                                        mean.device_ref<float>(), rstd.device_ref<float>());
+        checkKoErrors(ko_stream_synchronize(stream));
+        mean.device_to_host();
+        rstd.device_to_host();
+        REQUIRE(std::fabs(mean.host_ref<float>()[5] - 98.0f) < 1e-3f);
+        REQUIRE(std::fabs(rstd.host_ref<float>()[4] - 1.0 / std::sqrt((197.0 * 197.0 - 1) / 12)) < 1e-7);
+    }
+    {
         constexpr int N = 128;
         Tensor A(N * N * 4), B(N * N * 4), C(N * N * 4), D(N * N * 4);
         for (int i = 0; i < N * N; ++i) {

@@ -45,10 +45,12 @@ def test_status_names_and_argument_errors_without_device():
     assert ko.status_name(0) == "KO_OK" and ko.status_name(2) == "KO_ERR_UNSUPPORTED_SHAPE"
     lib = ko.lib()
     # argument validation happens before anything touches the device
-    assert lib.ko_softmax_f32(None, None, 4, 130, None, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
-    assert "multiple of the vector width" in ko.last_error()
+    assert lib.ko_softmax_f32(None, None, 4, (1 << 30) + 4, None, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert "too large" in ko.last_error()
+    assert lib.ko_softmax_f32(None, None, 4, 130, None, 0, None) == ko.KO_ERR_INVALID_ARGUMENT  # any row length; null pointers
     assert lib.ko_softmax_f32(None, None, -1, 128, None, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
-    assert lib.ko_layernorm_f32(None, None, None, None, None, None, 4, 770, 1e-5, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert lib.ko_layernorm_f32(None, None, None, None, None, None, 4, (1 << 30) + 4, 1e-5, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert lib.ko_layernorm_f32(None, None, None, None, None, None, 4, 770, 1e-5, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert lib.ko_sgemm_f32(-1, 1, 1, 1.0, None, None, 0.0, None, None, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert lib.ko_gemm_f16f32acc(8, 8, 12, 1.0, 1, 1, 1, 0.0, None, 1, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert lib.ko_set_tuning(b"no.such.knob", 1) == ko.KO_ERR_INVALID_ARGUMENT

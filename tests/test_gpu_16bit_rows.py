@@ -79,7 +79,8 @@ def test_softmax16_in_place_and_errors(ko, bf16):
     _, ref64 = oracle.softmax16(xb, bf16=bf16)
     assert_softmax16_close(_to64(ko.softmax16_host(xb, dtype=dt, in_place=True), bf16), ref64, bf16)
     d = ko.DeviceBuffer(4096)
-    assert ko.lib().ko_softmax_16(d.ptr, d.ptr, 2, 12, None, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert ko.lib().ko_softmax_16(d.ptr, d.ptr, 2, 12, None, 0, dt, 0, None) == ko.KO_OK  # any row length
+    assert ko.lib().ko_softmax_16(d.ptr, d.ptr, 2, (1 << 30) + 8, None, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert ko.lib().ko_softmax_16(d.ptr, d.ptr, 2, 16, None, 0, 7, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert ko.lib().ko_softmax_16(d.ptr, d.ptr, 2, 8192, None, 0, dt, 1, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert ko.lib().ko_softmax_16(None, d.ptr, 2, 16, None, 0, dt, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
@@ -143,7 +144,8 @@ def test_layernorm16_plain_in_place_and_errors(ko, bf16):
     assert_layernorm16_close((_to64(y, bf16), mean, rstd), (ref64, rmean, rrstd), bf16)
     d = ko.DeviceBuffer(4096)
     L = ko.lib()
-    assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 12, 1e-5, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
+    assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 12, 1e-5, 0, dt, 0, None) == ko.KO_OK  # any row length
+    assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, (1 << 30) + 8, 1e-5, 0, dt, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 2, 16, 1e-5, 0, 9, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert L.ko_layernorm_16(d.ptr, d.ptr, None, None, None, None, 0, 16, 1e-5, 0, dt, 0, None) == ko.KO_OK
 

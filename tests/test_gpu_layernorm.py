@@ -112,7 +112,7 @@ def test_layernorm_properties(ko):
 def test_layernorm_errors(ko):
     buf = ko.DeviceBuffer(1 << 16)
     with pytest.raises(ko.KoError) as e:
-        ko.layernorm(buf, buf, 4, 770)
+        ko.layernorm(buf, buf, 4, (1 << 30) + 4)
     assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
     with pytest.raises(ko.KoError) as e:
         ko.layernorm(buf, None, 4, 768)
