@@ -350,8 +350,9 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
     // Byte offset of this thread's first vector in a row (vector k lies k * THREADS * 16 bytes further).  The
     // row loop passes it through an empty asm: addresses are then formed per use from a uniform base and this
     // one register, instead of 2 * VPL pointers to gamma and beta being kept across rows (which spilled).
-    uint32_t first = threadIdx.x * 16u;
-    constexpr uint32_t kStep = THREADS * 16u;
+    uint32_t first = threadIdx.x * Io<IO>::kBytes;
+    constexpr uint32_t kStep = THREADS * Io<IO>::kBytes;
+    static_assert(LV == 0 || Io<IO>::kBytes == 16, "the LDS tail is filled 16 bytes per lane");
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
 #pragma unroll
                     for (int e = 0; e < E; ++e) x[u][e] -= x0;
                     normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                    Io<IO>::store_stream(dst, 16u * j, y);
+                    Io<IO>::store_stream(dst, Io<IO>::kBytes * j, y);
                 }
             }
         }
@@ -916,8 +917,21 @@ int launch_nocache(const Args<IO> &a) {
     return launch_nocache_threads<IO, 1024>(a);
 }
 
+// A row in the registers of one 1024-thread workgroup, element by element: 1024 * VPL columns, and with REST what
+// lies beyond them streamed (read twice).
+template <int IO, int VPL, bool REST>
+int launch_block_by_element(const Args<IO> &a) {
+    int64_t grid = static_cast<int64_t>(compute_units()) * 4;  // two workgroups per resident slot walk the rows
+    if (grid > a.rows) grid = a.rows;
+    layernorm_block_kernel<IO, 1024, VPL, 0, REST><<<dim3(static_cast<unsigned>(grid)), dim3(1024), 0, a.stream>>>(
+        a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 // Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
-// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes) and is read once; longer rows are read twice.
+// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes), up to 65536 in those of a workgroup, and is read
+// once; of longer rows the far end is read twice.
 template <int IO>
 int launch_by_element(const Args<IO> &a) {
     static_assert(Io<IO>::E == 1, "");
@@ -930,7 +944,11 @@ int launch_by_element(const Args<IO> &a) {
     if (cols <= 512) return launch_wave_full<IO, 64, 8, false>(a);
     if (cols <= 1024) return launch_wave_full<IO, 64, 16, false>(a);
     if (cols <= 2048) return launch_wave_full<IO, 64, 32, false>(a);
-    return launch_nocache<IO>(a);
+    if (cols <= 4096) return launch_block_by_element<IO, 4, false>(a);
+    if (cols <= 8192) return launch_block_by_element<IO, 8, false>(a);
+    if (cols <= 16384) return launch_block_by_element<IO, 16, false>(a);
+    if (cols <= 32768) return launch_block_by_element<IO, 32, false>(a);
+    return launch_block_by_element<IO, 64, true>(a);  // (without REST this one spills; with it, it does not)
 }
 
 template <int IO>

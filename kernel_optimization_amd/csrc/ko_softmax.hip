@@ -239,8 +239,9 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
     // Byte offset of this thread's first vector in a row (vector k lies k * THREADS * 16 bytes further); passed
     // through an empty asm per row so that addresses are formed per use from the uniform row pointer and this
     // one register rather than kept as VPL pointer pairs.
-    uint32_t first = threadIdx.x * 16u;
-    constexpr uint32_t kStep = THREADS * 16u;
+    uint32_t first = threadIdx.x * Io<IO>::kBytes;
+    constexpr uint32_t kStep = THREADS * Io<IO>::kBytes;
+    static_assert(LV == 0 || Io<IO>::kBytes == 16, "the LDS tail is filled 16 bytes per lane");
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
@@ -656,8 +657,20 @@ int launch_nocache(const Args<IO> &a) {
     return launch_nocache_threads<IO, 1024, MASKED>(a);
 }
 
+// A row of up to 1024 * VPL columns in the registers of one 1024-thread workgroup, element by element.
+template <int IO, int VPL, bool MASKED>
+int launch_block_by_element(const Args<IO> &a) {
+    int64_t grid = static_cast<int64_t>(compute_units()) * 4;  // two workgroups per resident slot walk the rows
+    if (grid > a.rows) grid = a.rows;
+    softmax_block_kernel<IO, 1024, VPL, MASKED><<<dim3(static_cast<unsigned>(grid)), dim3(1024), 0, a.stream>>>(
+        a.in, a.out, a.rows, a.cols, a.valid_len, a.rows_per_seq);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 // Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
-// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes) and is read once; longer rows are read twice.
+// 16 or 64 lanes (column j in lane j % lanes, slot j / lanes), up to 65536 in those of a workgroup, and is read
+// once; longer rows are read twice.
 template <int IO, bool MASKED>
 int launch_by_element(const Args<IO> &a) {
     static_assert(Io<IO>::E == 1, "");
@@ -670,6 +683,11 @@ int launch_by_element(const Args<IO> &a) {
     if (cols <= 512) return launch_wave<IO, 64, 8, MASKED, true>(a);
     if (cols <= 1024) return launch_wave<IO, 64, 16, MASKED, true>(a);
     if (cols <= 2048) return launch_wave<IO, 64, 32, MASKED, true>(a);
+    if (cols <= 4096) return launch_block_by_element<IO, 4, MASKED>(a);
+    if (cols <= 8192) return launch_block_by_element<IO, 8, MASKED>(a);
+    if (cols <= 16384) return launch_block_by_element<IO, 16, MASKED>(a);
+    if (cols <= 32768) return launch_block_by_element<IO, 32, MASKED>(a);
+    if (cols <= 65536) return launch_block_by_element<IO, 64, MASKED>(a);
     return launch_nocache<IO, MASKED>(a);
 }
 
