@@ -208,8 +208,11 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
 
         // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
+        // (written through at once only when rows are whole 64-byte lines: a row that ends inside a line would
+        // send that line out twice, half-filled each time)
         typename Io<IO>::elem *dst0 = out + (row - sub) * cols;
         const uint32_t sub_off = static_cast<uint32_t>(sub) * static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem);
+        const bool whole_lines = (static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem)) % 64 == 0;
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
@@ -234,7 +237,8 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
                 }
 #pragma unroll
                 for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[e], b[e]);
-                Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, y);
+                if (whole_lines) Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, y);
+                else Io<IO>::template store<true>(dst0 + static_cast<int64_t>(sub) * cols + E * j, y);
             }
         }
         if (row_ok && l == 0) {
