@@ -208,11 +208,10 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
 
         // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
-        // (written through at once only when rows are whole 64-byte lines: a row that ends inside a line would
-        // send that line out twice, half-filled each time)
+        // (written through at once only when rows are whole 64-byte lines: see store_row_vec)
         typename Io<IO>::elem *dst0 = out + (row - sub) * cols;
         const uint32_t sub_off = static_cast<uint32_t>(sub) * static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem);
-        const bool whole_lines = (static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem)) % 64 == 0;
+        const bool whole_lines = rows_are_whole_lines<IO>(cols);
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
@@ -237,8 +236,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
                 }
 #pragma unroll
                 for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[k][e] - mean) * rstd, g[e], b[e]);
-                if (whole_lines) Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, y);
-                else Io<IO>::template store<true>(dst0 + static_cast<int64_t>(sub) * cols + E * j, y);
+                store_row_vec<IO>(whole_lines, dst0, sub_off + Io<IO>::kBytes * j, y);
             }
         }
         if (row_ok && l == 0) {
@@ -357,6 +355,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
     uint32_t first = threadIdx.x * Io<IO>::kBytes;
     constexpr uint32_t kStep = THREADS * Io<IO>::kBytes;
     static_assert(LV == 0 || Io<IO>::kBytes == 16, "the LDS tail is filled 16 bytes per lane");
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
@@ -454,7 +453,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
 #pragma unroll
                     for (int e = 0; e < E; ++e) x[u][e] -= x0;
                     normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                    Io<IO>::store_stream(dst, Io<IO>::kBytes * j, y);
+                    store_row_vec<IO>(whole_lines, dst, Io<IO>::kBytes * j, y);
                 }
             }
         }
@@ -467,7 +466,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[e] -= x0;
                 normalize_vec<IO>(x, mean, rstd, gamma, beta, E * j, y);
-                Io<IO>::store_stream(dst, first + (VPL + k) * kStep, y);
+                store_row_vec<IO>(whole_lines, dst, first + (VPL + k) * kStep, y);
             }
         }
 #pragma unroll
@@ -490,7 +489,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
                         y[e] = t;
                     }
                 }
-                Io<IO>::store_stream(dst, first + k * kStep, y);
+                store_row_vec<IO>(whole_lines, dst, first + k * kStep, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -513,6 +512,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
     constexpr int E = Io<IO>::E;
     __shared__ float lds[48];
     const int nvec = cols / E;
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const typename Io<IO>::elem *src = in + row * cols;
         const float x0 = Io<IO>::scalar(src);
@@ -572,7 +572,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] -= x0;
                 normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
-                Io<IO>::store_stream(dst, Io<IO>::kBytes * j, y);
+                store_row_vec<IO>(whole_lines, dst, Io<IO>::kBytes * j, y);
             }
         }
         if (threadIdx.x == 0) {
@@ -606,6 +606,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_batch_kernel(const ty
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
     const uint32_t first = threadIdx.x * 16u;
     constexpr uint32_t kStep = THREADS * 16u;
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
 
     Raw loaded[R][VPL];  // all loads first, conversions afterwards
 #pragma unroll
@@ -686,7 +687,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_batch_kernel(const ty
                 float y[E];
 #pragma unroll
                 for (int e = 0; e < E; ++e) y[e] = __builtin_fmaf((v[r][k][e] - mean) * rstd, g[k][e], b[k][e]);
-                Io<IO>::store_stream(dst, first + k * kStep, y);
+                store_row_vec<IO>(whole_lines, dst, first + k * kStep, y);
             }
         }
         if (threadIdx.x == 0) {

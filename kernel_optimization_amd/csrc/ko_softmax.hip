@@ -165,13 +165,11 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
         s = wave::allreduce<LPR, wave::Sum>(s);
         const float inv = 1.0f / s;
 
-        // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset.  Written
-        // through at once (see stream_store16) only when rows are whole 64-byte lines: a row that ends inside a
-        // line would send that line out twice, half-filled each time, and the memory side has to merge them
-        // ([49152, 1000]: 75.5 us written through, 67.7 us left to the L2 to put together).
+        // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset; written through
+        // at once only when rows are whole 64-byte lines (see store_row_vec)
         typename Io<IO>::elem *dst0 = out + row0 * cols;
         const uint32_t sub_off = static_cast<uint32_t>(sub) * static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem);
-        const bool whole_lines = (static_cast<uint32_t>(cols) * sizeof(typename Io<IO>::elem)) % 64 == 0;
+        const bool whole_lines = rows_are_whole_lines<IO>(cols);
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
@@ -179,8 +177,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const typename Io<IO>
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
                 if constexpr (NT) {
-                    if (whole_lines) Io<IO>::store_stream(dst0, sub_off + Io<IO>::kBytes * j, v[k]);
-                    else Io<IO>::template store<true>(dst0 + static_cast<int64_t>(sub) * cols + E * j, v[k]);
+                    store_row_vec<IO>(whole_lines, dst0, sub_off + Io<IO>::kBytes * j, v[k]);
                 } else {
                     Io<IO>::template store<false>(dst0 + static_cast<int64_t>(sub) * cols + E * j, v[k]);
                 }
@@ -250,6 +247,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
     uint32_t first = threadIdx.x * Io<IO>::kBytes;
     constexpr uint32_t kStep = THREADS * Io<IO>::kBytes;
     static_assert(LV == 0 || Io<IO>::kBytes == 16, "the LDS tail is filled 16 bytes per lane");
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         asm volatile("" : "+v"(first));
         const typename Io<IO>::elem *src = in + row * cols;
@@ -351,7 +349,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
             if (j < nvec) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] *= inv;
-                Io<IO>::store_stream(dst, first + k * kStep, v[k]);
+                store_row_vec<IO>(whole_lines, dst, first + k * kStep, v[k]);
             }
         }
 #pragma unroll
@@ -364,7 +362,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_kernel(const typename I
                     if constexpr (IO != IO_F32) x[e] = exp_for_storage<IO>(x[e] - m);
                     x[e] *= inv;
                 }
-                Io<IO>::store_stream(dst, first + (VPL + k) * kStep, x);
+                store_row_vec<IO>(whole_lines, dst, first + (VPL + k) * kStep, x);
             }
         }
     }
@@ -390,6 +388,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
     constexpr int E = Io<IO>::E;
     __shared__ float lds[16];
     const int nvec = cols / E;
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const typename Io<IO>::elem *src = in + row * cols;
         int vlen = cols;
@@ -443,7 +442,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
                 if (j >= nvec) break;
 #pragma unroll
                 for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
-                Io<IO>::store_stream(dst, Io<IO>::kBytes * j, x[u]);
+                store_row_vec<IO>(whole_lines, dst, Io<IO>::kBytes * j, x[u]);
             }
         }
     }
