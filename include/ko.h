@@ -102,7 +102,8 @@ int ko_event_destroy(ko_event_t event);
 /* ---- row softmax: replaces
  *      softmax<K><<<grid, block, K::smem_in_bytes, stream>>>(T *in, T *out)
  *      (nn_operators/softmax/softmax.h:168-174, launched at softmax/main.cu:58-60).
- * in, out: row-major [rows, cols] fp32, contiguous; in == out is allowed.
+ * in, out: row-major [rows, cols] fp32, contiguous; in == out is allowed.  Tensors that start on 16-byte
+ * boundaries are the fast case; any 4-byte aligned address is accepted (walked element by element, see cols).
  * Any cols: a multiple of 4 (one 16-byte vector: the reference's vec_len = 4, softmax.h:21) is the fast case;
  * other row lengths start their rows off 16-byte boundaries and are walked element by element (what the
  * reference's descriptors do with vec_len = 1 or 2), at 0.6-0.9 of the rate.

@@ -982,14 +982,18 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
     if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: cols=%lld too large", (long long)cols);
     if (rows == 0) return KO_OK;
     if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: null in/out pointer");
-    uintptr_t align = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
-                      reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta);
-    if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: in/out/gamma/beta must be 16-byte aligned");
+    const uintptr_t addresses = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
+                                reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta);
+    if (addresses & (sizeof(elem) - 1))
+        return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: in/out/gamma/beta must be aligned to their element type");
+    if ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 3)
+        return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: mean/rstd must be 4-byte aligned");
     if (!(eps >= 0.0f)) return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: eps must be >= 0");
     const double denom = unbiased ? static_cast<double>(cols - 1) : static_cast<double>(cols);
-    if (cols % E != 0) {
-        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2): every
-        // policy walks such a row element by element (launch_by_element); the WARP policy's row limit stays.
+    if (cols % E != 0 || (addresses & 15) != 0) {
+        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2, or
+        // tensors that start off one): every policy walks such a row element by element (launch_by_element); the
+        // WARP policy's row limit stays.
         constexpr int BY_ELEMENT = io_by_element(IO);
         if (policy != KO_POLICY_AUTO && policy != KO_POLICY_WARP && policy != KO_POLICY_BLOCK && policy != KO_POLICY_BLOCK_NOCACHE)
             return fail(KO_ERR_INVALID_ARGUMENT, "layernorm: unknown policy %d", policy);

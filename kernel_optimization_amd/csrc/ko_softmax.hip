@@ -735,13 +735,15 @@ int entry(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *
     if (cols > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: cols=%lld too large", (long long)cols);
     if (rows == 0) return KO_OK;
     if (!in || !out) return fail(KO_ERR_INVALID_ARGUMENT, "softmax: null in/out pointer");
-    if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15)
-        return fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be 16-byte aligned");
+    const uintptr_t addresses = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out);
+    if (addresses & (sizeof(typename Io<IO>::elem) - 1))
+        return fail(KO_ERR_INVALID_ARGUMENT, "softmax: in/out must be aligned to their element type");
     if (valid_len && rows_per_seq <= 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "softmax: valid_len given but rows_per_seq=%lld", (long long)rows_per_seq);
-    if (cols % E != 0) {
-        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2): every
-        // policy walks such a row element by element (launch_by_element); the policies' row limits stay.
+    if (cols % E != 0 || (addresses & 15) != 0) {
+        // Rows that do not start on 16-byte boundaries (the reference's descriptors with vec_len = 1 or 2, or a
+        // tensor that starts off one): every policy walks such a row element by element (launch_by_element); the
+        // policies' row limits stay.
         constexpr int BY_ELEMENT = io_by_element(IO);
         const int64_t nvec = (cols + E - 1) / E;
         if (policy != KO_POLICY_AUTO && policy != KO_POLICY_WARP && policy != KO_POLICY_BLOCK && policy != KO_POLICY_BLOCK_NOCACHE)

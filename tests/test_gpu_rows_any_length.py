@@ -125,3 +125,47 @@ def test_layernorm_any_length_special_values(ko, cols):
     for name, a, r in zip(("y", "mean", "rstd"), got, ref):
         ok = sv.check_rows(a, r, classes, "layernorm %s cols %d" % (name, cols))
     assert_layernorm_close(tuple(a[ok] for a in got), tuple(r[ok] for r in ref))
+
+
+@pytest.mark.parametrize("cols", [128, 768, 1001, 5000])
+def test_rows_of_tensors_that_start_off_a_16_byte_boundary(ko, cols):
+    """A view into a larger allocation: in, out, gamma and beta one or three elements past a 16-byte boundary (fp32
+    and binary16).  The row length may be a multiple of the vector width or not; the element-wise kernels take it
+    either way, and a pointer that is not even aligned to its element is refused."""
+    rows = 70
+    x = inputs.normal_f32((rows, cols), 770 + cols, 0.5, 2.0)
+    g, b = inputs.normal_f32((cols,), 771, 1.0, 0.1), inputs.normal_f32((cols,), 772, 0.0, 0.1)
+    n = rows * cols
+    for off in (1, 3):
+        dx, dy = ko.DeviceBuffer((n + 8) * 4), ko.DeviceBuffer((n + 8) * 4)
+        dg, db = ko.DeviceBuffer((cols + 8) * 4), ko.DeviceBuffer((cols + 8) * 4)
+        dx.upload(np.concatenate([np.zeros(off, np.float32), x.ravel(), np.zeros(8 - off, np.float32)]))
+        dg.upload(np.concatenate([np.zeros(off, np.float32), g, np.zeros(8 - off, np.float32)]))
+        db.upload(np.concatenate([np.zeros(off, np.float32), b, np.zeros(8 - off, np.float32)]))
+        dy.upload(np.full(n + 8, 7.0, np.float32))
+        ko.softmax(dx.ptr + 4 * off, dy.ptr + 4 * off, rows, cols)
+        ko.synchronize()
+        out = dy.download(np.float32, (n + 8,))
+        assert_softmax_close(out[off:off + n].reshape(rows, cols), oracle.softmax(x))
+        assert np.all(out[:off] == 7.0) and np.all(out[off + n:] == 7.0)
+        dm, dr = ko.DeviceBuffer(rows * 4), ko.DeviceBuffer(rows * 4)
+        ko.layernorm(dx.ptr + 4 * off, dy.ptr + 4 * off, rows, cols, dm, dr, dg.ptr + 4 * off, db.ptr + 4 * off)
+        ko.synchronize()
+        out = dy.download(np.float32, (n + 8,))
+        got = (out[off:off + n].reshape(rows, cols), dm.download(np.float32, (rows,)), dr.download(np.float32, (rows,)))
+        assert_layernorm_close(got, oracle.layernorm(x, g, b))
+        assert np.all(out[:off] == 7.0) and np.all(out[off + n:] == 7.0)
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax(dx.ptr + 2, dy.ptr, rows, cols)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+    # binary16: three elements (6 bytes) past the boundary
+    xb = _bits(x, False)
+    hx, hy = ko.DeviceBuffer((n + 8) * 2), ko.DeviceBuffer((n + 8) * 2)
+    hx.upload(np.concatenate([np.zeros(3, np.uint16), xb.ravel(), np.zeros(5, np.uint16)]))
+    ko.softmax16(hx.ptr + 6, hy.ptr + 6, rows, cols, dtype=ko.F16)
+    ko.synchronize()
+    _, ref64 = oracle.softmax16(xb)
+    assert_softmax16_close(_to64(hy.download(np.uint16, (n + 8,))[3:3 + n].reshape(rows, cols), False), ref64, False)
+    with pytest.raises(ko.KoError) as e:
+        ko.softmax16(hx.ptr + 1, hy.ptr, rows, cols, dtype=ko.F16)
+    assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
