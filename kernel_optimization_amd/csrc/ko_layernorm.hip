@@ -37,65 +37,37 @@
 namespace ko {
 namespace {
 
+// 1/n for the streaming update: the n-th element a lane folds always has count n,
+// so the division of layernorm.h:18 becomes a multiplication by a constant.
+template <int N>
+struct Reciprocals {
+    float v[N + 1];
+    constexpr Reciprocals() : v{} {
+        v[0] = 0.0f;
+        for (int i = 1; i <= N; ++i) v[i] = 1.0f / static_cast<float>(i);
+    }
+};
+
 // 1 / sqrt(x) from the hardware instruction (1 ulp; the gate on rstd is 1e-5 relative).  A correctly rounded
 // square root followed by a correctly rounded division is some 25 instructions that every lane of a row runs.
 // Special values as with the division: +inf -> 0, 0 -> +inf, NaN and negative -> NaN.
 __device__ __forceinline__ float rsqrt_1ulp(float x) { return __builtin_amdgcn_rsqf(x); }
 
-// The streaming update of the reference (WelfordUpdate, layernorm.h:13-23) for values that arrive one at a time (the
-// parts of a long row that are not held in registers): 1/count comes from the hardware reciprocal (1 ulp).  M2 is
-// accumulated against the mean actually formed, so the triplet stays consistent and the deviation is far inside
-// the 1e-5 gate.
+__device__ __forceinline__ void welford_update(wave::Welford &w, float x, float inv_count) {
+    w.count += 1.0f;
+    const float d = x - w.mean;
+    w.mean = __builtin_fmaf(d, inv_count, w.mean);
+    w.m2 = __builtin_fmaf(d, x - w.mean, w.m2);
+}
+
+// The same update where the count is not a compile-time constant: 1/count comes from the hardware reciprocal
+// (1 ulp).  M2 is accumulated against the mean actually formed, so the triplet stays consistent and the
+// deviation is far inside the 1e-5 gate.
 __device__ __forceinline__ void welford_update_counted(wave::Welford &w, float x) {
     w.count += 1.0f;
     const float d = x - w.mean;
     w.mean = __builtin_fmaf(d, __builtin_amdgcn_rcpf(w.count), w.mean);
     w.m2 = __builtin_fmaf(d, x - w.mean, w.m2);
-}
-
-// (count, mean, M2) of the values a thread holds in registers - VPL vectors of E values, of which the first `valid`
-// vectors belong to the row - in two passes of independent operations (E running sums, then E running sums of
-// squared deviations from the thread's own mean) instead of valid * E Welford updates that each wait for the one
-// before.  1 / count comes from the hardware reciprocal (1 ulp): M2 is
-// taken against the mean actually formed, which is off by a few 1e-8 of the spread at most, so the triplet merges
-// like an exact one far inside the 1e-5 gate.
-template <int VPL, int E>
-__device__ __forceinline__ wave::Welford triplet_of(const float (&v)[VPL][E], int valid) {
-    float s[E], q[E];
-#pragma unroll
-    for (int e = 0; e < E; ++e) s[e] = q[e] = 0.0f;
-#pragma unroll
-    for (int k = 0; k < VPL; ++k) {
-        if (k < valid) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) s[e] += v[k][e];
-        }
-    }
-    float sum = s[0];
-#pragma unroll
-    for (int e = 1; e < E; ++e) sum += s[e];
-    const float n = static_cast<float>(valid * E);
-    const float mean = sum * __builtin_amdgcn_rcpf(valid > 0 ? n : 1.0f);
-#pragma unroll
-    for (int k = 0; k < VPL; ++k) {
-        if (k < valid) {
-#pragma unroll
-            for (int e = 0; e < E; ++e) {
-                const float d = v[k][e] - mean;
-                q[e] = __builtin_fmaf(d, d, q[e]);
-            }
-        }
-    }
-    float m2 = q[0];
-#pragma unroll
-    for (int e = 1; e < E; ++e) m2 += q[e];
-    return wave::Welford{n, mean, m2};
-}
-// how many of a thread's vectors first, first + step, ... lie below nvec (at most vpl)
-__device__ __forceinline__ int valid_vectors(int first, int step, int nvec, int vpl) {
-    const int left = nvec - first;
-    const int n = left > 0 ? (left + step - 1) / step : 0;
-    return n < vpl ? n : vpl;
 }
 
 template <int IO>
@@ -133,6 +105,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     constexpr int E = Io<IO>::E;
     constexpr int RPW = 64 / LPR;
     constexpr bool NT = true;  // streaming accesses: every byte is touched once
+    constexpr Reciprocals<VPL * E> rcp;
     const int lane = threadIdx.x & 63;
     const int sub = lane / LPR;
     const int l = lane % LPR;
@@ -218,10 +191,15 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
             w = wave::Welford{static_cast<float>(VPL * E), lane_mean, m2};
         } else {
 #pragma unroll
-            for (int k = 0; k < VPL; ++k)
+            for (int k = 0; k < VPL; ++k) {
+                const int j = l + k * LPR;
 #pragma unroll
                 for (int e = 0; e < E; ++e) v[k][e] -= x0;
-            w = triplet_of<VPL, E>(v, valid_vectors(l, LPR, nvec, VPL));
+                if (FULL || j < nvec) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
+                }
+            }
         }
         if constexpr (FULL) w = wave::welford_allreduce_equal<LPR>(w);
         else w = wave::welford_allreduce<LPR>(w);
@@ -350,6 +328,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
     __shared__ float lds[48];
     extern __shared__ __attribute__((aligned(16))) char tail_bytes[];  // Raw tail[LV][THREADS]
     Raw *tail = reinterpret_cast<Raw *>(tail_bytes);
+    constexpr Reciprocals<VPL * E> rcp;
     constexpr int UNROLL = 2;                       // vectors per thread and trip of the streamed part
     constexpr int kCached = (VPL + LV) * THREADS;   // vectors of a row held on chip
     const int nvec = cols / E;
@@ -405,11 +384,17 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_kernel(const typename
             for (int k = 0; k < VPL; ++k) Io<IO>::unpack(loaded[k], v[k]);
         }
         const float x0 = Io<IO>::scalar(src);
+        wave::Welford w{0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int k = 0; k < VPL; ++k)
+        for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
 #pragma unroll
             for (int e = 0; e < E; ++e) v[k][e] -= x0;
-        wave::Welford w = triplet_of<VPL, E>(v, valid_vectors(threadIdx.x, THREADS, nvec, VPL));
+            if (j < nvec) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) welford_update(w, v[k][e], rcp.v[E * k + e + 1]);
+            }
+        }
         // (the loops over the tail are kept rolled: unrolled, the compiler fetches all of it from LDS at once and spills)
 #pragma unroll 1
         for (int k = 0; k < LV; ++k) {
@@ -616,6 +601,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_batch_kernel(const ty
     constexpr int WAVES = THREADS / 64;
     typedef typename Io<IO>::raw Raw;
     __shared__ float lds[R * 3 * 16];
+    constexpr Reciprocals<VPL * E> rcp;
     const int nvec = cols / E;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
     const uint32_t first = threadIdx.x * 16u;
@@ -656,13 +642,18 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_batch_kernel(const ty
     wave::Welford w[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
+        w[r] = wave::Welford{0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
+            const int j = threadIdx.x + k * THREADS;
             Io<IO>::unpack(loaded[r][k], v[r][k]);
 #pragma unroll
             for (int e = 0; e < E; ++e) v[r][k][e] -= x0[r];
+            if (j < nvec) {  // a thread's valid vectors are its first ones, so the n-th element it folds has count n
+#pragma unroll
+                for (int e = 0; e < E; ++e) welford_update(w[r], v[r][k][e], rcp.v[E * k + e + 1]);
+            }
         }
-        w[r] = triplet_of<VPL, E>(v[r], valid_vectors(threadIdx.x, THREADS, nvec, VPL));
         w[r] = wave::welford_allreduce<64>(w[r]);
     }
     if constexpr (WAVES > 1) {
