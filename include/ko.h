@@ -109,7 +109,11 @@ int ko_event_destroy(ko_event_t event);
  * reference's descriptors do with vec_len = 1 or 2), at 0.6-0.9 of the rate.
  * valid_len: NULL for no mask, else device int32[ceil(rows / rows_per_seq)];
  * row r belongs to sequence r / rows_per_seq and every column
- * j >= valid_len[seq] takes the value -10000 before the softmax. */
+ * j >= valid_len[seq] takes the value -10000 before the softmax.
+ * Workspace: a few long rows (fewer rows than a quarter of the compute units, 256 KB and more each) run as two
+ * launches that pass partial results through the (device, stream) workspace described at ko_sgemm_f32; the same
+ * holds for ko_layernorm_f32 and the 16-bit forms.  Without a workspace (first such call inside a graph capture)
+ * they run as one launch, one workgroup per row. */
 int ko_softmax_f32(const float *in, float *out, int64_t rows, int64_t cols,
                    const int32_t *valid_len, int64_t rows_per_seq, ko_stream_t stream);
 

@@ -582,6 +582,105 @@ __global__ __launch_bounds__(THREADS) void layernorm_nocache_kernel(const typena
     }
 }
 
+// ------------------------------------------- few rows: a row split over workgroups
+// With fewer rows than compute units one workgroup per row leaves most of the chip idle.  Such rows are cut into
+// `parts` pieces of `piece` vectors each, one workgroup per piece, in two launches with nothing but the kernel
+// boundary between them: the first leaves every piece's Welford triplet (of x - x0, x0 the row's first element)
+// in a workspace, the second merges a row's triplets - in piece order, every workgroup the same way, so the result
+// is the same bits from call to call - and writes its piece of the output, reading the piece a second time.
+// blockIdx.x = piece, blockIdx.y = row.
+template <int IO, int THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_pieces_stats_kernel(const typename Io<IO>::elem *in, int cols,
+                                                                         int piece, wave::Welford *__restrict__ triplets) {
+    constexpr int E = Io<IO>::E;
+    constexpr int UNROLL = 4;
+    __shared__ float lds[48];
+    const int nvec = cols / E;
+    const int64_t row = blockIdx.y;
+    const int lo = static_cast<int>(blockIdx.x) * piece;
+    const int hi = lo + piece < nvec ? lo + piece : nvec;
+    const typename Io<IO>::elem *src = in + row * cols;
+    const float x0 = Io<IO>::scalar(src);
+    wave::Welford w{0.0f, 0.0f, 0.0f};
+    for (int j0 = lo + threadIdx.x; j0 < hi; j0 += THREADS * UNROLL) {
+        float x[UNROLL][E];
+        typename Io<IO>::raw loaded[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            loaded[u] = typename Io<IO>::raw{};
+            if (j0 + u * THREADS < hi) loaded[u] = Io<IO>::template load_raw<false>(src + E * (j0 + u * THREADS));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (j0 + u * THREADS >= hi) break;
+#pragma unroll
+            for (int e = 0; e < E; ++e) welford_update_counted(w, x[u][e] - x0);
+        }
+    }
+    w = block_welford_allreduce<THREADS>(w, lds);
+    if (threadIdx.x == 0) {
+        triplets[row * gridDim.x + blockIdx.x] = w;
+        // x0 goes along (behind all the triplets): in place, the second launch finds the row's first element
+        // overwritten by whichever workgroup got to piece 0 first
+        if (blockIdx.x == 0) reinterpret_cast<float *>(triplets + static_cast<int64_t>(gridDim.y) * gridDim.x)[row] = x0;
+    }
+}
+
+template <int IO, int THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_pieces_apply_kernel(const typename Io<IO>::elem *in,
+                                                                         typename Io<IO>::elem *out,
+                                                                         float *__restrict__ mean_out,
+                                                                         float *__restrict__ rstd_out,
+                                                                         const typename Io<IO>::elem *__restrict__ gamma,
+                                                                         const typename Io<IO>::elem *__restrict__ beta,
+                                                                         int cols, float eps, float inv_denominator, int piece,
+                                                                         const wave::Welford *__restrict__ triplets) {
+    constexpr int E = Io<IO>::E;
+    constexpr int UNROLL = 4;
+    const int nvec = cols / E;
+    const int64_t row = blockIdx.y;
+    const int parts = static_cast<int>(gridDim.x);
+    const int lo = static_cast<int>(blockIdx.x) * piece;
+    const int hi = lo + piece < nvec ? lo + piece : nvec;
+    const typename Io<IO>::elem *src = in + row * cols;
+    const float x0 = reinterpret_cast<const float *>(triplets + static_cast<int64_t>(gridDim.y) * parts)[row];
+    // the row's triplet from its pieces', merged in piece order (wave-uniform loads)
+    const wave::Welford *mine = triplets + row * parts;
+    wave::Welford w = mine[0];
+    for (int i = 1; i < parts; ++i) w = wave::welford_merge(w, mine[i]);
+    const float mean = w.mean;  // of the shifted row
+    const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
+    typename Io<IO>::elem *dst = out + row * cols;
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
+    for (int j0 = lo + threadIdx.x; j0 < hi; j0 += THREADS * UNROLL) {
+        float x[UNROLL][E];
+        typename Io<IO>::raw loaded[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            loaded[u] = typename Io<IO>::raw{};
+            if (j0 + u * THREADS < hi) loaded[u] = Io<IO>::template load_raw<true>(src + E * (j0 + u * THREADS));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) Io<IO>::unpack(loaded[u], x[u]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = j0 + u * THREADS;
+            if (j >= hi) break;
+            float y[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) x[u][e] -= x0;
+            normalize_vec<IO>(x[u], mean, rstd, gamma, beta, E * j, y);
+            store_row_vec<IO>(whole_lines, dst, Io<IO>::kBytes * j, y);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (mean_out) mean_out[row] = rstd != rstd ? rstd : x0 + mean;  // no statistics for a row with NaN or inf
+        if (rstd_out) rstd_out[row] = rstd;
+    }
+}
+
 // Rows of a few vectors per thread (up to 2048 vectors: 8192 fp32 columns): one workgroup per group of R rows,
 // dispatched in row order and gone when its rows are written (a one-shot launch keeps the memory system busier
 // than a grid that walks the rows in step: [32768, 4096] without gamma and beta 181 -> 165 us, the time of the
@@ -963,6 +1062,40 @@ int launch_by_element(const Args<IO> &a) {
     return launch_block_by_element<IO, 64, true>(a);  // (without REST this one spills; with it, it does not)
 }
 
+// Few long rows (see layernorm_pieces_stats_kernel).  Pieces of at least 1024 vectors (16 KB), two workgroups per
+// compute unit in all.  Returns -1 when the
+// shape is left to the one-workgroup-per-row kernels, or when the stream has no workspace to be had (inside a
+// graph capture on a stream that never ran a call that needs one).
+template <int IO>
+int launch_pieces(const Args<IO> &a) {
+    constexpr int THREADS = 256;
+    const int nvec = a.cols / Io<IO>::E;
+    const int cu = compute_units();
+    // two launches have a fixed cost of some 10 us: it pays from rows of 256 KB on for up to a quarter of the
+    // compute units' worth of rows ([64, 128256]: 29 -> 22 us, [32, 128256] 28 -> 14 us, [1, 16777216] 3.8 ms ->
+    // 96 us; [64, 32768] 9 against 10 us), from rows of 1 MB on for up to half ([128, 524288]: 168 -> 149 us;
+    // [128, 128256] 35 against 42 us)
+    if (!((a.rows * 4 <= cu && nvec >= 16384) || (a.rows * 2 <= cu && nvec >= 65536))) return -1;
+    int parts = static_cast<int>(2 * cu / a.rows);
+    if (parts > nvec / 1024) parts = nvec / 1024;
+    if (parts < 2) return -1;
+    int piece = (nvec + parts - 1) / parts;
+    piece = (piece + THREADS - 1) / THREADS * THREADS;  // whole trips of the workgroup; the last piece is the short one
+    parts = (nvec + piece - 1) / piece;
+    void *workspace = nullptr;
+    if (const int st = stream_workspace(a.stream, &workspace); st != KO_OK) return st;
+    if (workspace == nullptr || static_cast<size_t>(a.rows) * (parts * sizeof(wave::Welford) + sizeof(float)) > kStreamWorkspaceBytes)
+        return -1;
+    wave::Welford *triplets = static_cast<wave::Welford *>(workspace);
+    const dim3 grid(static_cast<unsigned>(parts), static_cast<unsigned>(a.rows));
+    layernorm_pieces_stats_kernel<IO, THREADS><<<grid, dim3(THREADS), 0, a.stream>>>(a.in, a.cols, piece, triplets);
+    KO_CHECK_LAUNCH();
+    layernorm_pieces_apply_kernel<IO, THREADS><<<grid, dim3(THREADS), 0, a.stream>>>(
+        a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.cols, a.eps, a.inv_denominator, piece, triplets);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 template <int IO>
 int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma, const void *beta, int64_t rows,
           int64_t cols, float eps, int unbiased, int policy, ko_stream_t stream) {
@@ -1001,6 +1134,7 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
                as_stream(stream)};
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
+        if (const int st = launch_pieces<IO>(a); st != -1) return st;
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
                                       : KO_POLICY_BLOCK;  // rows past what the chip holds stream their far end twice
     }

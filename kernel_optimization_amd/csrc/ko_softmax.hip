@@ -448,6 +448,105 @@ __global__ __launch_bounds__(THREADS) void softmax_nocache_kernel(const typename
     }
 }
 
+// ------------------------------------------- few rows: a row split over workgroups
+// With fewer rows than compute units (the softmax over a vocabulary for a batch of a few dozen rows) one workgroup
+// per row leaves most of the chip idle.  Such rows are cut into `parts` pieces of `piece` vectors each, one
+// workgroup per piece, in two launches with nothing but the kernel boundary between them: the first leaves every
+// piece's (maximum, sum of exponentials against that maximum) in a workspace, the second folds a row's pairs - in
+// piece order, every workgroup the same way, so the result is the same bits from call to call - and writes its
+// piece of the output, reading the piece a second time (it is the only traffic that is added; a tensor of a few
+// rows sits in the last-level cache).  blockIdx.x = piece, blockIdx.y = row.
+struct PiecePair {
+    float m, s;
+};
+
+template <int IO, int THREADS, bool MASKED>
+__global__ __launch_bounds__(THREADS) void softmax_pieces_stats_kernel(const typename Io<IO>::elem *in, int cols,
+                                                                       const int32_t *__restrict__ valid_len,
+                                                                       int64_t rows_per_seq, int piece,
+                                                                       PiecePair *__restrict__ pairs) {
+    constexpr int E = Io<IO>::E;
+    constexpr int UNROLL = 4;
+    __shared__ float lds[16];
+    const int nvec = cols / E;
+    const int64_t row = blockIdx.y;
+    const int lo = static_cast<int>(blockIdx.x) * piece;
+    const int hi = lo + piece < nvec ? lo + piece : nvec;
+    const typename Io<IO>::elem *src = in + row * cols;
+    int vlen = cols;
+    if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+    float m = -FLT_MAX, s = 0.0f;
+    for (int j0 = lo + threadIdx.x; j0 < hi; j0 += THREADS * UNROLL) {
+        float x[UNROLL][E];
+        typename Io<IO>::raw loaded[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = j0 + u * THREADS;
+            loaded[u] = typename Io<IO>::raw{};
+            if (j < hi) loaded[u] = fetch_row_vec<IO, MASKED, false>(src + E * j, j, vlen);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) finish_row_vec<IO, MASKED>(loaded[u], j0 + u * THREADS, vlen, x[u]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (j0 + u * THREADS >= hi) break;
+#pragma unroll
+            for (int e = 0; e < E; ++e) online_add(m, s, x[u][e]);
+        }
+    }
+    const float gm = block_allreduce<THREADS, wave::Max>(m, lds, -FLT_MAX);
+    s *= exp_nonpositive(m - gm);  // threads that saw nothing: s = 0
+    const float gs = block_allreduce<THREADS, wave::Sum>(s, lds, 0.0f);
+    if (threadIdx.x == 0) pairs[row * gridDim.x + blockIdx.x] = PiecePair{gm, gs};
+}
+
+template <int IO, int THREADS, bool MASKED>
+__global__ __launch_bounds__(THREADS) void softmax_pieces_apply_kernel(const typename Io<IO>::elem *in,
+                                                                       typename Io<IO>::elem *out, int cols,
+                                                                       const int32_t *__restrict__ valid_len,
+                                                                       int64_t rows_per_seq, int piece,
+                                                                       const PiecePair *__restrict__ pairs) {
+    constexpr int E = Io<IO>::E;
+    constexpr int UNROLL = 4;
+    const int nvec = cols / E;
+    const int64_t row = blockIdx.y;
+    const int parts = static_cast<int>(gridDim.x);
+    const int lo = static_cast<int>(blockIdx.x) * piece;
+    const int hi = lo + piece < nvec ? lo + piece : nvec;
+    const typename Io<IO>::elem *src = in + row * cols;
+    int vlen = cols;
+    if constexpr (MASKED) vlen = clamp_len(valid_len[row / rows_per_seq], cols);
+    // the row's maximum and sum from its pieces' pairs, folded in piece order (wave-uniform loads)
+    const PiecePair *mine = pairs + row * parts;
+    float gm = -FLT_MAX;
+    for (int i = 0; i < parts; ++i) gm = fmaxf(gm, mine[i].m);
+    float gs = 0.0f;
+    for (int i = 0; i < parts; ++i) gs += mine[i].s * exp_nonpositive(mine[i].m - gm);
+    const float inv = 1.0f / gs;
+    typename Io<IO>::elem *dst = out + row * cols;
+    const bool whole_lines = rows_are_whole_lines<IO>(cols);
+    for (int j0 = lo + threadIdx.x; j0 < hi; j0 += THREADS * UNROLL) {
+        float x[UNROLL][E];
+        typename Io<IO>::raw loaded[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = j0 + u * THREADS;
+            loaded[u] = typename Io<IO>::raw{};
+            if (j < hi) loaded[u] = fetch_row_vec<IO, MASKED, true>(src + E * j, j, vlen);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) finish_row_vec<IO, MASKED>(loaded[u], j0 + u * THREADS, vlen, x[u]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = j0 + u * THREADS;
+            if (j >= hi) break;
+#pragma unroll
+            for (int e = 0; e < E; ++e) x[u][e] = exp_for_storage<IO>(x[u][e] - gm) * inv;
+            store_row_vec<IO>(whole_lines, dst, Io<IO>::kBytes * j, x[u]);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ dispatch
 template <int IO>
 struct Args {
@@ -698,11 +797,46 @@ int launch_by_element(const Args<IO> &a) {
     return launch_nocache<IO, MASKED>(a);
 }
 
+// Few long rows (see softmax_pieces_stats_kernel).  Pieces of at least 1024 vectors (16 KB), two workgroups per
+// compute unit in all.  Returns -1 when the
+// shape is left to the one-workgroup-per-row kernels, or when the stream has no workspace to be had (inside a
+// graph capture on a stream that never ran a call that needs one).
+template <int IO, bool MASKED>
+int launch_pieces(const Args<IO> &a) {
+    constexpr int THREADS = 256;
+    const int nvec = a.cols / Io<IO>::E;
+    const int cu = compute_units();
+    // two launches have a fixed cost of some 10 us: it pays from rows of 256 KB on for up to a quarter of the
+    // compute units' worth of rows ([64, 128256]: 29 -> 22 us, [32, 128256] 28 -> 14 us, [1, 16777216] 3.8 ms ->
+    // 96 us; [64, 32768] 9 against 10 us), from rows of 1 MB on for up to half ([128, 524288]: 168 -> 149 us;
+    // [128, 128256] 35 against 42 us)
+    if (!((a.rows * 4 <= cu && nvec >= 16384) || (a.rows * 2 <= cu && nvec >= 65536))) return -1;
+    int parts = static_cast<int>(2 * cu / a.rows);
+    if (parts > nvec / 1024) parts = nvec / 1024;
+    if (parts < 2) return -1;
+    int piece = (nvec + parts - 1) / parts;
+    piece = (piece + THREADS - 1) / THREADS * THREADS;  // whole trips of the workgroup; the last piece is the short one
+    parts = (nvec + piece - 1) / piece;
+    void *workspace = nullptr;
+    if (const int st = stream_workspace(a.stream, &workspace); st != KO_OK) return st;
+    if (workspace == nullptr || static_cast<size_t>(a.rows) * parts * sizeof(PiecePair) > kStreamWorkspaceBytes) return -1;
+    PiecePair *pairs = static_cast<PiecePair *>(workspace);
+    const dim3 grid(static_cast<unsigned>(parts), static_cast<unsigned>(a.rows));
+    softmax_pieces_stats_kernel<IO, THREADS, MASKED><<<grid, dim3(THREADS), 0, a.stream>>>(a.in, a.cols, a.valid_len,
+                                                                                          a.rows_per_seq, piece, pairs);
+    KO_CHECK_LAUNCH();
+    softmax_pieces_apply_kernel<IO, THREADS, MASKED><<<grid, dim3(THREADS), 0, a.stream>>>(
+        a.in, a.out, a.cols, a.valid_len, a.rows_per_seq, piece, pairs);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 template <int IO, bool MASKED>
 int dispatch(const Args<IO> &a, int policy) {
     constexpr int E = Io<IO>::E;
     const int nvec = a.cols / E;
     if (policy == KO_POLICY_AUTO) {
+        if (const int st = launch_pieces<IO, MASKED>(a); st != -1) return st;
         policy = nvec <= kWaveMaxVecs ? KO_POLICY_WARP
                  : nvec <= (MASKED ? kBlockMaxVecsMasked<IO> : kBlockAutoMaxVecs<IO>) ? KO_POLICY_BLOCK
                                          : KO_POLICY_BLOCK_NOCACHE;

@@ -1,6 +1,6 @@
 """The operators are plain kernel launches on the caller's stream, so a caller can capture them into a HIP graph
 (the reference's drivers launch on one non-blocking stream as well, softmax/main.cu:28-29).  This test captures a
-softmax -> LayerNorm -> 16-bit GEMM -> SGEMM -> 16-bit GEMM (persistent kernel) -> K-sliced SGEMM and 16-bit GEMM sequence with the HIP runtime that libko.so itself is linked against,
+softmax -> LayerNorm -> 16-bit GEMM -> SGEMM -> 16-bit GEMM (persistent kernel) -> K-sliced SGEMM and 16-bit GEMM -> softmax and LayerNorm of a few long rows (cut into pieces) sequence with the HIP runtime that libko.so itself is linked against,
 replays the graph several times with eager work and synchronisations in between, and compares every replay bit
 for bit with the eager results.  One eager pass comes first: the library's one-time set-up (device properties,
 kernel attributes) is not stream work and belongs in front of a capture."""
@@ -57,6 +57,9 @@ def test_operators_replay_from_a_hip_graph(ko):
     a5, b5, d5 = ko.DeviceBuffer(m5 * k5 * 2), ko.DeviceBuffer(n5 * k5 * 2), ko.DeviceBuffer(m5 * n5 * 2)
     ko.fill_uniform_16(a5, m5 * k5, 513)
     ko.fill_uniform_16(b5, n5 * k5, 514)
+    rows6, cols6 = 8, 131072  # a few long rows: cut into pieces that hand partial results over through the workspace
+    x6 = ko.DeviceBuffer.from_numpy(inputs.normal_f32((rows6, cols6), 515, 0.0, 4.0))
+    s6, l6 = ko.DeviceBuffer(rows6 * cols6 * 4), ko.DeviceBuffer(rows6 * cols6 * 4)
     ko.fill_uniform_16(a3, m3 * k3, 509)
     ko.fill_uniform_16(b3, n3 * k3, 510)
     ko.fill_uniform_16(a2, m2 * k2, 507)
@@ -76,21 +79,25 @@ def test_operators_replay_from_a_hip_graph(ko):
         ko.gemm16(m3, n3, k3, a3, b3, d3, stream=stream)
         ko.sgemm(m4, n4, k4, a4, b4, d4, stream=stream)
         ko.gemm16(m5, n5, k5, a5, b5, d5, stream=stream)
+        ko.softmax(x6, s6, rows6, cols6, stream=stream)
+        ko.layernorm(s6, l6, rows6, cols6, stream=stream)
 
     def outputs():
         return (dl.download(np.uint32, (rows, cols)), dmean.download(np.uint32, (rows,)),
                 d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)),
-                d3.download(np.uint16, (m3, n3)), d4.download(np.uint32, (m4, n4)), d5.download(np.uint16, (m5, n5)))
+                d3.download(np.uint16, (m3, n3)), d4.download(np.uint32, (m4, n4)), d5.download(np.uint16, (m5, n5)),
+                l6.download(np.uint32, (rows6, cols6)))
 
     def clear():
         for buf, nbytes in ((ds, rows * cols * 4), (dl, rows * cols * 4), (dmean, rows * 4), (d16, m * n * 2), (d32, m * n * 4),
-                            (d2, m2 * n2 * 2), (d3, m3 * n3 * 2), (d4, m4 * n4 * 4), (d5, m5 * n5 * 2)):
+                            (d2, m2 * n2 * 2), (d3, m3 * n3 * 2), (d4, m4 * n4 * 4), (d5, m5 * n5 * 2),
+                            (s6, rows6 * cols6 * 4), (l6, rows6 * cols6 * 4)):
             buf.upload(np.zeros(nbytes, np.uint8))
 
     chain()
     stream.synchronize()
     want = outputs()
-    assert want[0].any() and want[2].any() and want[3].any() and want[6].any() and want[7].any()
+    assert want[0].any() and want[2].any() and want[3].any() and want[6].any() and want[7].any() and want[8].any()
 
     graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
     assert hip.hipStreamBeginCapture(stream.handle, 0) == 0  # hipStreamCaptureModeGlobal
