@@ -660,7 +660,9 @@ def main():
                                        ("layernorm", 8192, 16384, ko.POLICY_BLOCK),
                                        ("layernorm", 2048, 65536, ko.POLICY_BLOCK),
                                        ("layernorm", 1024, 131072, ko.POLICY_BLOCK),
-                                       ("layernorm", 1024, 131072, ko.POLICY_BLOCK_NOCACHE)):
+                                       ("layernorm", 1024, 131072, ko.POLICY_BLOCK_NOCACHE),
+                                       # a vocabulary for a batch of 32 rows: each row cut into pieces (two launches)
+                                       ("softmax", 32, 128256, ko.POLICY_AUTO)):
             res = bench_long_rows(op, rows, cols, policy, args.steps, args.warmup)
             res["steps"], res["warmup"] = args.steps, args.warmup
             others.append(res)
