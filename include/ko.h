@@ -262,7 +262,7 @@ int ko_debug_wave_allreduce(const float *in, float *out, int group, int op, ko_s
 /* What the GEMMs' host-side planners decide for a shape (16-byte aligned operands, 256 compute units when no
  * device is visible): the number of K slices (1 = the problem goes out whole), the depth of every slice but the
  * last, and the tiling of the sliced launch (SGEMM: the kernel variant number, 0 = chosen as for the whole
- * problem; 16-bit GEMM: 128 or 64, the tile edge).  Touches no device memory and launches nothing. */
+ * problem; 16-bit GEMM: 128 or 64, the tile edge, or 32 for 32 x 256 tiles).  Touches no device memory and launches nothing. */
 int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
 int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
 

@@ -1227,6 +1227,7 @@ using TileBig = Tiling<256, 256, 2, 4, 1, true, 1>;     // 8 waves, wave tile 12
 using TileSmall = Tiling<128, 128, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x64, two register stages
 using TileSmallN = Tiling<128, 64, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64x32
 using TileTiny = Tiling<64, 64, 2, 2, 2, true, 1>;      // 4 waves, wave tile 32x32
+using TileSkinny = Tiling<32, 256, 1, 4, 2, true, 1>;   // 4 waves side by side, wave tile 32x64: at most 32 rows of A
 
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
@@ -1291,7 +1292,7 @@ __global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, i
 //     (2048 x 768 x 3072: 25.5 whole, 27 in four slices).
 struct SlicePlan16 {
     int slices = 1, k_slice = 0;
-    bool tiles_128 = false;  // 128 x 128 tiles (else 64 x 64)
+    int tile = 64;  // 128: 128 x 128 tiles, 64: 64 x 64, 32: the 32 x 256 tiles of a problem with at most 32 rows
 };
 
 SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
@@ -1300,33 +1301,41 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     if (forced == 1 || p.N % 8 != 0 || p.ldd % 4 != 0) return plan;
     const int64_t cu = compute_units();
     const double out_bytes = 4.0 * p.M * p.N;
-    auto set = [&](int64_t slices, bool tiles_128) {
+    auto set = [&](int64_t slices, int tile) {
         if (slices < 2) return;
         const int64_t depth = ((p.K + slices - 1) / slices + kBK - 1) / kBK * kBK;
         slices = (p.K + depth - 1) / depth;
         if (slices < 2 || slices > 65535 || slices * out_bytes > static_cast<double>(workspace_bytes)) return;
         plan.slices = static_cast<int>(slices);
         plan.k_slice = static_cast<int>(depth);
-        plan.tiles_128 = tiles_128;
+        plan.tile = tile;
     };
     const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
     const int64_t t64 = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64);
     if (forced >= 2) {
-        set(forced, t128 * forced >= cu / 2);
+        set(forced, t128 * forced >= cu / 2 ? 128 : 64);
         return plan;
     }
-    if (p.K < 2048) return plan;
     const int64_t fit = static_cast<int64_t>(static_cast<double>(workspace_bytes) / out_bytes);  // slices the workspace holds
     auto capped = [&](int64_t slices, int64_t min_depth) {
         if (slices > p.K / min_depth) slices = p.K / min_depth;
         return slices < fit ? slices : fit;
     };
+    if (p.M <= 32 && p.N >= 256 && p.K >= 1024) {
+        // A batch of a few rows against a weight matrix: the time is B's, read once.  32 x 256 tiles (one matrix
+        // instruction's worth of rows), slices at least 256 deep up to two workgroups per compute unit, so that
+        // every compute unit streams its share of B.
+        const int64_t skinny = (p.N + 255) / 256;
+        if (skinny <= cu) set(capped(2 * cu / skinny, 256), 32);
+        if (plan.slices > 1) return plan;
+    }
+    if (p.K < 2048) return plan;
     if (4 * t128 <= cu) {
         const int64_t s128 = capped(cu / t128, 512), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
-        if (s64 >= 2 && s64 * t64 >= s128 * t128) set(s64, false);
-        else set(s128, true);
+        if (s64 >= 2 && s64 * t64 >= s128 * t128) set(s64, 64);
+        else set(s128, 128);
     } else if (t128 <= cu) {
-        set(capped(2 * cu / t128, 2048), true);
+        set(capped(2 * cu / t128, 2048), 128);
     }
     return plan;
 }
@@ -1336,7 +1345,9 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
     Params part = p;
     part.k_slice = plan.k_slice;
     part.partial = workspace;
-    int st = plan.tiles_128 ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream) : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
+    int st = plan.tile == 128  ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream)
+             : plan.tile == 32 ? launch<TileSkinny, BF16, B_ROW_MAJOR>(part, stream)
+                               : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
     if (st != KO_OK) return st;
     const int64_t groups = static_cast<int64_t>(p.M) * (p.N / 4);
     gemm16_slices_sum_kernel<BF16><<<dim3(static_cast<unsigned>((groups + 63) / 64)), dim3(64), 0, stream>>>(part, plan.slices);
@@ -1358,7 +1369,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
     if (variant <= 0 && col_cut && row_cuts == 2 && p.k_slice == 0) {
         // the whole problem, before any cut: few tiles and a deep K go out as K slices
         const int64_t big = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
-        if (2 * big < compute_units()) {
+        if (2 * big < compute_units() || p.M <= 32) {
             if (const SlicePlan16 plan = plan_k_slices16(p, kStreamWorkspaceBytes); plan.slices > 1) {
                 void *workspace = nullptr;
                 if (const int st = stream_workspace(stream, &workspace); st != KO_OK) return st;
@@ -1425,6 +1436,9 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // the two are level).
         if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K >= 2 * kBK)
             return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
+        // at most 32 rows: one matrix instruction's worth of rows per tile, 256 columns wide (8 x 4096 x 4096 in
+        // 64 x 64 tiles loads 64 rows of A per tile and multiplies 56 of them for nothing)
+        if (p.M <= 32 && p.N >= 256) return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
         if (big_tiles < compute_units()) {
             // Fewer big tiles than that: the largest of the small tilings that still gives every compute unit one
             // and a half workgroups (two are resident at a time), else the smallest (1024^3: 64 x 64 tiles 8.8 us,
@@ -1450,6 +1464,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 10: return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         case 11: return launch<TileTiny, BF16, B_ROW_MAJOR>(p, stream);
         case 12: return launch<TileSmallN, BF16, B_ROW_MAJOR>(p, stream);
+        case 13: return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
         case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
@@ -1512,9 +1527,9 @@ KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices,
     p.ldk = p.K;
     const int64_t big = ((m + 255) / 256) * ((n + 255) / 256);
     SlicePlan16 plan;
-    if (2 * big < compute_units()) plan = plan_k_slices16(p, kStreamWorkspaceBytes);  // as launch_variant asks
+    if (2 * big < compute_units() || m <= 32) plan = plan_k_slices16(p, kStreamWorkspaceBytes);  // as launch_variant asks
     *slices = plan.slices;
     *k_slice = plan.k_slice;
-    *tile = plan.slices > 1 ? (plan.tiles_128 ? 128 : 64) : 0;
+    *tile = plan.slices > 1 ? plan.tile : 0;
     return KO_OK;
 }

@@ -12,7 +12,7 @@ import pytest
 import kernel_optimization_amd as ko
 
 WORKSPACE = 32 << 20
-SIZES = [64, 100, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
+SIZES = [8, 32, 64, 100, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
 DEPTHS = [64, 512, 767, 768, 1300, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
 
 
@@ -40,10 +40,12 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
 def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
     for k in DEPTHS:
         plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
-        _check(m, n, k, plan, k_tile=64, min_k=2048)
+        _check(m, n, k, plan, k_tile=64, min_k=1024 if m <= 32 else 2048)
         if n % 8:
             assert plan[0] == 1, (m, n, k, plan)           # partial products are written four columns at a time
-        assert plan[2] in ((128, 64) if plan[0] > 1 else (0,))
+        assert plan[2] in ((128, 64, 32) if plan[0] > 1 else (0,))
+        if plan[2] == 32:
+            assert m <= 32
 
 
 def test_measured_decisions_stay_put():

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 13, 16, 21, 33, 35, 36, 37, 40, 41]
 SGEMM_PIPELINED = [13, 16, 21, 33, 35, 36, 37, 40, 41]  # two K tiles per loop trip; 33 on: direct-to-LDS
-GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 30, 50, 52, 53]
+GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 13, 30, 50, 52, 53]
 
 
 @pytest.fixture
@@ -535,7 +535,9 @@ def test_gemm16_bias_activation(ko, act, bf16, b_col_major, m, n, k):
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k,slices", [(512, 512, 8192, 0), (256, 384, 2048, 3), (300, 520, 1096, 2), (768, 768, 4096, 7),
-                                          (130, 72, 4104, 5)])
+                                          (130, 72, 4104, 5),
+                                          # at most 32 rows: 32 x 256 tiles, slices chosen by the planner
+                                          (8, 4096, 4096, 0), (1, 512, 8192, 0), (32, 264, 1096, 0), (20, 1000, 2048, 0)])
 def test_gemm16_k_slices(ko, m, n, k, slices, b_col_major, bf16):
     """A deep K on few tiles goes out as K slices of the register pipeline (fp32 partial products into the stream's
     workspace) and a kernel that sums them in slice order and applies alpha, beta C, bias and the activation once.
