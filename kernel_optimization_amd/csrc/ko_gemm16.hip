@@ -1321,7 +1321,7 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
         if (slices > p.K / min_depth) slices = p.K / min_depth;
         return slices < fit ? slices : fit;
     };
-    if (p.M <= 32 && p.N >= 256 && p.K >= 1024) {
+    if (p.M <= 32 && p.N >= 256 && p.K >= 2048) {
         // A batch of a few rows against a weight matrix: the time is B's, read once.  32 x 256 tiles (one matrix
         // instruction's worth of rows), slices at least 256 deep up to two workgroups per compute unit, so that
         // every compute unit streams its share of B.
@@ -1436,9 +1436,10 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // the two are level).
         if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K >= 2 * kBK)
             return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
-        // at most 32 rows: one matrix instruction's worth of rows per tile, 256 columns wide (8 x 4096 x 4096 in
-        // 64 x 64 tiles loads 64 rows of A per tile and multiplies 56 of them for nothing)
-        if (p.M <= 32 && p.N >= 256) return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
+        // at most 32 rows and tiles for every compute unit: one matrix instruction's worth of rows per tile, 256
+        // columns wide (64 x 64 tiles load 64 rows of A per tile and multiply most of them for nothing); with
+        // fewer tiles the smaller tilings below put more workgroups to work (8 x 3072 x 768: 8 us against 13 us)
+        if (p.M <= 32 && (p.N + 255) / 256 >= compute_units()) return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
         if (big_tiles < compute_units()) {
             // Fewer big tiles than that: the largest of the small tilings that still gives every compute unit one
             // and a half workgroups (two are resident at a time), else the smallest (1024^3: 64 x 64 tiles 8.8 us,

@@ -40,7 +40,7 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
 def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
     for k in DEPTHS:
         plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
-        _check(m, n, k, plan, k_tile=64, min_k=1024 if m <= 32 else 2048)
+        _check(m, n, k, plan, k_tile=64, min_k=2048)
         if n % 8:
             assert plan[0] == 1, (m, n, k, plan)           # partial products are written four columns at a time
         assert plan[2] in ((128, 64, 32) if plan[0] > 1 else (0,))
