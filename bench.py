@@ -695,6 +695,11 @@ def main():
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(4096, 30522, 768))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
         others.append(res)
+        # a batch of eight rows against a weight matrix: 32 x 256 tiles in slices of K, every compute unit streaming
+        # its share of B
+        res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(8, 8192, 8192))
+        res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
+        others.append(res)
         # a 16-bit weight-gradient shape: 36 tiles of 128 x 128 in seven slices of K
         res, _ = bench_gemm16(4, args.steps, max(args.warmup, SECONDARY_MIN_WARMUP), vendor, shape=(768, 768, 16384))
         res["steps"], res["warmup"] = args.steps, max(args.warmup, SECONDARY_MIN_WARMUP)
