@@ -236,9 +236,14 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
     name = c["name"] if shape is None else "gemm_f16_%dx%dx%d" % (m, n, k)
     if b_row_major:
         name = name.replace("gemm_f16_", "gemm_f16_rowmajorB_")
+    # below the ridge of the roofline (flops per byte of A, B and D under MFMA peak / HBM peak) the bound is HBM
+    nbytes = 2 * (m * k + k * n + m * n)
+    if flops / nbytes < MFMA_PEAK_TFLOPS["f16"] * 1e12 / (HBM_PEAK_GBS * 1e9):
+        roof = _roofline("hbm", nbytes / dev / 1e9, HBM_PEAK_GBS, "GB/s", name)
+    else:
+        roof = _roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", name)
     res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
-               ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
-               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", name),
+               ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets, roofline=roof,
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
