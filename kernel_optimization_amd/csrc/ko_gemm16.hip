@@ -1313,7 +1313,7 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
     const int64_t t64 = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64);
     if (forced >= 2) {
-        set(forced, t128 * forced >= cu / 2 ? 128 : 64);
+        set(forced, p.M <= 32 && p.N >= 256 ? 32 : t128 * forced >= cu / 2 ? 128 : 64);
         return plan;
     }
     const int64_t fit = static_cast<int64_t>(static_cast<double>(workspace_bytes) / out_bytes);  // slices the workspace holds
