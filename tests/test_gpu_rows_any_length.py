@@ -60,7 +60,8 @@ def test_softmax_any_length_leaves_what_lies_behind_the_rows_alone(ko):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("rows,cols", [(5, 1), (64, 3), (1000, 7), (129, 65), (2048, 197), (300, 1004), (17, 4099), (6, 50257)])
+@pytest.mark.parametrize("rows,cols", [(5, 1), (64, 3), (1000, 7), (129, 65), (2048, 197), (300, 1004), (17, 4099), (6, 50257),
+                                       (300, 70001)])
 def test_softmax16_rows_of_any_length(ko, rows, cols, bf16):
     dt = ko.BF16 if bf16 else ko.F16
     xb = _bits(inputs.normal_f32((rows, cols), 720 + cols, 0.0, 4.0), bf16)
@@ -103,7 +104,8 @@ def test_layernorm_rows_of_any_length(ko, rows, cols, affine, unbiased):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("rows,cols", [(64, 3), (1000, 7), (129, 65), (2048, 197), (300, 1004), (17, 4099), (6, 50257)])
+@pytest.mark.parametrize("rows,cols", [(64, 3), (1000, 7), (129, 65), (2048, 197), (300, 1004), (17, 4099), (6, 50257),
+                                       (300, 70001)])
 def test_layernorm16_rows_of_any_length(ko, rows, cols, bf16):
     dt = ko.BF16 if bf16 else ko.F16
     xb = _bits(inputs.normal_f32((rows, cols), 750 + cols, 0.5, 2.0), bf16)
