@@ -618,8 +618,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params whole) 
         if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
     }
 
-    if (p.partial != nullptr) store_partial<WTM, WTN>(p, acc, lane, m0 + wm * WTM, n0 + wn * WTN);
-    else store_tile<WTM, WTN, SWIZZLE, BF16, EDGE>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+    if (p.partial != nullptr) {
+        store_partial<WTM, WTN>(p, acc, lane, m0 + wm * WTM, n0 + wn * WTN);
+    } else if (!EDGE || (m0 + BM <= M && n0 + BN <= N)) {
+        // a tile that lies inside the matrix takes the coalesced epilogue in the edge form of the kernel too (a
+        // ragged K, or the inner tiles of a ragged M or N: 16384 x 3072 x 8 is 100 MB of output and nothing else)
+        store_tile<WTM, WTN, SWIZZLE, BF16, false>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+    } else {
+        store_tile<WTM, WTN, SWIZZLE, BF16, true>(p, acc, lds + wave * (WTM * WTN / 8), lane, m0 + wm * WTM, n0 + wn * WTN);
+    }
 }
 
 // Direct-to-LDS kernels for full tiles with K-contiguous operands (column-major B):

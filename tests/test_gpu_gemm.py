@@ -719,3 +719,23 @@ def test_gemm16_rows_of_c_and_d_off_16_byte_boundaries_whole_output(ko, m, n, k,
         want = exact if c is None else exact + 2.0 * C + bias
         np.testing.assert_array_equal(out[:m * n].reshape(m, n), f16(want))
         assert np.all(out[m * n:] == 0x7e7e)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("m,n,k", [(2048, 1024, 8), (1024, 2048, 40), (4096, 4096, 32), (1300, 2100, 24)])
+def test_gemm16_shallow_k_whole_output(ko, m, n, k, bf16):
+    """K below one K tile (a rank-8 to rank-40 update): the edge form of the register pipeline pads K with zeros, and
+    its tiles that lie inside the matrix take the coalesced epilogue (1300 x 2100 has both kinds of tile).  Small
+    integers: the whole output, with C and a bias, equals the rounded exact result."""
+    rng = np.random.default_rng(m + k)
+    f16 = lambda x: oracle.f64_to_bf16(x) if bf16 else oracle.f64_to_f16(x)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float64)
+    B = rng.integers(-4, 5, (n, k)).astype(np.float64)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float64)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float64)
+    exact = A @ B.T
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16)
+    got = ko.gemm16_host(f16(A), f16(B), m, n, k, **kw)
+    np.testing.assert_array_equal(got, f16(exact))
+    got = ko.gemm16_host(f16(A), f16(B), m, n, k, C_bits=f16(C), alpha=1.0, beta=-1.0, bias_bits=f16(bias), **kw)
+    np.testing.assert_array_equal(got, f16(exact - C + bias))
