@@ -782,6 +782,10 @@ int run(Params p, hipStream_t s, int variant) {
         const bool big = t128 >= cu && 97 * ((t128 + cu - 1) / cu) <= 31 * ((t64 + cu - 1) / cu);
         variant = big ? (k >= 2048 ? 40 : 36)
                       : (2 * t64 <= cu ? 41 : (15 * k_pad256 <= 16 * k_pad128 ? 35 : 33));
+        // a K of one 32-deep K tile or less (a low-rank update: the time is the output's): the register pipeline
+        // takes it as one K tile, the direct-to-LDS kernels pad it to a pair of them (8192 x 3072 x 8: 31 us
+        // against 47 us)
+        if (big && k <= 32) variant = 16;
         // Operand rows off 16-byte boundaries are loaded four bytes per lane, four times as many loads with an
         // address each: the 128 x 128 x 64 form would spill registers there.
         const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&

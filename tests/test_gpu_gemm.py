@@ -739,3 +739,16 @@ def test_gemm16_shallow_k_whole_output(ko, m, n, k, bf16):
     np.testing.assert_array_equal(got, f16(exact))
     got = ko.gemm16_host(f16(A), f16(B), m, n, k, C_bits=f16(C), alpha=1.0, beta=-1.0, bias_bits=f16(bias), **kw)
     np.testing.assert_array_equal(got, f16(exact - C + bias))
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 2304, 8), (4096, 1024, 32), (2100, 2500, 20)])
+def test_sgemm_shallow_k_is_exact_on_small_integers(ko, m, n, k):
+    """A K of one 32-deep K tile or less on enough 128 x 128 tiles to fill the chip goes to the register pipeline
+    (one K tile instead of a padded pair).  Small integers: exact, with alpha, beta and C."""
+    rng = np.random.default_rng(m + k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B), ref)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C)
