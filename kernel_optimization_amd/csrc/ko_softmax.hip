@@ -605,6 +605,15 @@ template <int IO, bool MASKED, bool NT>
 int launch_wave_lpr(const Args<IO> &a, int lpr) {
     const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + lpr - 1) / lpr;
+    if constexpr (!MASKED) {
+        // Rows of one to four vectors (the softmax over 8 or 16 experts for every token): 1, 2 or 4 lanes per row
+        // with one vector each, 16 to 64 rows per wavefront, whose one load still covers a contiguous stretch of
+        // memory ([16777216, 4]: 466 -> 83 us, the time of the same-bytes copy).  More vectors per lane of such
+        // a small group would stride through memory (three vectors of one lane each: [8388608, 12] 236 -> 356 us).
+        if (lpr == 1 && vpl == 1) return launch_wave<IO, 1, 1, false, true>(a);
+        if (lpr == 2 && vpl == 1) return launch_wave<IO, 2, 1, false, true>(a);
+        if (lpr == 4 && vpl == 1) return launch_wave<IO, 4, 1, false, true>(a);
+    }
     switch (lpr) {
         case 8: return launch_wave_vpl<IO, 8, MASKED, NT>(a, vpl);
         case 16: return launch_wave_vpl<IO, 16, MASKED, NT>(a, vpl);
@@ -638,9 +647,10 @@ constexpr int kBlockAutoMaxVecs = 1024 * (96 / Io<IO>::E + 4);
 // row (measured on [786432, 512] binary16, mean valid length 288: 64 x 1 309 us, 32 x 2 230 us).
 int default_lanes_per_row(int nvec, bool masked, int masked_min_vpl) {
     int best = 64, best_waste = 1 << 30;
-    for (int lpr = 8; lpr <= 64; lpr <<= 1) {
+    // (groups of 1, 2 and 4 lanes: without a mask, one vector per lane)
+    for (int lpr = masked ? 8 : 1; lpr <= 64; lpr <<= 1) {
         int vpl = (nvec + lpr - 1) / lpr;
-        if (vpl > 8) continue;
+        if (vpl > (lpr < 8 ? 1 : 8)) continue;
         if (vpl == 5) vpl = 6;
         if (vpl == 7) vpl = 8;
         const int waste = lpr * vpl - nvec;
@@ -658,7 +668,7 @@ int launch_wave_any(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     int lpr = tuning(knob_softmax_lanes_per_row);
     if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec, MASKED, IO == IO_F32 ? 4 : 2);
-    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    while (lpr < 64 && (nvec + lpr - 1) / lpr > (lpr < 8 ? 1 : kWaveMaxVpl)) lpr <<= 1;
     // Streaming (non-temporal) accesses by default: every byte is touched once.  Knob: 2 = off
     // (fp32 storage only; the 16-bit kernels are built with streaming accesses).
     if constexpr (IO == IO_F32) {
@@ -781,6 +791,12 @@ template <int IO, bool MASKED>
 int launch_by_element(const Args<IO> &a) {
     static_assert(Io<IO>::E == 1, "");
     const int cols = a.cols;
+    if constexpr (!MASKED) {  // rows of a few columns: as many lanes as columns, up to 64 rows per wavefront
+        if (cols <= 1) return launch_wave<IO, 1, 1, false, true>(a);
+        if (cols <= 2) return launch_wave<IO, 2, 1, false, true>(a);
+        if (cols <= 4) return launch_wave<IO, 4, 1, false, true>(a);
+        if (cols <= 8) return launch_wave<IO, 8, 1, false, true>(a);
+    }
     if (cols <= 16) return launch_wave<IO, 16, 1, MASKED, true>(a);
     if (cols <= 32) return launch_wave<IO, 16, 2, MASKED, true>(a);
     if (cols <= 64) return launch_wave<IO, 16, 4, MASKED, true>(a);

@@ -170,3 +170,12 @@ def test_rows16_large(ko, bf16):
     y, mean, rstd = ko.layernorm16_host(xb, gb, bb, 1e-5, False, dtype=dt)
     _, ref64, rmean, rrstd = oracle.layernorm16(xb, gb, bb, 1e-5, False, bf16)
     assert_layernorm16_close((_to64(y, bf16), mean, rstd), (ref64, rmean, rrstd), bf16)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("cols", [8, 16, 24, 32, 48, 64, 128])
+def test_softmax16_rows_of_a_few_vectors(ko, cols, bf16):
+    for rows in (1, 63, 64, 65, 5000):
+        xb = _bits(inputs.normal_f32((rows, cols), 950 + rows + cols, 0.0, 4.0), bf16)
+        _, ref64 = oracle.softmax16(xb, bf16=bf16)
+        assert_softmax16_close(_to64(ko.softmax16_host(xb, dtype=ko.BF16 if bf16 else ko.F16), bf16), ref64, bf16)

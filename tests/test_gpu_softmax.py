@@ -217,3 +217,21 @@ def test_masked_softmax_full_size_cfg5(ko):
             blk = yb[i * rows_per_seq:(i + 1) * rows_per_seq]
             assert np.all(blk[:, L:] == 0.0)  # padded columns are exact zeros
             assert blk[:, :L].min() >= 0.0
+
+
+@pytest.mark.parametrize("cols", [4, 8, 12, 16, 20, 24, 28, 32, 36, 48, 64])
+def test_softmax_rows_of_a_few_vectors(ko, cols):
+    """Rows of one to sixteen vectors (the softmax over 8 or 16 experts for every token): 1, 2 or 4 lanes per row, 16 to
+    64 rows per wavefront; row counts around a wavefront's worth, and special values."""
+    for rows in (1, 15, 16, 17, 63, 64, 65, 1000, 100001):
+        x = inputs.normal_f32((rows, cols), 900 + rows + cols, 0.0, 4.0)
+        assert_softmax_close(ko.softmax_host(x), oracle.softmax(x))
+    x = inputs.normal_f32((777, cols), 901, 0.0, 4.0)
+    assert_softmax_close(ko.softmax_host(x, in_place=True), oracle.softmax(x))
+    import special_values as sv
+    base = inputs.normal_f32((5, cols), 902 + cols, 0.0, 4.0)
+    xs, classes = sv.build(sv.SOFTMAX_ROWS, cols, base, repeat=11)
+    ref = oracle.softmax(xs)
+    got = ko.softmax_host(xs)
+    ok = sv.check_rows(got, ref, classes, "softmax cols %d" % cols)
+    assert_softmax_close(got[ok], ref[ok])
