@@ -854,6 +854,11 @@ template <int IO>
 int launch_wave_lpr(const Args<IO> &a, int lpr) {
     const int nvec = a.cols / Io<IO>::E;
     const int vpl = (nvec + lpr - 1) / lpr;
+    // rows of one to four vectors: 1, 2 or 4 lanes per row with one vector each, 16 to 64 rows per wavefront, one
+    // load of which still covers a contiguous stretch of memory
+    if (vpl == 1 && lpr == 1) return launch_wave<IO, 1, 1>(a);
+    if (vpl == 1 && lpr == 2) return launch_wave<IO, 2, 1>(a);
+    if (vpl == 1 && lpr == 4) return launch_wave<IO, 4, 1>(a);
     switch (lpr) {
         case 8: return launch_wave_vpl<IO, 8>(a, vpl);
         case 16: return launch_wave_vpl<IO, 16>(a, vpl);
@@ -876,9 +881,9 @@ constexpr int kBlockMaxVecs = 1024 * (80 / Io<IO>::E);  // in registers; BLOCK t
 // of the group then covers the longest contiguous piece of the row.
 int default_lanes_per_row(int nvec) {
     int best = 64, best_waste = 1 << 30;
-    for (int lpr = 8; lpr <= 64; lpr <<= 1) {
+    for (int lpr = 1; lpr <= 64; lpr <<= 1) {  // (groups of 1, 2 and 4 lanes: one vector per lane)
         int vpl = (nvec + lpr - 1) / lpr;
-        if (vpl > 8) continue;
+        if (vpl > (lpr < 8 ? 1 : 8)) continue;
         if (vpl == 5) vpl = 6;
         if (vpl == 7) vpl = 8;
         const int waste = lpr * vpl - nvec;
@@ -895,7 +900,7 @@ int launch_wave_any(const Args<IO> &a) {
     const int nvec = a.cols / Io<IO>::E;
     int lpr = tuning(knob_layernorm_lanes_per_row);
     if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = default_lanes_per_row(nvec);
-    while (lpr < 64 && (nvec + lpr - 1) / lpr > kWaveMaxVpl) lpr <<= 1;
+    while (lpr < 64 && (nvec + lpr - 1) / lpr > (lpr < 8 ? 1 : kWaveMaxVpl)) lpr <<= 1;
     return launch_wave_lpr<IO>(a, lpr);
 }
 
@@ -1047,6 +1052,10 @@ template <int IO>
 int launch_by_element(const Args<IO> &a) {
     static_assert(Io<IO>::E == 1, "");
     const int cols = a.cols;
+    if (cols <= 1) return launch_wave_full<IO, 1, 1, false>(a);  // rows of a few columns: as many lanes as columns
+    if (cols <= 2) return launch_wave_full<IO, 2, 1, false>(a);
+    if (cols <= 4) return launch_wave_full<IO, 4, 1, false>(a);
+    if (cols <= 8) return launch_wave_full<IO, 8, 1, false>(a);
     if (cols <= 16) return launch_wave_full<IO, 16, 1, false>(a);
     if (cols <= 32) return launch_wave_full<IO, 16, 2, false>(a);
     if (cols <= 64) return launch_wave_full<IO, 16, 4, false>(a);

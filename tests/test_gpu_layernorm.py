@@ -142,3 +142,17 @@ def test_layernorm_full_size_cfg2(ko):
     assert_layernorm_close(got, oracle.layernorm(x, g, b, eps=1e-5))
     hostg = inputs.normal_f32((cols,), inputs.tensor_seed(2, 1), 1.0, 0.1)
     assert np.all(np.abs(hostg - g) <= 2.0 ** -22 * np.maximum(np.abs(hostg), 1.0))
+
+
+@pytest.mark.parametrize("affine", [True, False])
+@pytest.mark.parametrize("cols", [4, 8, 12, 16, 20, 32, 48, 64])
+def test_layernorm_rows_of_a_few_vectors(ko, cols, affine):
+    """Rows of one to sixteen vectors: 1, 2 or 4 lanes per row up to four vectors, 16 to 64 rows per wavefront; row
+    counts around a wavefront's worth, both variance divisors, in place."""
+    g = inputs.normal_f32((cols,), 961, 1.0, 0.1) if affine else None
+    b = inputs.normal_f32((cols,), 962, 0.0, 0.1) if affine else None
+    for rows in (1, 15, 16, 17, 63, 64, 65, 1000, 100001):
+        x = inputs.normal_f32((rows, cols), 960 + rows + cols, 0.5, 2.0)
+        assert_layernorm_close(ko.layernorm_host(x, g, b, 1e-5, rows % 2 == 0), oracle.layernorm(x, g, b, 1e-5, rows % 2 == 0))
+    x = inputs.normal_f32((777, cols), 963, 0.5, 2.0)
+    assert_layernorm_close(ko.layernorm_host(x, g, b, in_place=True), oracle.layernorm(x, g, b))
