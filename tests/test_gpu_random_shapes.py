@@ -65,3 +65,47 @@ def test_rows16_random_shapes(ko, rows, cols, bf16):
     _, ref64, rmean, rrstd = oracle.layernorm16(xb, gb, None, 1e-5, False, bf16)
     y, mean, rstd = ko.layernorm16_host(xb, gb, None, 1e-5, False, dtype=dt)
     assert_layernorm16_close((_to64(y, bf16), mean, rstd), (ref64, rmean, rrstd), bf16)
+
+
+def _gemm_shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        m = int(np.exp(rng.uniform(0, np.log(6000))))
+        n = int(np.exp(rng.uniform(0, np.log(6000))))
+        k = 8 * int(np.exp(rng.uniform(0, np.log(1024))))
+        if m * n <= 6_000_000 and (m + n) * k <= 12_000_000:
+            out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k", _gemm_shapes(4, 30))
+def test_gemm16_random_shapes_are_exact_on_small_integers(ko, m, n, k):
+    """Random M, N and K (a multiple of 8), both layouts of B, binary16 and bfloat16 by turns, with C and a bias:
+    small integers, so the whole output equals the exact result rounded once."""
+    bf16 = bool((m + n) % 2)
+    b_col_major = bool(k // 8 % 2)
+    rng = np.random.default_rng(m * 7 + n)
+    f16 = lambda x: oracle.f64_to_bf16(x) if bf16 else oracle.f64_to_f16(x)
+    A = rng.integers(-2, 3, (m, k)).astype(np.float64)
+    B = rng.integers(-2, 3, (n, k)).astype(np.float64)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float64)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float64)
+    exact = A @ B.T
+    Bm = B if b_col_major else np.ascontiguousarray(B.T)
+    kw = dict(b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR, dtype=ko.BF16 if bf16 else ko.F16)
+    np.testing.assert_array_equal(ko.gemm16_host(f16(A), f16(Bm), m, n, k, **kw), f16(exact))
+    got = ko.gemm16_host(f16(A), f16(Bm), m, n, k, C_bits=f16(C), alpha=1.0, beta=-1.0, bias_bits=f16(bias), **kw)
+    np.testing.assert_array_equal(got, f16(exact - C + bias))
+
+
+@pytest.mark.parametrize("m,n,k", _gemm_shapes(5, 30))
+def test_sgemm_random_shapes_are_exact_on_small_integers(ko, m, n, k):
+    k = max(1, k // 8 * (1 + m % 8) // 1) if m % 3 else k + m % 5   # not only multiples of 8
+    rng = np.random.default_rng(m * 11 + n)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    C = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B), ref)
+    np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C)
