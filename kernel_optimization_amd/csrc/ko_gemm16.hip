@@ -129,7 +129,8 @@ struct Params {
     int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
     int ldb;                    // row-major B: elements between its rows (N, or more likewise)
     // K slices (gemm16_kernel only): workgroups with blockIdx.y = s multiply k in [s * k_slice, (s + 1) * k_slice) and
-    // write their M x N partial product as fp32 (no alpha, C, bias or activation) behind partial + s * M * N
+    // write their M x N partial product as fp32 (no alpha, C, bias or activation; rows partial_ld(N) floats apart)
+    // behind partial + s * M * partial_ld(N)
     int k_slice;                // 0: no slices
     float *partial;
     int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
@@ -373,6 +374,10 @@ __device__ __forceinline__ u32x4 read_b_transposed(const u32x4 *sb, int k0, int 
     return __builtin_bit_cast(u32x4, static_cast<short8v>(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7)));
 }
 
+// Floats between rows of a partial product: N rounded up to whole groups of four columns, so that every group a
+// lane holds is stored and fetched as one aligned 16-byte access whatever N is.
+__host__ __device__ __forceinline__ int64_t partial_ld(int n) { return (static_cast<int64_t>(n) + 3) & ~int64_t{3}; }
+
 // The problem a workgroup of a K-sliced launch works on: its K range of A and B, its own partial product.
 template <bool B_ROW_MAJOR>
 __device__ __forceinline__ Params slice_of(Params p) {
@@ -381,14 +386,14 @@ __device__ __forceinline__ Params slice_of(Params p) {
         const int k0 = s * p.k_slice;
         p.A += k0;
         p.B += B_ROW_MAJOR ? static_cast<int64_t>(k0) * p.ldb : static_cast<int64_t>(k0);
-        p.partial += static_cast<int64_t>(s) * p.M * p.N;
+        p.partial += static_cast<int64_t>(s) * p.M * partial_ld(p.N);
         p.K = p.K - k0 < p.k_slice ? p.K - k0 : p.k_slice;
     }
     return p;
 }
 
-// One wave's accumulator tile as fp32 into a partial product (rows of N floats; N a multiple of 4, so a lane's four
-// consecutive columns are inside the matrix together or not at all).
+// One wave's accumulator tile as fp32 into a partial product.  A lane's four consecutive columns start at a
+// multiple of 4: a group that starts inside the matrix ends inside the padded row.
 template <int WTM, int WTN>
 __device__ __forceinline__ void store_partial(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], int lane, int row0,
                                               int col0) {
@@ -405,10 +410,13 @@ __device__ __forceinline__ void store_partial(const Params &p, float16v (&acc)[W
                 const int n = col0 + j * 32 + 8 * q + 4 * fhalf;
                 if (n >= p.N) continue;
                 const float4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                *reinterpret_cast<float4v *>(p.partial + static_cast<int64_t>(m) * p.N + n) = v;
+                *reinterpret_cast<float4v *>(p.partial + m * partial_ld(p.N) + n) = v;
             }
     }
 }
+
+// Sixteen bytes of zeros in device memory: what a load fetches in place of a chunk that lies past the end of K.
+__device__ __attribute__((aligned(16))) const uint32_t zero_chunk16[4] = {0u, 0u, 0u, 0u};
 
 template <class T, bool BF16, bool B_ROW_MAJOR, bool EDGE>
 __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params whole) {
@@ -450,65 +458,110 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_kernel(const Params whole) 
     constexpr int ROWS_PER_ITER = THREADS / kChunks;  // rows covered by one load instruction of the workgroup
     const uint32_t lane_off_a = static_cast<uint32_t>((tid / kChunks) * ldk + (tid % kChunks) * 8) * 2u;
 
-    auto load_global = [&](int kt, auto slot) {
-        constexpr int S = decltype(slot)::value;
-        const int k0 = kt * kBK;
+    // EDGE: no load sits under a per-lane branch - the compiler could not count the loads in flight behind one
+    // and would wait for all of them, the tile fetched ahead included, before it touches the older set.  Each
+    // lane keeps the addresses of its chunks of K tile 0, rows past M or N clamped to the last one (they feed
+    // outputs that are never stored); in the last K tile the chunks at or past K are fetched from a chunk of
+    // zeros instead (a select of the address, not a branch).
+    // Row-major B: a chunk of eight columns that begins past N starts at column 0 instead, and one that ends past
+    // N is fetched whole where the next row of B lies behind it - columns past N of B only reach columns past N
+    // of D.  That needs a row of at least eight columns and is not done in the last K tile, whose elements are
+    // fetched one by one, again from zeros where they lie past N or K; shorter rows go that way in every K tile.
+    // (the chunk of zeros and the operands are both global memory: said in the pointer type, or the loads become
+    // flat ones, which also count as LDS operations)
+    typedef const __attribute__((address_space(1))) u32x4 *global_chunk_t;
+    typedef const __attribute__((address_space(1))) uint16_t *global_elem_t;
+    typedef const __attribute__((address_space(1))) u32x4_rows *global_rows_t;
+    const uint16_t *edge_a[EDGE ? A_ITERS : 1], *edge_b[EDGE ? B_ITERS : 1];
+    const uint16_t *const zeros = reinterpret_cast<const uint16_t *>(&zero_chunk16);
+    const bool past_k_last = (tid % kChunks) * 8 >= K - (KT - 1) * kBK;  // this lane's chunk of the last K tile (A, column-major B)
+    if constexpr (EDGE) {
 #pragma unroll
         for (int i = 0; i < A_ITERS; ++i) {
             const int idx = tid + i * THREADS;
-            const int row = idx / kChunks, c = idx % kChunks;
-            int gr = m0 + row;
-            const int kc = k0 + c * 8;
-            if constexpr (EDGE) {
-                gr = gr < M ? gr : M - 1;  // rows past the edge re-read the last row; their results are never stored
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.A + static_cast<int64_t>(gr) * ldk + kc);
-                ra[S][i] = v;
+            const int gr = m0 + idx / kChunks;
+            edge_a[i] = p.A + static_cast<int64_t>(gr < M ? gr : M - 1) * ldk + (idx % kChunks) * 8;
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITERS; ++i) {
+            const int idx = tid + i * THREADS;
+            if constexpr (B_ROW_MAJOR) {
+                constexpr int NCH = BN / 8;
+                const int gn = n0 + (idx % NCH) * 8;
+                edge_b[i] = p.B + static_cast<int64_t>(idx / NCH) * p.ldb + (gn < N ? gn : 0);
             } else {
-                const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + i * ROWS_PER_ITER) * ldk + k0);
-                ra[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
+                const int gr = n0 + idx / kChunks;
+                edge_b[i] = p.B + static_cast<int64_t>(gr < N ? gr : N - 1) * ldk + (idx % kChunks) * 8;
             }
         }
-        if constexpr (!B_ROW_MAJOR) {
+    }
+    // The addresses run along with the K tile they point at, in their own registers: an address formed in a
+    // temporary per load would take the registers of a load still in flight and wait for it.
+    int edge_kt = 0;                                  // the K tile edge_a and edge_b point at
+    const bool whole_chunks = !B_ROW_MAJOR || N >= 8; // K tiles before the last one need no per-lane care
+
+    auto load_global = [&](int kt, auto slot) {
+        constexpr int S = decltype(slot)::value;
+        const int k0 = kt * kBK;
+        if constexpr (EDGE) {
+            const int64_t ahead = static_cast<int64_t>(kt - edge_kt) * kBK;  // wave-uniform; K tiles are asked for in rising order
+            edge_kt = kt;
+            const bool last = kt == KT - 1;  // wave-uniform
+            // in the last K tile (which may be asked for again, never left) the chunks at or past K turn to the zeros
+            const bool to_zeros = last && past_k_last;
+#pragma unroll
+            for (int i = 0; i < A_ITERS; ++i) edge_a[i] = to_zeros ? zeros : edge_a[i] + ahead;
 #pragma unroll
             for (int i = 0; i < B_ITERS; ++i) {
-                const int idx = tid + i * THREADS;
-                const int row = idx / kChunks, c = idx % kChunks;
-                int gr = n0 + row;
-                const int kc = k0 + c * 8;
-                if constexpr (EDGE) {
-                    gr = gr < N ? gr : N - 1;
-                    u32x4 v = {0u, 0u, 0u, 0u};
-                    if (kc < K) v = *reinterpret_cast<const u32x4 *>(p.B + static_cast<int64_t>(gr) * ldk + kc);
-                    rb[S][i] = v;
-                } else {
-                    const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + i * ROWS_PER_ITER) * ldk + k0);
-                    rb[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
+                if constexpr (B_ROW_MAJOR) edge_b[i] += ahead * p.ldb;
+                else edge_b[i] = to_zeros ? zeros : edge_b[i] + ahead;
+            }
+            if constexpr (B_ROW_MAJOR) {
+                // both sides of this branch issue their loads unmasked, so the loads in flight can still be counted
+                if (!last && whole_chunks) {
+#pragma unroll
+                    for (int i = 0; i < A_ITERS; ++i) ra[S][i] = *(global_chunk_t)edge_a[i];
+#pragma unroll
+                    for (int i = 0; i < B_ITERS; ++i) rb[S][i] = *(global_rows_t)edge_b[i];
+                    return;
                 }
             }
-        } else {
-            // B[k][n] row-major: a chunk is 8 consecutive n of one k.
+#pragma unroll
+            for (int i = 0; i < A_ITERS; ++i) ra[S][i] = *(global_chunk_t)edge_a[i];
 #pragma unroll
             for (int i = 0; i < B_ITERS; ++i) {
+                if constexpr (!B_ROW_MAJOR) {
+                    rb[S][i] = *(global_chunk_t)edge_b[i];
+                } else {
+                    const int idx = tid + i * THREADS;
+                    constexpr int NCH = BN / 8;
+                    const int gk = k0 + idx / NCH;
+                    const int gn = n0 + (idx % NCH) * 8;
+                    const uint16_t *src = p.B + static_cast<int64_t>(gk) * p.ldb + gn;
+                    uint32_t t[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = *(global_elem_t)(gk < K && gn + e < N ? src + e : zeros);
+                    rb[S][i] = u32x4{t[0] | (t[1] << 16), t[2] | (t[3] << 16), t[4] | (t[5] << 16), t[6] | (t[7] << 16)};
+                }
+            }
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < A_ITERS; ++i) {
+            const char *base = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + i * ROWS_PER_ITER) * ldk + k0);
+            ra[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITERS; ++i) {
+            if constexpr (!B_ROW_MAJOR) {
+                const char *base = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + i * ROWS_PER_ITER) * ldk + k0);
+                rb[S][i] = *reinterpret_cast<const u32x4 *>(base + lane_off_a);
+            } else {
+                // B[k][n] row-major: a chunk is 8 consecutive n of one k; rows of B may start at any element (ldb
+                // not a multiple of 8)
                 const int idx = tid + i * THREADS;
                 constexpr int NCH = BN / 8;
-                const int kr = idx / NCH, c = idx % NCH;
-                const int gk = k0 + kr;
-                const int gn = n0 + c * 8;
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (!EDGE || gk < K) {
-                    const uint16_t *src = p.B + static_cast<int64_t>(gk) * p.ldb + gn;
-                    if (!EDGE || gn + 8 <= N) {  // rows of B may start at any element (ldb not a multiple of 8)
-                        v = *reinterpret_cast<const u32x4_rows *>(src);
-                    } else {
-                        uint16_t t[8];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) t[e] = gn + e < N ? src[e] : static_cast<uint16_t>(0);
-                        v = u32x4{t[0] | (uint32_t(t[1]) << 16), t[2] | (uint32_t(t[3]) << 16),
-                                  t[4] | (uint32_t(t[5]) << 16), t[6] | (uint32_t(t[7]) << 16)};
-                    }
-                }
-                rb[S][i] = v;
+                rb[S][i] = *reinterpret_cast<const u32x4_rows *>(p.B + static_cast<int64_t>(k0 + idx / NCH) * p.ldb + n0 + (idx % NCH) * 8);
             }
         }
     };
@@ -823,7 +876,6 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
     else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
-__device__ __attribute__((aligned(16))) const uint32_t zero_chunk16[4] = {0u, 0u, 0u, 0u};
 
 // EDGE_K: K is any multiple of 8 and is padded with zeros up to the next multiple of 128 - a lane whose
 // 16-byte chunk (or, for a row-major B, whose row) lies at or past K fetches 16 zero bytes instead, chosen per
@@ -1253,16 +1305,18 @@ int launch_direct(const Params &p, hipStream_t stream) {
 }
 
 // D = act(alpha * (P_0 + ... + P_{slices-1}) + beta * C + bias), rounded once, from the fp32 partial products of a
-// K-sliced launch, summed in slice order.  One thread per four consecutive columns.
+// K-sliced launch, summed in slice order.  One thread per four consecutive columns; the last group of a row whose
+// length is not a multiple of 4 finishes its columns one by one.
 template <bool BF16>
 __global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, int slices) {
     typedef float float4v __attribute__((ext_vector_type(4)));
-    const int groups_per_row = p.N / 4;
+    const int64_t ldp = partial_ld(p.N);
+    const int groups_per_row = static_cast<int>(ldp / 4);
     const int64_t g = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
     if (g >= static_cast<int64_t>(p.M) * groups_per_row) return;
     const int m = static_cast<int>(g / groups_per_row), n = static_cast<int>(g % groups_per_row) * 4;
-    const int64_t count = static_cast<int64_t>(p.M) * p.N;
-    const float *src = p.partial + static_cast<int64_t>(m) * p.N + n;
+    const int64_t count = p.M * ldp;
+    const float *src = p.partial + m * ldp + n;
     float4v acc = *reinterpret_cast<const float4v *>(src);
     int s = 1;
     for (; s + 8 <= slices; s += 8) {
@@ -1275,15 +1329,29 @@ __global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, i
     for (; s < slices; ++s) acc += *reinterpret_cast<const float4v *>(src + s * count);
     const bool use_c = p.C != nullptr && p.beta != 0.0f;
     const int64_t off = static_cast<int64_t>(m) * p.ldd + n;
-    u32x2 c2 = {0, 0}, b2 = {0, 0};
-    if (use_c) c2 = *reinterpret_cast<const u32x2 *>(p.C + off);
-    if (p.bias) b2 = *reinterpret_cast<const u32x2 *>(p.bias + n);
     float v[4] = {acc[0], acc[1], acc[2], acc[3]};
-    finish4<BF16>(p, v, c2, b2, use_c);
-    u32x2 o;
-    o[0] = pack2<BF16>(v[0], v[1]);
-    o[1] = pack2<BF16>(v[2], v[3]);
-    *reinterpret_cast<u32x2 *>(p.D + off) = o;
+    if (n + 3 < p.N) {
+        u32x2 c2 = {0, 0}, b2 = {0, 0};
+        if (use_c) c2 = *reinterpret_cast<const u32x2_rows *>(p.C + off);
+        if (p.bias) b2 = *reinterpret_cast<const u32x2_rows *>(p.bias + n);
+        finish4<BF16>(p, v, c2, b2, use_c);
+        u32x2 o;
+        o[0] = pack2<BF16>(v[0], v[1]);
+        o[1] = pack2<BF16>(v[2], v[3]);
+        *reinterpret_cast<u32x2_rows *>(p.D + off) = o;
+    } else {
+        u32x2 c2 = {0, 0}, b2 = {0, 0};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (n + e >= p.N) continue;
+            if (use_c) c2[e >> 1] |= static_cast<uint32_t>(p.C[off + e]) << ((e & 1) * 16);
+            if (p.bias) b2[e >> 1] |= static_cast<uint32_t>(p.bias[n + e]) << ((e & 1) * 16);
+        }
+        finish4<BF16>(p, v, c2, b2, use_c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) p.D[off + e] = from_float<BF16>(v[e]);
+    }
 }
 
 // K slices for a deep K on few output tiles (weight-gradient shapes: 768 x 768 x 16384 is 36 tiles of 128 x 128).
@@ -1305,9 +1373,9 @@ struct SlicePlan16 {
 SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     SlicePlan16 plan;
     const int forced = tuning(knob_gemm16_k_slices);
-    if (forced == 1 || p.N % 8 != 0 || p.ldd % 4 != 0) return plan;
+    if (forced == 1) return plan;
     const int64_t cu = compute_units();
-    const double out_bytes = 4.0 * p.M * p.N;
+    const double out_bytes = 4.0 * p.M * partial_ld(p.N);  // of one partial product
     auto set = [&](int64_t slices, int tile) {
         if (slices < 2) return;
         const int64_t depth = ((p.K + slices - 1) / slices + kBK - 1) / kBK * kBK;
@@ -1356,7 +1424,7 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
              : plan.tile == 32 ? launch<TileSkinny, BF16, B_ROW_MAJOR>(part, stream)
                                : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
     if (st != KO_OK) return st;
-    const int64_t groups = static_cast<int64_t>(p.M) * (p.N / 4);
+    const int64_t groups = p.M * (partial_ld(p.N) / 4);
     gemm16_slices_sum_kernel<BF16><<<dim3(static_cast<unsigned>((groups + 63) / 64)), dim3(64), 0, stream>>>(part, plan.slices);
     KO_CHECK_LAUNCH();
     return KO_OK;

@@ -691,9 +691,9 @@ int launch_direct(Params p, hipStream_t stream) {
     // Operand rows have to start on 16-byte boundaries and K must not end inside a 16-byte chunk.
     const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                          p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
-    if (!aligned && p.k_slice > 0) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: K slices need 16-byte aligned operand rows");
-    if (!aligned && tuning(knob_sgemm_unaligned) == 1) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
-    // K-sliced launches: every slice but the last is k_slice deep (a multiple of 4), the last takes the rest.
+    if (!aligned && p.k_slice == 0 && tuning(knob_sgemm_unaligned) == 1) return launch<BM, BN, FALLBACK_BK, WAVES_M, WAVES_N, KSPLIT, true>(p, stream);
+    // K-sliced launches: every slice but the last is k_slice deep (a multiple of 4, so aligned operand rows stay
+    // aligned in every slice), the last takes the rest.
     const int slices = p.k_slice > 0 ? (p.K + p.k_slice - 1) / p.k_slice : 1;
     const int k_last = p.K - (slices - 1) * (p.k_slice > 0 ? p.k_slice : 0);
     const int k_each = slices > 1 ? p.k_slice : p.K;
@@ -718,40 +718,48 @@ int launch_direct(Params p, hipStream_t stream) {
 
 // D = alpha * (P_0 + P_1 + ... + P_{slices-1}) + beta * C over the M x N partial products a K-sliced launch
 // left behind `partials`, summed in slice order whatever order the slices finished in.
-// One 64-lane workgroup per 256 (VEC) or 64 outputs: the problems that are sliced have few outputs, and small
+// One 64-lane workgroup per 256 outputs: the problems that are sliced have few outputs, and small
 // workgroups spread them over more compute units.  The partial products of eight slices are fetched together
 // (they come from memory behind the L2s: another XCD wrote them) and added one after the other.
-template <bool VEC>
 __global__ __launch_bounds__(64) void sgemm_slices_sum_kernel(const float *__restrict__ partials, int slices,
                                                               int64_t count, float alpha, float beta,
                                                               const float *C, float *D) {  // C may be D
-    constexpr int W = VEC ? 4 : 1;
-    typedef float vec_t __attribute__((ext_vector_type(W)));
-    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x) * W;
+    // four floats that start on any 4-byte boundary (an odd M x N puts every other partial product off the
+    // 16-byte grid): still one access each
+    typedef float vec_t __attribute__((ext_vector_type(4)));
+    typedef vec_t vec_any_t __attribute__((aligned(4)));
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x) * 4;
     if (i >= count) return;
     const float *src = partials + i;
-    vec_t acc = *reinterpret_cast<const vec_t *>(src);
-    int s = 1;
-    for (; s + 8 <= slices; s += 8) {
-        vec_t v[8];
+    if (i + 4 <= count) {
+        vec_t acc = *reinterpret_cast<const vec_any_t *>(src);
+        int s = 1;
+        for (; s + 8 <= slices; s += 8) {
+            vec_t v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const vec_t *>(src + (s + j) * count);
+            for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const vec_any_t *>(src + (s + j) * count);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc += v[j];
+            for (int j = 0; j < 8; ++j) acc += v[j];
+        }
+        for (; s < slices; ++s) acc += *reinterpret_cast<const vec_any_t *>(src + s * count);
+        acc *= alpha;
+        if (C != nullptr && beta != 0.0f) acc += beta * *reinterpret_cast<const vec_any_t *>(C + i);
+        __builtin_nontemporal_store(acc, reinterpret_cast<vec_any_t *>(D + i));
+    } else {
+        for (int64_t e = i; e < count; ++e) {  // the last one to three outputs
+            float acc = partials[e];
+            for (int s = 1; s < slices; ++s) acc += partials[e + s * count];
+            acc *= alpha;
+            if (C != nullptr && beta != 0.0f) acc += beta * C[e];
+            D[e] = acc;
+        }
     }
-    for (; s < slices; ++s) acc += *reinterpret_cast<const vec_t *>(src + s * count);
-    acc *= alpha;
-    if (C != nullptr && beta != 0.0f) acc += beta * *reinterpret_cast<const vec_t *>(C + i);
-    __builtin_nontemporal_store(acc, reinterpret_cast<vec_t *>(D + i));
 }
 
 int sum_slices(const float *partials, int slices, const Params &p, hipStream_t stream) {
     const int64_t count = static_cast<int64_t>(p.M) * p.N;
-    const bool vec = count % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.C) | reinterpret_cast<uintptr_t>(p.D)) & 15) == 0;
-    const int64_t threads = vec ? count / 4 : count;
-    const dim3 grid(static_cast<unsigned>((threads + 63) / 64));
-    if (vec) sgemm_slices_sum_kernel<true><<<grid, 64, 0, stream>>>(partials, slices, count, p.alpha, p.beta, p.C, p.D);
-    else sgemm_slices_sum_kernel<false><<<grid, 64, 0, stream>>>(partials, slices, count, p.alpha, p.beta, p.C, p.D);
+    const dim3 grid(static_cast<unsigned>(((count + 3) / 4 + 63) / 64));
+    sgemm_slices_sum_kernel<<<grid, 64, 0, stream>>>(partials, slices, count, p.alpha, p.beta, p.C, p.D);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
@@ -808,7 +816,7 @@ int run(Params p, hipStream_t s, int variant) {
 
 // K slices.  The slices are workgroups of one launch (blockIdx.y); their partial products go to a workspace and
 // a second kernel sums them in slice order, so the result does not depend on which slice finished first.
-// Operands must be as the direct-to-LDS kernels want them (rows on 16-byte boundaries).  Two cases:
+// Two cases:
 //   - few output tiles (tiles for at most half of the compute units, 256 x 256 x 2048: 32 tiles of 32 x 64 on 256
 //     CUs) and K >= 768: as many slices as bring the launch up to one workgroup per compute unit, each at
 //     least 256 deep and a multiple of 128 (whole pairs of K tiles); the tiling as for the unsliced problem;
@@ -827,9 +835,10 @@ SlicePlan plan_k_slices(const Params &p, size_t workspace_bytes) {
     SlicePlan plan;
     const int forced = tuning(knob_sgemm_k_slices);
     if (forced == 1) return plan;
+    // operand rows off 16-byte boundaries: the same plans (the four-byte loads make every tiling slower by about
+    // the same factor), without the 128 x 128 x 64 form
     const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                          p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
-    if (!aligned) return plan;
     const int64_t cu = compute_units();
     const int64_t t64 = ((p.M + 63) / 64) * ((p.N + 63) / 64);
     auto set = [&](int64_t slices, int variant) {
@@ -882,7 +891,9 @@ SlicePlan plan_k_slices(const Params &p, size_t workspace_bytes) {
             if (us < best_sliced) {
                 best_sliced = us;
                 best_slices = slices;
-                best_variant = t.variant != 0 ? t.variant : t.bm == 128 ? (depth >= 2048 ? 40 : 36) : (depth % 256 == 0 ? 35 : 33);
+                best_variant = t.variant != 0 ? t.variant
+                               : t.bm == 128  ? (depth >= 2048 && aligned ? 40 : 36)
+                                              : (depth % 256 == 0 ? 35 : 33);
             }
         }
     }

@@ -12,11 +12,11 @@ import pytest
 import kernel_optimization_amd as ko
 
 WORKSPACE = 32 << 20
-SIZES = [8, 32, 64, 100, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
+SIZES = [8, 31, 32, 64, 100, 107, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
 DEPTHS = [64, 512, 767, 768, 1300, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
 
 
-def _check(m, n, k, plan, k_tile, min_k):
+def _check(m, n, k, plan, k_tile, min_k, row_pad=1):
     slices, k_slice, _ = plan
     assert slices >= 1
     if slices == 1:
@@ -24,7 +24,7 @@ def _check(m, n, k, plan, k_tile, min_k):
     assert k >= min_k, (m, n, k, plan)
     assert k_slice > 0 and k_slice % k_tile == 0, (m, n, k, plan)
     assert (slices - 1) * k_slice < k <= slices * k_slice, (m, n, k, plan)   # no empty slice, none missing
-    assert slices * m * n * 4 <= WORKSPACE, (m, n, k, plan)
+    assert slices * m * (-(-n // row_pad) * row_pad) * 4 <= WORKSPACE, (m, n, k, plan)
 
 
 @pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
@@ -34,15 +34,14 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
         _check(m, n, k, plan, k_tile=128, min_k=768)
         if plan[0] > 1 and plan[2]:
             assert plan[2] in (33, 35, 36, 40), plan       # the direct-to-LDS tilings
+            assert plan[2] != 40 or (n % 4 == 0 and k % 4 == 0), plan   # not with four-byte operand loads
 
 
 @pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
 def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
     for k in DEPTHS:
         plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
-        _check(m, n, k, plan, k_tile=64, min_k=2048)
-        if n % 8:
-            assert plan[0] == 1, (m, n, k, plan)           # partial products are written four columns at a time
+        _check(m, n, k, plan, k_tile=64, min_k=2048, row_pad=4)   # rows of partial products: whole groups of 4
         assert plan[2] in ((128, 64, 32) if plan[0] > 1 else (0,))
         if plan[2] == 32:
             assert m <= 32
@@ -59,6 +58,9 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (4, 2048, 64)
     assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
     assert ko.gemm_plan(16384, 3072, 768, sixteen_bit=True)[0] == 1
+    # operand rows off 16-byte boundaries are sliced like the others
+    assert ko.gemm_plan(282, 31, 13104)[0] > 1
+    assert ko.gemm_plan(282, 31, 13104, sixteen_bit=True)[0] > 1
 
 
 def test_bad_arguments_are_refused():

@@ -84,7 +84,9 @@ def sgemm_k_slices(ko):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 256, 2048), (128, 64, 4096), (100, 200, 3000), (33, 68, 1300), (512, 512, 8192),
-                                   (64, 64, 516), (1, 4, 16384), (320, 192, 1024)])
+                                   (64, 64, 516), (1, 4, 16384), (320, 192, 1024),
+                                   # operand rows off 16-byte boundaries (four-byte loads) and an M x N that is no multiple of 4
+                                   (282, 31, 13104), (48, 107, 7144), (100, 201, 3001), (16, 1001, 4008), (339, 670, 6784)])
 def test_sgemm_deep_k_on_few_tiles_is_cut_into_slices(ko, sgemm_k_slices, m, n, k):
     """Few output tiles and a deep K: the default dispatch cuts K into slices that run as workgroups of one
     launch and sums their partial products in a second kernel.  Small integers make every product and sum
@@ -536,6 +538,9 @@ def test_gemm16_bias_activation(ko, act, bf16, b_col_major, m, n, k):
 @pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k,slices", [(512, 512, 8192, 0), (256, 384, 2048, 3), (300, 520, 1096, 2), (768, 768, 4096, 7),
                                           (130, 72, 4104, 5),
+                                          # rows of D off 8-byte boundaries, a ragged last group of four columns
+                                          (282, 31, 13104, 0), (48, 107, 7144, 0), (130, 75, 4104, 5), (16, 1001, 4008, 0),
+                                          (339, 670, 6784, 0), (33, 2, 2048, 3),
                                           # at most 32 rows: 32 x 256 tiles, slices chosen by the planner
                                           (8, 4096, 4096, 0), (1, 512, 8192, 0), (32, 264, 2120, 0), (20, 1000, 2048, 0)])
 def test_gemm16_k_slices(ko, m, n, k, slices, b_col_major, bf16):
