@@ -1404,7 +1404,9 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
         if (skinny <= cu) set(capped(2 * cu / skinny, 256), 32);
         if (plan.slices > 1) return plan;
     }
-    if (p.K < 2048) return plan;
+    // (few tiles: from K = 1536 on - 128 x 128 x 1536 9.9 us whole, 8.7 in three slices; 100 x 100 x 1536 13.2 and
+    // 9.1; at K = 1024 the second launch costs what the slices gain)
+    if (p.K < (4 * t128 <= cu ? 1536 : 2048)) return plan;
     if (4 * t128 <= cu) {
         const int64_t s128 = capped(cu / t128, 512), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
         if (s64 >= 2 && s64 * t64 >= s128 * t128) set(s64, 64);
@@ -1441,8 +1443,9 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         split_knob = tuning(knob_gemm16_split_rows);
         if (variant < 0) variant = 0;
     }
-    if (variant <= 0 && col_cut && row_cuts == 2 && p.k_slice == 0) {
-        // the whole problem, before any cut: few tiles and a deep K go out as K slices
+    if (variant <= 0 && p.k_slice == 0) {
+        // the whole problem, or a part cut off it (the launches of one call follow each other on the stream and may
+        // use its workspace one after the other): few tiles and a deep K go out as K slices
         const int64_t big = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
         if (2 * big < compute_units() || p.M <= 32) {
             if (const SlicePlan16 plan = plan_k_slices16(p, kStreamWorkspaceBytes); plan.slices > 1) {

@@ -13,7 +13,7 @@ import kernel_optimization_amd as ko
 
 WORKSPACE = 32 << 20
 SIZES = [8, 31, 32, 64, 100, 107, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
-DEPTHS = [64, 512, 767, 768, 1300, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
+DEPTHS = [64, 512, 767, 768, 1300, 1535, 1536, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
 
 
 def _check(m, n, k, plan, k_tile, min_k, row_pad=1):
@@ -41,7 +41,7 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
 def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
     for k in DEPTHS:
         plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
-        _check(m, n, k, plan, k_tile=64, min_k=2048, row_pad=4)   # rows of partial products: whole groups of 4
+        _check(m, n, k, plan, k_tile=64, min_k=1536, row_pad=4)   # rows of partial products: whole groups of 4
         assert plan[2] in ((128, 64, 32) if plan[0] > 1 else (0,))
         if plan[2] == 32:
             assert m <= 32
