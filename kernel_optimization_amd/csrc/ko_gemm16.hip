@@ -1471,6 +1471,20 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // Columns that do not fill the last column of big tiles: the full tile columns go out on their own -
         // to the pinned kernel when the rest of the shape allows - and the remaining columns (fewer than 256)
         // as a launch of their own; C, D and a row-major B keep their row strides.
+        // A shallow K on a shape that is not whole 256 x 256 tiles: the time is the output's, and what counts is that
+        // a compute unit has a second workgroup to load and multiply while the first one stores (128 x 128 tiles,
+        // two workgroups per compute unit), not the rate of the main loop - neither the cuts below (whose parts
+        // run one after the other, each a launch that ends in a round of stores) nor 256 x 256 tiles pay.  Measured,
+        // whole on 128 x 128 tiles against cut (hipBLASLt), us: 4197 x 11928 x 64 48 / 58 (31), x 128 55 / 78 (38),
+        // x 256 81 / 71 (58); 4880 x 7768 x 256 52 / 60 (41), x 512 82 / 82; 1351 x 18488 x 256 41 / 45, x 512 65 / 60;
+        // 8148 x 1800 x 512 30 / 37 (27); 3000 x 5000 x 256 22 / 29 (22), x 512 34 / 38 (28).
+        {
+            const int64_t cu = compute_units();
+            const bool ragged = p.M % 256 != 0 || p.N % 256 != 0;
+            if (ragged && split_knob != 1 && 2 * big_tiles >= cu &&
+                (p.K <= 128 || (p.K <= 256 && 2 * big_tiles <= 5 * cu) || (p.K <= 512 && 4 * big_tiles <= 5 * cu)))
+                return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
+        }
         if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && (!B_ROW_MAJOR || (p.ldd % 8 == 0 && p.ldb % 8 == 0)) &&
             p.K >= 2 * kBK && 2 * static_cast<int64_t>(p.M / 256) * (p.N / 256) >= compute_units()) {
             const int n1 = p.N - p.N % 256;
