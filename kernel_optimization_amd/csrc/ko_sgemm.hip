@@ -794,6 +794,15 @@ int run(Params p, hipStream_t s, int variant) {
         // takes it as one K tile, the direct-to-LDS kernels pad it to a pair of them (8192 x 3072 x 8: 31 us
         // against 47 us)
         if (big && k <= 32) variant = 16;
+        // A shallow K on many small tiles: the time is the output's, and the direct-to-LDS 64 x 64 kernels - three
+        // stages, K padded to a pair of 64-deep tiles - spend it on their prologue (9523 x 344 x 32: 22 us; the
+        // 128 x 128 register pipeline 10.5; x 256: 38 against 28 on direct 128 x 128 tiles).  128 x 128 tiles
+        // where their rounds come out nearly full, else the 64 x 64 register pipeline (597 x 7992 x 128, 315 big
+        // tiles on 256 compute units: 23 us against 30 and 32).
+        if (!big && k <= 256 && t64 >= 2 * cu) {
+            const int64_t rounds128 = (t128 + cu - 1) / cu;
+            variant = k <= 32 ? 16 : (5 * t128 >= 4 * rounds128 * cu ? 36 : 13);
+        }
         // Operand rows off 16-byte boundaries are loaded four bytes per lane, four times as many loads with an
         // address each: the 128 x 128 x 64 form would spill registers there.
         const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
