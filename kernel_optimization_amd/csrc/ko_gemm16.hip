@@ -1477,12 +1477,14 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // run one after the other, each a launch that ends in a round of stores) nor 256 x 256 tiles pay.  Measured,
         // whole on 128 x 128 tiles against cut (hipBLASLt), us: 4197 x 11928 x 64 48 / 58 (31), x 128 55 / 78 (38),
         // x 256 81 / 71 (58); 4880 x 7768 x 256 52 / 60 (41), x 512 82 / 82; 1351 x 18488 x 256 41 / 45, x 512 65 / 60;
-        // 8148 x 1800 x 512 30 / 37 (27); 3000 x 5000 x 256 22 / 29 (22), x 512 34 / 38 (28).
+        // 8148 x 1800 x 512 30 / 37 (27); 3000 x 5000 x 256 22 / 29 (22), x 512 34 / 38 (28); 4071 x 2328 x 768
+        // (160 big tiles) 32 / 41 (24), 12521 x 989 x 768 40 / 52 (30), 3000 x 5000 x 768 (240) 46 / 48.
         {
             const int64_t cu = compute_units();
             const bool ragged = p.M % 256 != 0 || p.N % 256 != 0;
             if (ragged && split_knob != 1 && 2 * big_tiles >= cu &&
-                (p.K <= 128 || (p.K <= 256 && 2 * big_tiles <= 5 * cu) || (p.K <= 512 && 4 * big_tiles <= 5 * cu)))
+                (p.K <= 128 || (p.K <= 256 && 2 * big_tiles <= 5 * cu) || (p.K <= 512 && 4 * big_tiles <= 5 * cu) ||
+                 (p.K <= 768 && 5 * big_tiles <= 4 * cu)))
                 return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
         }
         if (col_cut && split_knob != 1 && p.N % 256 != 0 && p.N > 256 && (!B_ROW_MAJOR || (p.ldd % 8 == 0 && p.ldb % 8 == 0)) &&
