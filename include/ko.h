@@ -166,8 +166,8 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * accepted.  m == 0 or n == 0 is a no-op;
  * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries.
  * Workspace: a problem with a deep K whose output tiles do not fill the chip (tiles for at most half of the
- * compute units and k >= 768, or rounds of tiles that leave many compute units idle and k >= 2048; operand
- * rows on 16-byte boundaries) is cut into slices of K that run side by side; their partial products go
+ * compute units and k >= 768, or rounds of tiles that leave many compute units idle and k >= 2048; any n)
+ * is cut into slices of K that run side by side; their partial products go
  * through 32 MiB of device memory that the library allocates at the first such call on a (device, stream)
  * pair and keeps until the process ends.  Calls on different streams therefore never share it.  A first
  * such call made while the stream is being captured into a graph allocates nothing and takes the unsliced
@@ -202,7 +202,8 @@ int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, co
  * m and n are free: an n that is not a multiple of 8 (rows of C and D off 16-byte boundaries) keeps the fast
  * kernels with a column-major B and costs about a tenth; with a row-major B (whose own rows are off 16-byte
  * boundaries then) it runs at about 0.6 of the rate.
- * Workspace: like ko_sgemm_f32, a deep K (k >= 2048) on few output tiles is cut into slices of K whose fp32
+ * Workspace: like ko_sgemm_f32, a deep K (k >= 2048; k >= 1536 on very few tiles; any n) on few output tiles -
+ * of the whole problem or of the parts a ragged shape is cut into - is cut into slices of K whose fp32
  * partial products go through the 32 MiB workspace of the (device, stream) pair, allocated at the first such
  * call on the stream; a first such call inside a graph capture allocates nothing and runs unsliced. */
 int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A, const void *B,
