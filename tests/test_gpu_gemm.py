@@ -566,6 +566,31 @@ def test_gemm16_k_slices(ko, m, n, k, slices, b_col_major, bf16):
         ko.set_tuning("gemm16.k_slices", 0)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+def test_gemm16_parts_cut_off_a_ragged_shape_are_sliced(ko, b_col_major, bf16):
+    """2108 x 4232 x 2048: the call is cut into a block of full 256 x 256 tiles, the 60 rows below it and the 136
+    columns to its right; the two cut-off parts have few tiles and a deep K and go out as K slices through the
+    stream's workspace, one after the other.  Sampled rows of all three parts (every column) against the oracle,
+    with the whole epilogue; with slices switched off the parts run whole and must agree to the same bound."""
+    m, n, k = 2108, 4232, 2048
+    A = _bits16((m, k), 81, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 82, bf16)
+    C = _bits16((m, n), 83, bf16)
+    bias = _bits16((n,), 84, bf16)
+    idx = np.concatenate([np.sort(np.random.default_rng(8).choice(2048, 24, replace=False)), np.arange(2048, m, 5)])
+    kw = dict(b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR, dtype=ko.BF16 if bf16 else ko.F16)
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, b_col_major=b_col_major, bf16=bf16, C_bits=C[idx], beta=0.5,
+                                 bias_bits=bias, act=2)
+    try:
+        for slices in (0, 1):
+            ko.set_tuning("gemm16.k_slices", slices)
+            got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
+            assert_gemm16_act_close(_to_f64(got[idx], bf16), ref64, ap + 2.0, k, bf16=bf16)
+    finally:
+        ko.set_tuning("gemm16.k_slices", 0)
+
+
 @pytest.mark.parametrize("variant", [0, 9, 30, 50])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_gemm16_bias_gelu_big(ko, variant, bf16):
