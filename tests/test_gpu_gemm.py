@@ -771,10 +771,14 @@ def test_gemm16_shallow_k_whole_output(ko, m, n, k, bf16):
     np.testing.assert_array_equal(got, f16(exact - C + bias))
 
 
-@pytest.mark.parametrize("m,n,k", [(2048, 2304, 8), (4096, 1024, 32), (2100, 2500, 20)])
+@pytest.mark.parametrize("m,n,k", [(2048, 2304, 8), (4096, 1024, 32), (2100, 2500, 20),
+                                   # many small tiles that make no full round of big ones, K up to 256
+                                   (9523, 344, 32), (9523, 343, 200), (597, 7992, 128), (597, 7990, 256), (3000, 1500, 72)])
 def test_sgemm_shallow_k_is_exact_on_small_integers(ko, m, n, k):
     """A K of one 32-deep K tile or less on enough 128 x 128 tiles to fill the chip goes to the register pipeline
-    (one K tile instead of a padded pair).  Small integers: exact, with alpha, beta and C."""
+    (one K tile instead of a padded pair); a K of up to 256 on many small tiles to 128 x 128 tiles or the 64 x 64
+    register pipeline instead of the three-stage direct-to-LDS kernels.  Small integers: exact, with alpha, beta
+    and C."""
     rng = np.random.default_rng(m + k)
     A = rng.integers(-4, 5, (m, k)).astype(np.float32)
     B = rng.integers(-4, 5, (k, n)).astype(np.float32)
