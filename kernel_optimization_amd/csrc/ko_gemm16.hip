@@ -889,7 +889,10 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     constexpr int KS = kBK / 16;
     constexpr int A_BYTES = BM * kBK * 2, B_BYTES = BN * kBK * 2;  // per stage
     constexpr int A_LOADS = A_BYTES / 1024 / WAVES, B_LOADS = B_BYTES / 1024 / WAVES;
-    constexpr int EPI_PARTS = (BM * BN * 2) / (A_BYTES + B_BYTES);
+    // passes of the epilogue's transpose: half of the waves put their part of a pass into the A stage just
+    // consumed, the other half into the B stage, and both halves must fit
+    constexpr int EPI_PARTS = (WTM * WTN * 2 * (WAVES / 2) + (A_BYTES < B_BYTES ? A_BYTES : B_BYTES) - 1) /
+                              (A_BYTES < B_BYTES ? A_BYTES : B_BYTES);
     constexpr int READS = TM + TN;
     static_assert(T::SWIZZLE == 1 && KS == 4, "");
     static_assert(WAVES % 2 == 0 && A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0, "");
@@ -1087,10 +1090,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // all reads issued so far have landed; the fake operands keep later MFMAs behind this point
     auto wait_frags = [&](int slot) {
         if constexpr (B_ROW) {
-            static_assert(!B_ROW || (TM == 4 && TN == 2), "");
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
-                           "+v"(b_lo[slot][0]), "+v"(b_hi[slot][0]), "+v"(b_lo[slot][TN - 1]), "+v"(b_hi[slot][TN - 1]));
+            static_assert(!B_ROW || ((TM == 4 || TM == 2) && TN == 2), "");
+            if constexpr (TM == 4)
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
+                               "+v"(b_lo[slot][0]), "+v"(b_hi[slot][0]), "+v"(b_lo[slot][TN - 1]), "+v"(b_hi[slot][TN - 1]));
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(af[slot][0]), "+v"(af[slot][TM - 1]), "+v"(b_lo[slot][0]), "+v"(b_hi[slot][0]),
+                               "+v"(b_lo[slot][TN - 1]), "+v"(b_hi[slot][TN - 1]));
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 bf[slot][j] = u32x4{b_lo[slot][j][0], b_lo[slot][j][1], b_hi[slot][j][0], b_hi[slot][j][1]};
@@ -1098,6 +1106,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             asm volatile("s_waitcnt lgkmcnt(0)"
                          : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
                            "+v"(bf[slot][0]), "+v"(bf[slot][1]));
+        } else if constexpr (TM == 2 && TN == 2) {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1]));
         } else if constexpr (TM == 2 && TN == 4) {
             asm volatile("s_waitcnt lgkmcnt(0)"
                          : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1]),
@@ -1288,6 +1298,7 @@ using TileSmallN = Tiling<128, 64, 2, 2, 2, true, 1>;   // 4 waves, wave tile 64
 using TileTiny = Tiling<64, 64, 2, 2, 2, true, 1>;      // 4 waves, wave tile 32x32
 using TileSkinny = Tiling<32, 256, 1, 4, 2, true, 1>;   // 4 waves side by side, wave tile 32x64: at most 32 rows of A
 
+using TileHalf = Tiling<128, 256, 2, 4, 1, true, 1>;    // pinned kernel only: 8 waves, wave tile 64x64
 using TileBigSpare = Tiling<256, 256, 2, 4, 1, true, 1, true>;  // the same, epilogue through the spare 32 KB of LDS
 using TileBigSpread = Tiling<256, 256, 2, 4, 1, true, 1, true, true>;  // and the loads issued one by one in K step 3
 
@@ -1501,6 +1512,32 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
                 return st;
             return launch_variant<BF16, B_ROW_MAJOR>(right, stream, false, 1, variant, split_knob);
         }
+        // Between half a chip's and a whole chip's worth of 128 x 256 tiles: the pinned kernel on those (8 waves
+        // of 64 x 64).  A K tile takes it as long as one of a 256 x 256 tile - what bounds both is how far ahead
+        // two LDS stages let the loads run - but twice as many compute units work: 1536 x 4096 x 4096 (96 big tiles)
+        // 93 -> 79 us, 7168 x 768 x 3072 (84) 62 -> 52, 8192 x 1024 x 1024 (128) 27 -> 21, 2048 x 2304 x 768 (72)
+        // 17.4 -> 15.3; with 128 or fewer of them (4096 x 1024 x 1024 18.5 against 16.5) or more than one per
+        // compute unit (3072 x 4096 x 4096: 143 against 113) the other tilings win.  Rows below the last whole
+        // 128 go out as a launch of their own.
+        if (split_knob != 1 && p.N % 256 == 0 && p.K >= 256) {
+            const int64_t cu = compute_units();
+            const int64_t rows128 = p.M / 128;
+            const int64_t half_tiles = rows128 * (p.N / 256);
+            // (the second launch costs about 2 us: 2000 x 3072 x 768 22 us whole on 128 x 128 tiles, 24 cut; from
+            // K = 1536 on the first one gains more than that - 7000 x 768 x 3072 66 -> 58, 2000 x 4096 x 4096 117 -> 103)
+            if (20 * half_tiles >= 11 * cu && half_tiles <= cu && (p.M % 128 == 0 || (row_cuts > 0 && p.K >= 1536))) {
+                if (p.M % 128 == 0) return launch_pinned<TileHalf, BF16, B_ROW_MAJOR>(p, stream);
+                const int64_t m1 = rows128 * 128;
+                Params top = p, bottom = p;
+                top.M = static_cast<int>(m1);
+                bottom.M = p.M - static_cast<int>(m1);
+                bottom.A = p.A + m1 * p.K;
+                bottom.C = p.C ? p.C + m1 * p.ldd : nullptr;
+                bottom.D = p.D + m1 * p.ldd;
+                if (const int st = launch_pinned<TileHalf, BF16, B_ROW_MAJOR>(top, stream); st != KO_OK) return st;
+                return launch_variant<BF16, B_ROW_MAJOR>(bottom, stream, false, row_cuts - 1, variant, split_knob);
+            }
+        }
         if (row_cuts > 0 && split_knob != 1 && p.K >= 256) {
             const int64_t cu = compute_units();
             const int64_t tn = (p.N + 255) / 256;
@@ -1564,6 +1601,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
         case 53: return launch_direct<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }

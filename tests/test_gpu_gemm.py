@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 SGEMM_VARIANTS = [0, 13, 16, 21, 33, 35, 36, 37, 40, 41]
 SGEMM_PIPELINED = [13, 16, 21, 33, 35, 36, 37, 40, 41]  # two K tiles per loop trip; 33 on: direct-to-LDS
-GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 13, 30, 50, 52, 53]
+GEMM16_VARIANTS = [0, 3, 6, 9, 10, 11, 12, 13, 30, 50, 52, 53, 54]
 
 
 @pytest.fixture
@@ -225,11 +225,12 @@ def _to_f64(bits, bf16):
 @pytest.mark.parametrize("gemm16_variant", GEMM16_VARIANTS, indirect=True)
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("b_col_major", [True, False])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768), (512, 768, 192)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 72), (33, 36, 8), (128, 384, 768), (512, 768, 192),
+                                   (384, 512, 256)])
 def test_gemm16_matches_oracle(ko, gemm16_variant, bf16, b_col_major, m, n, k):
     if gemm16_variant == 30 and not b_col_major:
         pytest.skip("the compiler-scheduled direct-to-LDS kernel takes column-major B")
-    if gemm16_variant >= 30 and (m % 256 or n % 256 or k % 64):
+    if gemm16_variant >= 30 and (m % (128 if gemm16_variant == 54 else 256) or n % 256 or k % 64):
         pytest.skip("the direct-to-LDS kernels take full tiles only")
     if gemm16_variant >= 50 and k % 128:
         pytest.skip("the pinned kernel takes an even number of K tiles")
