@@ -1513,8 +1513,8 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             return launch_variant<BF16, B_ROW_MAJOR>(right, stream, false, 1, variant, split_knob);
         }
         // Between half a chip's and a whole chip's worth of 128 x 256 tiles: the pinned kernel on those (8 waves
-        // of 64 x 64).  A K tile takes it as long as one of a 256 x 256 tile - what bounds both is how far ahead
-        // two LDS stages let the loads run - but twice as many compute units work: 1536 x 4096 x 4096 (96 big tiles)
+        // of 64 x 64).  A K tile takes it as long as one of a 256 x 256 tile (a third LDS stage did not change
+        // that), but twice as many compute units work: 1536 x 4096 x 4096 (96 big tiles)
         // 93 -> 79 us, 7168 x 768 x 3072 (84) 62 -> 52, 8192 x 1024 x 1024 (128) 27 -> 21, 2048 x 2304 x 768 (72)
         // 17.4 -> 15.3; with 128 or fewer of them (4096 x 1024 x 1024 18.5 against 16.5) or more than one per
         // compute unit (3072 x 4096 x 4096: 143 against 113) the other tilings win.  Rows below the last whole
