@@ -569,6 +569,34 @@ def test_gemm16_k_slices(ko, m, n, k, slices, b_col_major, bf16):
 
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k", [(1536, 4096, 2048), (1608, 4096, 2048), (2048, 2304, 392)])
+def test_gemm16_between_half_and_a_whole_chip_of_128x256_tiles(ko, m, n, k, b_col_major, bf16):
+    """Shapes whose 256 x 256 tiles would cover half of the chip or less take 128 x 256 tiles of the pinned kernel
+    (192, 192 and 144 of them here; the second shape's last 72 rows go out as a launch of their own, the third
+    has a K that ends inside a pair of K tiles).  Sampled rows of every part against the oracle, with the whole
+    epilogue, and - in the rows the pinned kernel wrote; the rows below them go out as K slices, which round
+    differently - the same bits as the 128 x 128 register pipeline (same K order, same instruction)."""
+    A = _bits16((m, k), 91, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 92, bf16)
+    C = _bits16((m, n), 93, bf16)
+    bias = _bits16((n,), 94, bf16)
+    idx = np.unique(np.concatenate([np.random.default_rng(9).choice(m, 40, replace=False), np.arange(m - 8, m)]))
+    kw = dict(b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR, dtype=ko.BF16 if bf16 else ko.F16)
+    _, ref64, ap = oracle.gemm16(A[idx], B, len(idx), n, k, b_col_major=b_col_major, bf16=bf16, C_bits=C[idx], beta=0.5,
+                                 bias_bits=bias, act=2)
+    got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
+    assert_gemm16_act_close(_to_f64(got[idx], bf16), ref64, ap + 2.0, k, bf16=bf16)
+    plain = ko.gemm16_host(A, B, m, n, k, **kw)
+    ko.set_tuning("gemm16.variant", 10)
+    try:
+        top = m // 128 * 128
+        np.testing.assert_array_equal(plain[:top], ko.gemm16_host(A, B, m, n, k, **kw)[:top])
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
 def test_gemm16_parts_cut_off_a_ragged_shape_are_sliced(ko, b_col_major, bf16):
     """2108 x 4232 x 2048: the call is cut into a block of full 256 x 256 tiles, the 60 rows below it and the 136
     columns to its right; the two cut-off parts have few tiles and a deep K and go out as K slices through the
