@@ -134,6 +134,8 @@ struct Params {
     int k_slice;                // 0: no slices
     float *partial;
     int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
+    int xcd_cols_log2;          // blocked tile order: the 8 XCDs' regions lie 2^this side by side (0: one below the other)
+    int region_cols;            //                     columns of tiles in a region (unused when they lie one below the other)
 };
 
 // x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
@@ -173,16 +175,18 @@ __device__ __forceinline__ void finish4(const Params &p, float (&v)[4], u32x2 c2
 
 // Persistent kernels: tile number t (0, 1, ...) of workgroup b when the grid has `grid` workgroups.
 // Workgroup b runs on XCD b % 8 and is the (b / 8)-th of the workgroups there.  With band_rows > 0
-// each XCD owns band_rows consecutive rows of tiles and walks them in blocks of block_cols columns:
-// the workgroups that are resident on one XCD at a time cover a band_rows x block_cols block of
-// tiles, the most compact footprint (fewest distinct A and B panels) their shared L2 can be given,
-// and the A panels of the band are reused from block to block.  Otherwise tiles are dealt in
-// row-major order from one contiguous range per XCD.
+// the tile grid is cut into 8 regions, 8 >> xcd_cols_log2 of them below each other and 1 << xcd_cols_log2
+// side by side, one per XCD, each band_rows rows of tiles high and region_cols columns wide (the whole width
+// when they all lie below each other); an XCD walks its region in blocks of block_cols columns: the
+// workgroups that are resident on it at a time cover a band_rows x block_cols block of tiles, a compact
+// footprint (few distinct A and B panels) in their shared L2, and the A panels of the band are reused
+// from block to block.  Otherwise tiles are dealt in row-major order from one contiguous range per XCD.
 __device__ __forceinline__ void tile_of(const Params &p, int b, int grid, int t, int &tile_m, int &tile_n) {
     if (p.band_rows > 0) {
         const int x = b & 7, j = b >> 3;
-        tile_m = x * p.band_rows + j % p.band_rows;
-        tile_n = t * p.block_cols + j / p.band_rows;
+        const int xr = x >> p.xcd_cols_log2, xc = x & ((1 << p.xcd_cols_log2) - 1);  // the XCD's place among the regions
+        tile_m = xr * p.band_rows + j % p.band_rows;
+        tile_n = xc * p.region_cols + t * p.block_cols + j / p.band_rows;
     } else {
         const int tile = xcd_remap(b + grid * t, p.nblocks);
         tile_m = tile / p.tiles_n;
@@ -1233,15 +1237,30 @@ int launch_pinned(Params p, hipStream_t stream) {
     p.nblocks = tiles_m * p.tiles_n;
     int grid = compute_units() / 8 * 8;
     if (grid > p.nblocks) grid = p.nblocks;
-    // Blocked tile order when the tile grid divides evenly over 8 XCDs x (grid / 8) workgroups.
+    // Blocked tile order when the tile grid divides evenly over 8 XCDs x (grid / 8) workgroups: of the ways to lay
+    // the 8 regions out (8 x 1, 4 x 2, 2 x 4, 1 x 8) the one whose resident block of tiles needs the fewest bytes
+    // of A and B panels - for a short, wide output regions side by side (1024 x 8192 x 4096 on 128 x 256 tiles took
+    // 102 us as eight bands of one tile row, its transpose 88).
     p.band_rows = 0;
     p.block_cols = 0;
+    p.xcd_cols_log2 = 0;
+    p.region_cols = 0;
     const int per_xcd = grid / 8;
-    if (tuning(knob_gemm16_mapping) != 1 && grid % 8 == 0 && tiles_m % 8 == 0) {
-        const int band = tiles_m / 8;
-        if (band <= per_xcd && per_xcd % band == 0 && p.tiles_n % (per_xcd / band) == 0) {
-            p.band_rows = band;
-            p.block_cols = per_xcd / band;
+    if (tuning(knob_gemm16_mapping) != 1 && grid % 8 == 0) {
+        int64_t best = 0;
+        for (int lg = 0; lg <= 3; ++lg) {
+            const int across = 1 << lg, down = 8 >> lg;
+            if (tiles_m % down != 0 || p.tiles_n % across != 0) continue;
+            const int band = tiles_m / down, region = p.tiles_n / across;
+            if (band > per_xcd || per_xcd % band != 0 || region % (per_xcd / band) != 0) continue;
+            const int64_t bytes = static_cast<int64_t>(band) * T::BM + static_cast<int64_t>(per_xcd / band) * T::BN;
+            if (p.band_rows == 0 || bytes < best) {
+                best = bytes;
+                p.band_rows = band;
+                p.block_cols = per_xcd / band;
+                p.xcd_cols_log2 = lg;
+                p.region_cols = region;
+            }
         }
     }
     kernel<<<dim3(static_cast<unsigned>(grid)), dim3(T::THREADS), lds_bytes, stream>>>(p);
