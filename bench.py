@@ -50,11 +50,15 @@ def _traffic(name):
     return _traffic_table().get(name, {}).get("traffic_bytes")
 
 
-def _roofline(bound, achieved, peak, unit, name):
+def _roofline(bound, achieved, peak, unit, name, launch_s=None):
+    """launch_s: the average launch duration the figure was taken over; with it and a counter-traffic entry the
+    HBM bytes that really moved are priced against the HBM peak as well (frac_on_traffic)."""
     roof = dict(bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak, traffic=_traffic(name))
     if roof["traffic"] is not None:
         roof["traffic_source"] = "profiles/hbm_traffic.json @ %s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE)" % \
             _traffic_table().get("_measured_at_commit", "unknown commit")
+        if launch_s and bound == "hbm":
+            roof["frac_on_traffic"] = roof["traffic"] / launch_s / 1e9 / HBM_PEAK_GBS
     return roof
 
 
@@ -119,6 +123,13 @@ def _add_copy_floor(res, floor_us):
     res["vs_copy_same_bytes"] = floor_us / res["kernel_us"]
 
 
+def _masked_bytes(vl, n_seq, rows_per_seq, rows, cols, elem_bytes):
+    """Bytes a masked row softmax has to move: every column written, the valid columns read, the lengths read."""
+    lens = np.minimum(vl.download(np.int32, (n_seq,)).astype(np.int64), cols)
+    seq_rows = np.minimum(rows_per_seq, rows - rows_per_seq * np.arange(n_seq, dtype=np.int64)).clip(min=0)
+    return int(elem_bytes * (rows * cols + (lens * seq_rows).sum()) + 4 * n_seq)
+
+
 def bench_softmax(cfg, steps, warmup, unmasked=False):
     """Configurations 1 and 5.  unmasked: the shape of the masked configuration without its mask, so that every
     algorithmic byte really moves (with the mask a third of the reads is skipped)."""
@@ -141,12 +152,23 @@ def bench_softmax(cfg, steps, warmup, unmasked=False):
         ko.fill_lengths_i32(vl, c["n_seq"], inputs.tensor_seed(cfg, 1), c["len_lo"], c["len_hi"])
     floor_us = _copy_floor_us(xs, ys, n, steps, warmup)
     wall, dev = _time_steps(lambda i: ko.softmax(xs[i % nsets], ys[i % nsets], rows, cols, vl, rps), steps, warmup)
+    full = work
+    if vl is not None:
+        # A padded column takes the value -10000 whatever the tensor holds, so the operator has to read only the
+        # valid columns; every column is written.  These are the bytes the roofline figure is taken over: counting
+        # the padded reads as well (as 2 R C 4 does) credits the kernel with bytes that nothing has to move, and
+        # puts the "fraction of peak" above 1.
+        work = _masked_bytes(vl, c["n_seq"], rps, rows, cols, 4)
     res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"]),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"], dev),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
+    if vl is not None:
+        res["bytes_basis"] = "every column written, valid columns read (padded columns need no read)"
+        res["roofline"]["frac_counting_padded_reads"] = full / dev / 1e9 / HBM_PEAK_GBS
+        res["bytes_counting_padded_reads"] = full
     _add_copy_floor(res, floor_us)
-    keep = dict(x=xs[0], y=ys[0], vl=vl, rows=rows, cols=cols, rps=rps)
+    keep = dict(x=xs[0], y=ys[0], vl=vl, rows=rows, cols=cols, rps=rps, work=work)
     return res, keep
 
 
@@ -170,7 +192,7 @@ def bench_layernorm(cfg, steps, warmup):
                                                    rs[i % nsets], g, b, c["eps"]), steps, warmup)
     res = dict(workload=c["name"], metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"]),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", c["name"], dev),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
     keep = dict(x=xs[0], y=ys[0], mean=ms[0], rstd=rs[0], g=g, b=b, rows=rows, cols=cols, eps=c["eps"])
@@ -193,7 +215,7 @@ def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
     wall, dev = _time_steps(lambda i: ko.sgemm(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets]), steps, warmup)
     res = dict(workload=wname, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f32"], "TFLOP/s", wname),
+               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f32"], "TFLOP/s", wname, dev),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -239,9 +261,9 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
     # below the ridge of the roofline (flops per byte of A, B and D under MFMA peak / HBM peak) the bound is HBM
     nbytes = 2 * (m * k + k * n + m * n)
     if flops / nbytes < MFMA_PEAK_TFLOPS["f16"] * 1e12 / (HBM_PEAK_GBS * 1e9):
-        roof = _roofline("hbm", nbytes / dev / 1e9, HBM_PEAK_GBS, "GB/s", name)
+        roof = _roofline("hbm", nbytes / dev / 1e9, HBM_PEAK_GBS, "GB/s", name, dev)
     else:
-        roof = _roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", name)
+        roof = _roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", name, dev)
     res = dict(workload=name, metric="tflops", unit="TFLOP/s", value=flops / wall / 1e12,
                ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets, roofline=roof,
                flops=flops, kernel_us=dev * 1e6)
@@ -280,7 +302,7 @@ def bench_gemm16_bias_gelu(steps, warmup, vendor):
     res_name = "gemm_f16_bias_gelu_%dx%dx%d" % (m, n, k)
     res = dict(workload=res_name, metric="tflops", unit="TFLOP/s",
                value=flops / wall / 1e12, ms_per_step=wall * 1e3, dtype="f16", buffer_sets=nsets,
-               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", res_name),
+               roofline=_roofline("mfma", flops / dev / 1e12, MFMA_PEAK_TFLOPS["f16"], "TFLOP/s", res_name, dev),
                flops=flops, kernel_us=dev * 1e6)
     if vendor is not None:
         us, na = ctypes.c_float(), ctypes.c_int()
@@ -336,7 +358,7 @@ def bench_long_rows(op, rows, cols, policy, steps, warmup):
     res_name = "%s_f32_%dx%d_%s" % (op, rows, cols, names[policy])
     res = dict(workload=res_name, metric="hbm_gbytes_per_s", unit="GB/s",
                value=work / wall / 1e9, ms_per_step=wall * 1e3, dtype="f32", buffer_sets=nsets,
-               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name, dev),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
     _add_copy_floor(res, floor_us)
     return res
@@ -376,11 +398,16 @@ def bench_rows16(kind, dtype_name, steps, warmup):
         name = "layernorm_%s_%dx%d" % (dtype_name, rows, cols)
     floor_us = _copy_floor_us(xs, ys, n // 2, steps, warmup)
     wall, dev = _time_steps(launch, steps, warmup)
+    full = work
+    if kind == "softmax":
+        work = _masked_bytes(vl, c["n_seq"], c["rows_per_seq"], rows, cols, 2)
     res_name = name
     res = dict(workload=name, metric="hbm_gbytes_per_s", unit="GB/s", value=work / wall / 1e9,
                ms_per_step=wall * 1e3, dtype=dtype_name + " storage, f32 arithmetic", buffer_sets=nsets,
-               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name),
+               roofline=_roofline("hbm", work / dev / 1e9, HBM_PEAK_GBS, "GB/s", res_name, dev),
                algorithmic_bytes=work, kernel_us=dev * 1e6)
+    if kind == "softmax":
+        res["roofline"]["frac_counting_padded_reads"] = full / dev / 1e9 / HBM_PEAK_GBS
     _add_copy_floor(res, floor_us)
     return res
 
@@ -428,11 +455,12 @@ def cpu_baseline_softmax(keep, cfg):
     sel = ref >= np.finfo(np.float32).tiny
     parity = dict(rows_checked=rows, max_abs_err=float(d.max()), max_rel_err=float((d[sel] / ref[sel]).max()),
                   gate="abs<=1e-6 and rel<=1e-5", ok=bool(d.max() <= 1e-6 and (d[sel] / ref[sel]).max() <= 1e-5))
-    return dict(value=2 * rows * cols * 4 / best / 1e9, unit="GB/s", cores=oracle.max_threads(), kind="port",
+    work = keep.get("work", 2 * rows * cols * 4)  # the byte count the GPU figure is taken over
+    return dict(value=work / best / 1e9, unit="GB/s", cores=oracle.max_threads(), kind="port",
                 sample="all %d rows x %d cols of the same device-resident input, %d threads, best of 3; "
                        "host cpus visible: %d" % (rows, cols, oracle.max_threads(), os.cpu_count() or 0),
                 seconds=best,
-                single_thread=dict(value=2 * rows1 * cols * 4 / single / 1e9, unit="GB/s", cores=1,
+                single_thread=dict(value=work * rows1 / rows / single / 1e9, unit="GB/s", cores=1,
                                    sample="first %d rows, 1 thread, one run" % rows1, seconds=single)), parity
 
 
@@ -462,9 +490,15 @@ def cpu_baseline_layernorm(keep):
     ey = float((np.abs(y - ry) / np.maximum(np.abs(ry), 1.0)).max())
     er = float((np.abs(rstd - rr) / rr).max())
     em = float((np.abs(mean - rm) / np.maximum(np.abs(rm), 1.0 / rr)).max())
+    # not gated: the elementwise-relative worst cases, which no fp32 evaluation keeps below 1e-5 where x - mean
+    # (for y) or the sum of the row (for mean) cancels; printed so that what the gates give up can be seen
+    big = np.abs(ry) >= 1e-2
+    ey_pure = float((np.abs(y - ry)[big] / np.abs(ry)[big]).max())
+    em_pure = float((np.abs(mean - rm) / np.maximum(np.abs(rm), 1e-3)).max())
     parity = dict(rows_checked=rows, max_y_err=ey, max_rstd_rel_err=er, max_mean_err=em,
                   gate="|dy| <= 1e-5 max(|y|, 1); rstd 1e-5 relative; mean 1e-5 of max(|mean|, std)",
-                  ok=bool(ey <= 1e-5 and er <= 1e-5 and em <= 1e-5))
+                  ok=bool(ey <= 1e-5 and er <= 1e-5 and em <= 1e-5),
+                  ungated=dict(max_y_rel_err_where_y_ge_1e_2=ey_pure, max_mean_err_over_max_mean_1e_3=em_pure))
     work = 2 * rows * cols * 4
     return dict(value=work / best / 1e9, unit="GB/s", cores=nthreads, kind="port",
                 sample="all %d rows x %d cols, %d threads, best of 3; host cpus visible: %d" % (
@@ -586,6 +620,105 @@ def bench_ceilings(steps, warmup, nbytes=1 << 30, full=False):
     if full:
         out["rows"] = rows
     return out
+
+
+# ------------------------------------------------------------------------------ the record
+
+MAX_LINE_BYTES = 4096
+CONFIG_LINES = ("softmax_f32_196608x128", "layernorm_f32_16384x768", "sgemm_f32_1024x1024x1024",
+                "gemm_f16_16384x3072x768", "masked_softmax_f32_786432x512", "softmax_f32_786432x512_unmasked",
+                "gemm_f16_bias_gelu_16384x3072x768")
+
+
+def _sig(v, digits=4):
+    return None if v is None else float("%.*g" % (digits, v))
+
+
+def _compact(res):
+    """The handful of numbers of one workload that go into the one-line record."""
+    roof = res["roofline"]
+    out = {"name": res["workload"], "value": _sig(res["value"]), "unit": res["unit"],
+           "kernel_us": _sig(res["kernel_us"]), "bound": roof["bound"], "frac": _sig(roof["frac"])}
+    if roof.get("frac_on_traffic") is not None:
+        out["frac_on_traffic"] = _sig(roof["frac_on_traffic"])
+    for key in ("vs_hipblaslt", "vs_rocblas", "vs_copy_same_bytes"):
+        if key in res:
+            out[key] = _sig(res[key])
+    if res.get("parity") is not None:
+        out["parity_ok"] = res["parity"]["ok"]
+    if res.get("cpu_baseline") is not None:
+        out["cpu"] = _sig(res["cpu_baseline"]["value"])
+        out["cpu_cores"] = res["cpu_baseline"]["cores"]
+    return out
+
+
+def headline_line(head, cpu, parity, others, copy, info, steps, warmup):
+    """The record: one JSON object of at most MAX_LINE_BYTES characters, printed as the last line of stdout.  It
+    carries the headline workload in full (roofline, CPU baseline, parity) and six numbers for each of the other
+    configurations; everything else goes to gpurun_out/bench_workloads.json and to earlier lines."""
+    roof = {k: (_sig(v, 5) if isinstance(v, float) else v) for k, v in head["roofline"].items()}
+    line = {
+        "metric": head["metric"], "value": _sig(head["value"], 6), "unit": head["unit"], "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": _sig(head["ms_per_step"], 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic (seeded counter-based generator, filled on the device)",
+        "config": {"workload": head["workload"], "buffer_sets": head["buffer_sets"],
+                   "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
+        "roofline": roof,
+        "cpu_baseline": None if cpu is None else {
+            "value": _sig(cpu["value"]), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
+            "sample": cpu["sample"], "seconds": _sig(cpu.get("seconds"))},
+        "parity": None if parity is None else {k: (_sig(v) if isinstance(v, float) else v)
+                                               for k, v in parity.items() if k != "ungated"},
+        "kernel_us": _sig(head["kernel_us"], 5),
+    }
+    if "bytes_basis" in head:
+        line["config"]["bytes_basis"] = head["bytes_basis"]
+    if head.get("copy_same_bytes_us") is not None:
+        line["copy_same_bytes_us"] = _sig(head["copy_same_bytes_us"], 5)
+    if copy is not None:
+        line["copy_ceiling_frac"] = _sig(copy["roofline"]["frac"])
+    for key in ("hipblaslt_tflops", "vs_hipblaslt", "max_abs_diff_vs_hipblaslt"):
+        if key in head:
+            line[key] = _sig(head[key])
+    by_name = {r["workload"]: r for r in others}
+    line["configs"] = [_compact(by_name[n]) for n in CONFIG_LINES if n in by_name]
+    line["details_file"] = "gpurun_out/bench_workloads.json"
+    # never let the record outgrow what a reader of the last line keeps: shed the optional parts first
+    for key in ("details_file", "copy_ceiling_frac", "copy_same_bytes_us", "max_abs_diff_vs_hipblaslt"):
+        if len(json.dumps(line)) <= MAX_LINE_BYTES:
+            break
+        line.pop(key, None)
+    while len(json.dumps(line)) > MAX_LINE_BYTES and line["configs"]:
+        line["configs"].pop()
+    return line
+
+
+
+
+def emit_record(head, cpu, parity, others, copy, ceilings, info, steps, warmup, out_dir=None):
+    """Writes everything that was measured to <out_dir>/bench_workloads.json, prints one short line per secondary
+    workload, and prints the record as the LAST line of stdout."""
+    line = headline_line(head, cpu, parity, others, copy, info, steps, warmup)
+    details = dict(line)
+    details["copy_ceiling"] = None if copy is None else {
+        "GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"], "workload": copy["workload"],
+        "independent_sources": ceilings}
+    details["headline"] = dict(head, cpu_baseline=cpu, parity=parity)
+    details["workloads"] = others
+    out_dir = out_dir or os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "bench_workloads.json"), "w") as f:
+            json.dump(details, f, indent=1)
+    except OSError:
+        line.pop("details_file", None)
+    for res in others:
+        print(json.dumps(_compact(res)))
+    sys.stdout.flush()
+    print(json.dumps(line))
+    sys.stdout.flush()
+    return line
 
 
 def main():
@@ -718,23 +851,7 @@ def main():
             res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
 
-    line = {
-        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
-        "data": "synthetic (seeded counter-based generator, filled on the device)",
-        "config": {"workload": head["workload"], "buffer_sets": head["buffer_sets"],
-                   "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
-        "roofline": head["roofline"], "cpu_baseline": cpu, "parity": parity,
-        "kernel_us": head["kernel_us"], "copy_same_bytes_us": head.get("copy_same_bytes_us"),
-        "copy_ceiling": None if copy is None else {"GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"],
-                                                   "workload": copy["workload"], "independent_sources": ceilings},
-        "workloads": others,
-    }
-    for key in ("hipblaslt_tflops", "vs_hipblaslt", "max_abs_diff_vs_hipblaslt"):
-        if key in head:
-            line[key] = head[key]
-    print(json.dumps(line))
+    emit_record(head, cpu, parity, others, copy, ceilings, info, args.steps, args.warmup)
 
 
 if __name__ == "__main__":

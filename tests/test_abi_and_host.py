@@ -2,6 +2,7 @@
 include/ko.h declares; the ctypes table covers the same set; error paths that need no device; the
 C++ host layer (Tensor, descriptors, 16-bit types) builds with a plain C++ compiler and passes its
 self test."""
+import json
 import os
 import re
 import subprocess
@@ -191,3 +192,54 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0
     assert "one GPU" in (r.stderr + r.stdout)
 
+
+
+def _canned_result(name, unit="GB/s", bound="hbm", extra=None):
+    res = dict(workload=name, metric="hbm_gbytes_per_s" if unit == "GB/s" else "tflops", unit=unit,
+               value=6543.21987654321, ms_per_step=0.40123456789, dtype="f32", buffer_sets=3,
+               roofline=dict(bound=bound, achieved=6555.123456789, peak=8000.0, unit=unit, frac=0.81939043209876,
+                             traffic=2636973206, traffic_source="profiles/hbm_traffic.json @ 0123abc (rocprofv3 --pmc "
+                             "FETCH_SIZE, WRITE_SIZE)", frac_on_traffic=0.8239876543),
+               algorithmic_bytes=3221225472, kernel_us=400.123456789, copy_same_bytes_us=470.987654321,
+               vs_copy_same_bytes=1.17654321, steps=20, warmup=300,
+               cpu_baseline=dict(value=15.87654321, unit=unit, cores=16, kind="port", seconds=12.3456789,
+                                 sample="all 786432 rows x 512 cols of the same device-resident input, 16 threads, "
+                                        "best of 3; host cpus visible: 384"),
+               parity=dict(rows_checked=786432, max_abs_err=5.9e-8, max_rel_err=3.1e-7,
+                           gate="abs<=1e-6 and rel<=1e-5", ok=True))
+    res.update(extra or {})
+    return res
+
+
+def test_bench_record_is_one_short_last_line(tmp_path, capsys):
+    """The record bench.py prints is the last line of stdout, parses as JSON, stays under 4096 characters however
+    many workloads were measured, and carries the roofline, the CPU baseline and the per-configuration numbers."""
+    import bench
+    head = _canned_result("masked_softmax_f32_786432x512", extra=dict(bytes_basis="every column written, valid "
+                          "columns read (padded columns need no read)"))
+    head["roofline"]["frac_counting_padded_reads"] = 1.0043
+    cpu, parity = head.pop("cpu_baseline"), head.pop("parity")
+    others = [_canned_result(n) for n in bench.CONFIG_LINES if n != head["workload"]]
+    others[2].update(unit="TFLOP/s", vs_hipblaslt=0.94321, vs_rocblas=0.92345)
+    others += [_canned_result("layernorm_f32_%dx%d_block" % (1024 << i, 131072 >> i)) for i in range(40)]
+    info = dict(name="AMD Instinct MI355X", arch="gfx950:sramecc+:xnack-", compute_units=256)
+    copy = _canned_result("copy_f32_1024MiB")
+    line = bench.emit_record(head, cpu, parity, others, copy, {"rows": list(range(1000))}, info, 20, 5,
+                             out_dir=str(tmp_path))
+    out = capsys.readouterr().out.rstrip("\n").split("\n")
+    assert len(out) == len(others) + 1
+    last = out[-1]
+    assert len(last) < bench.MAX_LINE_BYTES <= 4096
+    rec = json.loads(last)
+    assert rec == line
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "parity", "configs"):
+        assert key in rec, key
+    assert rec["config"]["workload"] == "masked_softmax_f32_786432x512" and "model" not in rec["config"]
+    assert set(rec["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"}
+    assert rec["roofline"]["frac"] <= 1.0
+    assert set(rec["cpu_baseline"]) >= {"value", "unit", "cores", "kind", "sample"}
+    assert [c["name"] for c in rec["configs"]] == [n for n in bench.CONFIG_LINES if n != head["workload"]]
+    assert all(len(l) < 1024 and json.loads(l)["name"] for l in out[:-1])
+    details = json.load(open(tmp_path / "bench_workloads.json"))
+    assert len(details["workloads"]) == len(others) and details["copy_ceiling"]["independent_sources"]
