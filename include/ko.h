@@ -89,7 +89,7 @@ int ko_memcpy_d2h_async(void *host_dst, const void *device_src, size_t bytes, ko
 int ko_memcpy_d2d_async(void *device_dst, const void *device_src, size_t bytes, ko_stream_t stream);
 
 int ko_stream_create(ko_stream_t *stream);       /* cudaStreamCreateWithFlags(NonBlocking), softmax/main.cu:29 */
-int ko_stream_destroy(ko_stream_t stream);
+int ko_stream_destroy(ko_stream_t stream);        /* waits for the stream's work, frees its workspace (see ko_sgemm_f32) */
 int ko_stream_synchronize(ko_stream_t stream);   /* softmax/main.cu:46,70 */
 int ko_device_synchronize(void);                 /* gemm/main.cu:152 */
 
@@ -163,16 +163,24 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * with C given, or D = A*B with C null (simt_gemm.h:325-373).
  * m, n, k multiples of 4 and 16-byte aligned pointers are not required (operand rows that do not start on
  * 16-byte boundaries are loaded four bytes at a time: about 0.7 of the aligned rate); any positive sizes are
- * accepted.  m == 0 or n == 0 is a no-op;
- * k == 0 (an empty product, D = beta * C) is not provided: KO_ERR_UNSUPPORTED_SHAPE, in both GEMM entries.
+ * accepted.  m == 0 or n == 0 is a no-op; k == 0 is the empty product, D = beta * C (zero without a C) in one
+ * scale-and-copy launch, as the reference's kernel leaves it when its main loop runs no K tile
+ * (simt_gemm.h:325-354); A and B may be NULL then.  The 16-bit entries do the same: D = activation(beta * C + bias).
  * Workspace: a problem with a deep K whose output tiles do not fill the chip (tiles for at most half of the
  * compute units and k >= 768, or rounds of tiles that leave many compute units idle and k >= 2048; any n)
  * is cut into slices of K that run side by side; their partial products go
  * through 32 MiB of device memory that the library allocates at the first such call on a (device, stream)
- * pair and keeps until the process ends.  Calls on different streams therefore never share it.  A first
- * such call made while the stream is being captured into a graph allocates nothing and takes the unsliced
- * kernels; so does every call once 64 pairs hold a workspace.  Results do not depend on the timing of the
- * slices (summed in slice order), but the sliced and the unsliced path round differently. */
+ * pair and keeps until ko_stream_destroy releases it (the default stream's: until the process ends).  Calls on
+ * different streams therefore never share it.  A first such call made while the stream is being captured into a
+ * graph allocates nothing and takes the unsliced kernels; so does every call while 64 live pairs hold a
+ * workspace.  Results do not depend on the timing of the slices (summed in slice order), but the sliced and the
+ * unsliced path round differently.
+ * Graphs: a sliced call captured on a stream that already has its workspace records that workspace's address.
+ * Replay such a graph only in stream order with the other work of the stream it was captured on (a replay on
+ * another stream, or two replays in flight at once, race on the workspace with each other and with eager
+ * sliced calls on the origin stream and give wrong sums), and not after that stream was destroyed (its
+ * workspace is freed then).  ko_sgemm_f32_static_scratch is the entry for graphs that must not depend on a
+ * stream's lifetime. */
 int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const float *B,
                  float beta, const float *C, float *D, ko_stream_t stream);
 
@@ -182,8 +190,8 @@ int ko_sgemm_f32(int64_t m, int64_t n, int64_t k, float alpha, const float *A, c
  * 32 MiB array that is part of the library's device code (one copy per GPU, held until the process ends)
  * instead of a workspace allocated for the stream: the call makes no hipMalloc or hipFree, also not the
  * first one on a stream.  A slice plan whose partial products exceed the array is refused with
- * KO_ERR_UNSUPPORTED_SHAPE (plans chosen by shape are chosen to fit; only a slice count forced through
- * ko_set_tuning("sgemm.k_slices") can exceed it).
+ * KO_ERR_UNSUPPORTED_SHAPE (plans chosen by shape are chosen to fit; only a slice count forced through the
+ * harness's tuning knob "sgemm.k_slices" can exceed it).
  * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams, different
  * threads) race on it and must be serialised by the caller.  Nothing in it has to start at zero: every
  * element the summing kernel reads was written by the same call.  The first call on a device looks up the
@@ -220,52 +228,6 @@ int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float alpha, con
                                const void *B, int b_layout, float beta, const void *C,
                                const void *bias, int activation, void *D, int in_dtype,
                                ko_stream_t stream);
-
-/* ---- seeded device fills: replace the host RNG loops of the benchmark drivers
- *      (softmax/main.cu:31-36, layernorm/main.cu:30-35, gemm/main.cu:46-66) with a
- *      counter-based generator that gives the same tensor on host and device:
- *      splitmix64(seed, counter) -> u in [0,1); uniform = lo + (hi-lo)*u;
- *      normal = mean + std * sqrt(-2 ln(1-u(2i))) * cos(2 pi u(2i+1)); evaluated in
- *      double, rounded once to the storage type.  `first` is the index of out[0]. */
-int ko_fill_normal_f32(float *out, int64_t n, uint64_t seed, double mean, double std,
-                       int64_t first, ko_stream_t stream);
-int ko_fill_uniform_f32(float *out, int64_t n, uint64_t seed, double lo, double hi, int64_t first,
-                        ko_stream_t stream);
-int ko_fill_uniform_16(void *out, int64_t n, uint64_t seed, double lo, double hi, int64_t first,
-                       int dtype, ko_stream_t stream);
-/* int32 lengths lo + floor((hi - lo + 1) * u), uniform on [lo, hi] */
-int ko_fill_lengths_i32(int32_t *out, int64_t n, uint64_t seed, int32_t lo, int32_t hi,
-                        ko_stream_t stream);
-
-/* ---- measurement helpers (no reference counterpart; used by the benchmark harness) */
-/* out[i] = in[i] for n floats, 128-bit accesses: the plain copy whose rate is the
- * practical HBM ceiling the bandwidth kernels are compared with. */
-int ko_copy_f32(const float *in, float *out, int64_t n, ko_stream_t stream);
-/* Streaming-rate probe: one launch that streams `nbytes` (a multiple of threads * vectors_per_thread * 16)
- * from `in` and/or to `out`: mode 0 write-only, 1 read-only, 2 copy, 3 copy that reads only the vectors whose
- * index modulo 128 is below `read_of_128` (a 512-column fp32 row with a padded tail) and writes all.
- * threads: workgroup size (multiple of 64); vectors_per_thread: 1, 2 or 4 16-byte vectors;
- * blocks_per_cu: 0 = one chunk per workgroup, else a grid of that many workgroups per compute unit walking
- * the chunks; load_policy: 0 plain, 1 non-temporal; store_policy: 0 plain, 1 nt, 2 sc1, 3 sc1 nt,
- * 4 sc0 sc1 nt (the cache-policy bits of the store instruction); lds_pad_bytes: dynamic LDS per workgroup,
- * never touched, which caps how many workgroups are resident per compute unit. */
-int ko_stream_probe(const void *in, void *out, int64_t nbytes, int mode, int vectors_per_thread,
-                    int threads, int blocks_per_cu, int load_policy, int store_policy, int read_of_128,
-                    int lds_pad_bytes, ko_stream_t stream);
-/* Integer tuning knobs by name ("softmax.lanes_per_row", ...); value 0 restores the default.
- * Unknown names return KO_ERR_INVALID_ARGUMENT. */
-int ko_set_tuning(const char *name, int value);
-int ko_get_tuning(const char *name, int *value);
-/* Cross-lane primitives check: each of the 64 lanes of one wavefront contributes
- * in[lane]; out[lane] receives the all-reduce over its group of `group` lanes
- * (group in {2,4,8,16,32,64}; op 0 = max, 1 = sum). */
-int ko_debug_wave_allreduce(const float *in, float *out, int group, int op, ko_stream_t stream);
-/* What the GEMMs' host-side planners decide for a shape (16-byte aligned operands, 256 compute units when no
- * device is visible): the number of K slices (1 = the problem goes out whole), the depth of every slice but the
- * last, and the tiling of the sliced launch (SGEMM: the kernel variant number, 0 = chosen as for the whole
- * problem; 16-bit GEMM: 128 or 64, the tile edge, or 32 for 32 x 256 tiles).  Touches no device memory and launches nothing. */
-int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
-int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
 
 #ifdef __cplusplus
 }

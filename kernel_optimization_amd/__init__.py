@@ -11,6 +11,7 @@ import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libko.so")
+HARNESS_PATH = os.path.join(_PKG, "lib", "libko_harness.so")
 
 KO_OK = 0
 KO_ERR_INVALID_ARGUMENT = 1
@@ -72,6 +73,10 @@ SIGNATURES = {
     "ko_sgemm_f32_static_scratch": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _f, _vp, _vp, _vp]),
     "ko_gemm_f16f32acc": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp]),
     "ko_gemm_f16f32acc_bias_act": (_int, [_i64, _i64, _i64, _f, _vp, _vp, _int, _f, _vp, _vp, _int, _vp, _int, _vp]),
+}
+
+# every symbol of libko_harness.so that include/ko_harness.h declares (tests and benchmark only)
+HARNESS_SIGNATURES = {
     "ko_fill_normal_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
     "ko_fill_uniform_f32": (_int, [_vp, _i64, _u64, _d, _d, _i64, _vp]),
     "ko_fill_uniform_16": (_int, [_vp, _i64, _u64, _d, _d, _i64, _int, _vp]),
@@ -81,6 +86,7 @@ SIGNATURES = {
     "ko_set_tuning": (_int, [ctypes.c_char_p, _int]),
     "ko_get_tuning": (_int, [ctypes.c_char_p, ctypes.POINTER(_int)]),
     "ko_debug_wave_allreduce": (_int, [_vp, _vp, _int, _int, _vp]),
+    "ko_debug_stream_workspace_count": (_int, [ctypes.POINTER(_int)]),
     "ko_debug_sgemm_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
                                    ctypes.POINTER(ctypes.c_int)]),
     "ko_debug_gemm16_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
@@ -88,6 +94,7 @@ SIGNATURES = {
 }
 
 _lib = None
+_harness = None
 
 
 class KoError(RuntimeError):
@@ -110,6 +117,24 @@ def lib():
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+def harness():
+    """Loads libko_harness.so (fills, probes, tuning knobs, debug views): what tests and the benchmark use beside
+    the operator library.  Raises if it is missing."""
+    global _harness
+    if _harness is None:
+        lib()
+        if not os.path.exists(HARNESS_PATH):
+            raise RuntimeError("libko_harness.so is not built: run `python -m kernel_optimization_amd.build` "
+                               "(expected %s)." % HARNESS_PATH)
+        H = ctypes.CDLL(HARNESS_PATH)
+        for name, (res, args) in HARNESS_SIGNATURES.items():
+            fn = getattr(H, name)
+            fn.restype = res
+            fn.argtypes = args
+        _harness = H
+    return _harness
 
 
 def status_name(status):
@@ -138,12 +163,12 @@ def device_available():
 
 
 def set_tuning(name, value):
-    check(lib().ko_set_tuning(name.encode(), int(value)))
+    check(harness().ko_set_tuning(name.encode(), int(value)))
 
 
 def get_tuning(name):
     v = _int(0)
-    check(lib().ko_get_tuning(name.encode(), ctypes.byref(v)))
+    check(harness().ko_get_tuning(name.encode(), ctypes.byref(v)))
     return v.value
 
 
@@ -285,7 +310,7 @@ def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
 def gemm_plan(m, n, k, sixteen_bit=False):
     """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM decides for a shape."""
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    fn = lib().ko_debug_gemm16_plan if sixteen_bit else lib().ko_debug_sgemm_plan
+    fn = harness().ko_debug_gemm16_plan if sixteen_bit else harness().ko_debug_sgemm_plan
     check(fn(m, n, k, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
     return a.value, b.value, c.value
 
@@ -306,23 +331,23 @@ def gemm16(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, b_layout=COL_MAJOR, dt
 
 
 def fill_normal_f32(out, n, seed, mean=0.0, std=1.0, first=0, stream=None):
-    check(lib().ko_fill_normal_f32(_p(out), n, seed, mean, std, first, _h(stream)))
+    check(harness().ko_fill_normal_f32(_p(out), n, seed, mean, std, first, _h(stream)))
 
 
 def fill_uniform_f32(out, n, seed, lo=-1.0, hi=1.0, first=0, stream=None):
-    check(lib().ko_fill_uniform_f32(_p(out), n, seed, lo, hi, first, _h(stream)))
+    check(harness().ko_fill_uniform_f32(_p(out), n, seed, lo, hi, first, _h(stream)))
 
 
 def fill_uniform_16(out, n, seed, lo=-1.0, hi=1.0, first=0, dtype=F16, stream=None):
-    check(lib().ko_fill_uniform_16(_p(out), n, seed, lo, hi, first, dtype, _h(stream)))
+    check(harness().ko_fill_uniform_16(_p(out), n, seed, lo, hi, first, dtype, _h(stream)))
 
 
 def fill_lengths_i32(out, n, seed, lo, hi, stream=None):
-    check(lib().ko_fill_lengths_i32(_p(out), n, seed, lo, hi, _h(stream)))
+    check(harness().ko_fill_lengths_i32(_p(out), n, seed, lo, hi, _h(stream)))
 
 
 def copy_f32(inp, out, n, stream=None):
-    check(lib().ko_copy_f32(_p(inp), _p(out), n, _h(stream)))
+    check(harness().ko_copy_f32(_p(inp), _p(out), n, _h(stream)))
 
 
 PROBE_WRITE, PROBE_READ, PROBE_COPY, PROBE_PARTIAL = 0, 1, 2, 3
@@ -332,7 +357,7 @@ STORE_POLICIES = {"plain": 0, "nt": 1, "sc1": 2, "sc1 nt": 3, "sc0 sc1 nt": 4}
 
 def stream_probe(inp, out, nbytes, mode, vectors_per_thread=1, threads=128, blocks_per_cu=0, load_policy=1,
                  store_policy=3, read_of_128=128, lds_pad_bytes=0, stream=None):
-    check(lib().ko_stream_probe(_p(inp), _p(out), nbytes, mode, vectors_per_thread, threads, blocks_per_cu,
+    check(harness().ko_stream_probe(_p(inp), _p(out), nbytes, mode, vectors_per_thread, threads, blocks_per_cu,
                                 load_policy, store_policy, read_of_128, lds_pad_bytes, _h(stream)))
 
 

@@ -1,7 +1,8 @@
-"""Builds the native parts in-tree: libko.so (HIP kernels + C ABI, gfx950) and the
+"""Builds the native parts in-tree: libko.so (HIP kernels + C ABI, gfx950), libko_harness.so (fills, probes,
+tuning and debug views for the tests and the benchmark) and the
 pure C++ host layer (Tensor, benchmark drivers) that sits on top of the C ABI.
 
-Usage: python -m kernel_optimization_amd.build [--jobs N] [--only lib|host|vendor] [--cmake]
+Usage: python -m kernel_optimization_amd.build [--jobs N] [--only lib|harness|host|vendor] [--cmake]
 """
 import argparse
 import concurrent.futures
@@ -62,6 +63,26 @@ def build_lib(jobs=4, verbose=False):
     return LIB_PATH
 
 
+def build_harness(jobs=4, verbose=False):
+    """libko_harness.so: seeded fills, copy and streaming-probe kernels, tuning knobs and debug views
+    (include/ko_harness.h).  Tests and the benchmark load it beside libko.so; it is no part of the product."""
+    hdir = os.path.join(PKG, "harness")
+    out_path = os.path.join(LIB_DIR, "libko_harness.so")
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs, cmds = [], []
+    for src in sorted(f for f in os.listdir(hdir) if f.endswith(".hip")):
+        obj = os.path.join(OBJ_DIR, "harness_" + src[:-4] + ".o")
+        objs.append(obj)
+        cmds.append([HIPCC, *HIP_FLAGS, "-I", CSRC, "-c", os.path.join(hdir, src), "-o", obj])
+    with concurrent.futures.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        for out in pool.map(_run, cmds):
+            if verbose and out.strip():
+                print(out)
+    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out_path, *objs, "-L", LIB_DIR, "-lko",
+          "-Wl,-rpath,$ORIGIN"])
+    return out_path
+
+
 def build_vendor(verbose=False):
     """libko_vendor.so: hipBLASLt and rocBLAS timed on the same buffers (comparison harness, not product)."""
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -111,15 +132,16 @@ def build_cmake(jobs=4, verbose=False, targets=()):
 
 def build_all(jobs=4, verbose=False):
     lib = build_lib(jobs=jobs, verbose=verbose)
+    harness = build_harness(jobs=jobs, verbose=verbose)
     vendor = build_vendor(verbose=verbose)
     host = build_host(verbose=verbose)
-    return lib, vendor, host
+    return lib, harness, vendor, host
 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    ap.add_argument("--only", choices=["lib", "host", "vendor"])
+    ap.add_argument("--only", choices=["lib", "harness", "host", "vendor"])
     ap.add_argument("-v", "--verbose", action="store_true")
     ap.add_argument("--cmake", action="store_true", help="build everything through CMakeLists.txt instead")
     args = ap.parse_args(argv)
@@ -128,6 +150,8 @@ def main(argv=None):
         return
     if args.only in (None, "lib"):
         print("built", build_lib(args.jobs, args.verbose))
+    if args.only in (None, "harness"):
+        print("built", build_harness(args.jobs, args.verbose))
     if args.only in (None, "vendor"):
         print("built", build_vendor(args.verbose))
     if args.only in (None, "host"):

@@ -1336,7 +1336,8 @@ int launch_direct(const Params &p, hipStream_t stream) {
 
 // D = act(alpha * (P_0 + ... + P_{slices-1}) + beta * C + bias), rounded once, from the fp32 partial products of a
 // K-sliced launch, summed in slice order.  One thread per four consecutive columns; the last group of a row whose
-// length is not a multiple of 4 finishes its columns one by one.
+// length is not a multiple of 4 finishes its columns one by one.  slices == 0 is the empty product (k == 0): nothing
+// is read through p.partial and D = act(beta * C + bias).
 template <bool BF16>
 __global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, int slices) {
     typedef float float4v __attribute__((ext_vector_type(4)));
@@ -1347,7 +1348,8 @@ __global__ __launch_bounds__(64) void gemm16_slices_sum_kernel(const Params p, i
     const int m = static_cast<int>(g / groups_per_row), n = static_cast<int>(g % groups_per_row) * 4;
     const int64_t count = p.M * ldp;
     const float *src = p.partial + m * ldp + n;
-    float4v acc = *reinterpret_cast<const float4v *>(src);
+    float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (slices > 0) acc = *reinterpret_cast<const float4v *>(src);
     int s = 1;
     for (; s + 8 <= slices; s += 8) {
         float4v t[8];
@@ -1640,11 +1642,11 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
     if (activation != KO_ACT_NONE && activation != KO_ACT_GELU_ERF && activation != KO_ACT_GELU_TANH)
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: activation=%d", activation);
     if (m == 0 || n == 0) return KO_OK;
-    if (k == 0 || k % 8 != 0)
-        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: k=%lld must be a positive multiple of 8", (long long)k);
+    if (k % 8 != 0)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: k=%lld must be a multiple of 8", (long long)k);
     if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: dimension too large");
-    if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: null A/B/D pointer");
+    if (!D || (k > 0 && (!A || !B))) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: null A/B/D pointer");
     uintptr_t align = reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
                       reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D);
     if (align & 15) return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: A, B, C and D must be 16-byte aligned");
@@ -1655,6 +1657,14 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
              static_cast<const uint16_t *>(bias), activation, static_cast<int>(n), static_cast<int>(n),
              0, nullptr, static_cast<int>(k)};
     hipStream_t s = as_stream(stream);
+    if (k == 0) {  // the empty product: D = act(beta * C + bias), one launch of the epilogue kernel; A and B are not touched
+        const int64_t groups = m * (partial_ld(p.N) / 4);
+        const dim3 grid(static_cast<unsigned>((groups + 63) / 64));
+        if (in_dtype == KO_F16) gemm16_slices_sum_kernel<false><<<grid, 64, 0, s>>>(p, 0);
+        else gemm16_slices_sum_kernel<true><<<grid, 64, 0, s>>>(p, 0);
+        KO_CHECK_LAUNCH();
+        return KO_OK;
+    }
     if (in_dtype == KO_F16)
         return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);
     return b_layout == KO_COL_MAJOR ? launch_variant<true, false>(p, s) : launch_variant<true, true>(p, s);
@@ -1667,10 +1677,10 @@ KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, co
                                       stream);
 }
 
-KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile) {
+int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile) {
     using namespace ko;
     if (!slices || !k_slice || !tile || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
-        return fail(KO_ERR_INVALID_ARGUMENT, "ko_debug_gemm16_plan: bad argument");
+        return fail(KO_ERR_INVALID_ARGUMENT, "gemm16_plan: bad argument");
     Params p{};
     p.M = static_cast<int>(m);
     p.N = static_cast<int>(n);

@@ -9,6 +9,7 @@
 #include <cstdio>
 
 #include "../../include/ko.h"
+#include "../../include/ko_harness.h"
 
 #define KO_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -68,13 +69,21 @@ int compute_units();
 int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done);
 
 // Device memory for the partial results of calls on `stream` of the current device: kStreamWorkspaceBytes,
-// allocated at the first request for that (device, stream) pair and kept until the process ends, so calls on
-// different streams never share it and calls on one stream use it in stream order.  `*workspace` stays null,
-// with KO_OK, where nothing may be allocated (the stream is being captured into a graph and has no workspace
-// yet, 64 pairs already hold one, the stream is hipStreamPerThread, or the allocation fails): the caller then
-// takes its path without a workspace.
+// allocated at the first request for that (device, stream) pair and kept until ko_stream_destroy releases it
+// (the default stream's until the process ends), so calls on different streams never share it and calls on one
+// stream use it in stream order.  `*workspace` stays null, with KO_OK, where nothing may be allocated (the
+// stream is being captured into a graph and has no workspace yet, 64 live pairs already hold one, the stream is
+// hipStreamPerThread, or the allocation fails): the caller then takes its path without a workspace.
 constexpr size_t kStreamWorkspaceBytes = size_t{32} << 20;
 int stream_workspace(hipStream_t stream, void **workspace);
+// Frees the workspace of (current device, stream), if it has one.  The caller has synchronised the stream.
+int release_stream_workspace(hipStream_t stream);
+// How many (device, stream) pairs hold a workspace right now.
+int stream_workspace_count();
+
+// What the GEMM planners decide for a shape, for the harness (ko_harness_hooks_t::sgemm_plan, gemm16_plan).
+int debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
+int debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
 
 }  // namespace ko
 

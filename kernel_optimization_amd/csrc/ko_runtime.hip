@@ -35,7 +35,7 @@ static const char *const kKnobNames[knob_count] = {
 #undef KO_KNOB_NAME
 };
 
-// Index of the knob called `name`, or -1.  Only ko_set_tuning / ko_get_tuning look names up.
+// Index of the knob called `name`, or -1.  Only the harness hooks look names up.
 static int find_knob(const char *name) {
     for (int i = 0; i < knob_count; ++i)
         if (std::strcmp(kKnobNames[i], name) == 0) return i;
@@ -67,24 +67,27 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
     return KO_OK;
 }
 
+namespace {
+struct WorkspaceEntry { int device; hipStream_t stream; void *memory; };
+constexpr int kMaxWorkspaces = 64;
+WorkspaceEntry g_workspaces[kMaxWorkspaces];
+int g_workspaces_used = 0;
+std::mutex g_workspaces_lock;
+}  // namespace
+
 int stream_workspace(hipStream_t stream, void **workspace) {
-    struct Entry { int device; hipStream_t stream; void *memory; };
-    constexpr int kMaxEntries = 64;
-    static Entry entries[kMaxEntries];
-    static int used = 0;
-    static std::mutex lock;
     *workspace = nullptr;
     // one handle value stands for a different stream in every host thread: no workspace can belong to it
     if (stream == hipStreamPerThread) return KO_OK;
     int dev = 0;
     KO_HIP(hipGetDevice(&dev));
-    std::lock_guard<std::mutex> guard(lock);
-    for (int i = 0; i < used; ++i)
-        if (entries[i].device == dev && entries[i].stream == stream) {
-            *workspace = entries[i].memory;
+    std::lock_guard<std::mutex> guard(g_workspaces_lock);
+    for (int i = 0; i < g_workspaces_used; ++i)
+        if (g_workspaces[i].device == dev && g_workspaces[i].stream == stream) {
+            *workspace = g_workspaces[i].memory;
             return KO_OK;
         }
-    if (used == kMaxEntries) return KO_OK;
+    if (g_workspaces_used == kMaxWorkspaces) return KO_OK;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
         (void)hipGetLastError();
@@ -98,9 +101,31 @@ int stream_workspace(hipStream_t stream, void **workspace) {
         (void)hipGetLastError();
         return KO_OK;
     }
-    entries[used++] = Entry{dev, stream, memory};
+    g_workspaces[g_workspaces_used++] = WorkspaceEntry{dev, stream, memory};
     *workspace = memory;
     return KO_OK;
+}
+
+int release_stream_workspace(hipStream_t stream) {
+    int dev = 0;
+    KO_HIP(hipGetDevice(&dev));
+    void *memory = nullptr;
+    {
+        std::lock_guard<std::mutex> guard(g_workspaces_lock);
+        for (int i = 0; i < g_workspaces_used; ++i)
+            if (g_workspaces[i].device == dev && g_workspaces[i].stream == stream) {
+                memory = g_workspaces[i].memory;
+                g_workspaces[i] = g_workspaces[--g_workspaces_used];
+                break;
+            }
+    }
+    if (memory != nullptr) KO_HIP(hipFree(memory));
+    return KO_OK;
+}
+
+int stream_workspace_count() {
+    std::lock_guard<std::mutex> guard(g_workspaces_lock);
+    return g_workspaces_used;
 }
 
 }  // namespace ko
@@ -119,21 +144,33 @@ KO_EXPORT const char *ko_status_name(int status) {
     }
 }
 
-KO_EXPORT int ko_set_tuning(const char *name, int value) {
-    if (!name) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: null name");
-    const int k = ko::find_knob(name);
-    if (k < 0) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: unknown knob \"%s\"", name);
-    ko::g_knobs[k].store(value, std::memory_order_relaxed);
+// ---- the door for libko_harness.so (ko_harness.h): tuning table, planners, workspace table, last error
+namespace ko {
+namespace {
+int hook_set_tuning(const char *name, int value) {
+    if (!name) return fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: null name");
+    const int k = find_knob(name);
+    if (k < 0) return fail(KO_ERR_INVALID_ARGUMENT, "ko_set_tuning: unknown knob \"%s\"", name);
+    g_knobs[k].store(value, std::memory_order_relaxed);
     return KO_OK;
 }
 
-KO_EXPORT int ko_get_tuning(const char *name, int *value) {
-    if (!name || !value) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: null argument");
-    const int k = ko::find_knob(name);
-    if (k < 0) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: unknown knob \"%s\"", name);
-    *value = ko::g_knobs[k].load(std::memory_order_relaxed);
+int hook_get_tuning(const char *name, int *value) {
+    if (!name || !value) return fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: null argument");
+    const int k = find_knob(name);
+    if (k < 0) return fail(KO_ERR_INVALID_ARGUMENT, "ko_get_tuning: unknown knob \"%s\"", name);
+    *value = g_knobs[k].load(std::memory_order_relaxed);
     return KO_OK;
 }
+
+int hook_set_last_error(int status, const char *message) { return fail(status, "%s", message ? message : ""); }
+
+const ko_harness_hooks_t kHooks = {hook_set_tuning, hook_get_tuning, debug_sgemm_plan, debug_gemm16_plan,
+                                   stream_workspace_count, hook_set_last_error};
+}  // namespace
+}  // namespace ko
+
+KO_EXPORT const ko_harness_hooks_t *ko_harness_hooks(void) { return &ko::kHooks; }
 
 KO_EXPORT int ko_device_info(ko_device_info_t *info) {
     if (!info) return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_device_info: null info");
@@ -237,6 +274,10 @@ KO_EXPORT int ko_stream_create(ko_stream_t *stream) {
 
 KO_EXPORT int ko_stream_destroy(ko_stream_t stream) {
     if (!stream) return KO_OK;
+    // The stream's workspace goes with it (the reference's Tensor frees what it allocated, common/tensor.cu:23-26):
+    // first wait for the launches that may still read or write it.
+    KO_HIP(hipStreamSynchronize(ko::as_stream(stream)));
+    if (const int st = ko::release_stream_workspace(ko::as_stream(stream)); st != KO_OK) return st;
     KO_HIP(hipStreamDestroy(ko::as_stream(stream)));
     return KO_OK;
 }

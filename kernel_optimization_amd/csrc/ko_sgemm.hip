@@ -717,7 +717,9 @@ int launch_direct(Params p, hipStream_t stream) {
 }
 
 // D = alpha * (P_0 + P_1 + ... + P_{slices-1}) + beta * C over the M x N partial products a K-sliced launch
-// left behind `partials`, summed in slice order whatever order the slices finished in.
+// left behind `partials`, summed in slice order whatever order the slices finished in.  slices == 0 is the
+// empty product (k == 0): nothing is read through `partials` and D = beta * C, or zero without a C - what the
+// reference's kernel leaves when its main loop runs no K tile (simt_gemm.h:325-354).
 // One 64-lane workgroup per 256 outputs: the problems that are sliced have few outputs, and small
 // workgroups spread them over more compute units.  The partial products of eight slices are fetched together
 // (they come from memory behind the L2s: another XCD wrote them) and added one after the other.
@@ -732,7 +734,8 @@ __global__ __launch_bounds__(64) void sgemm_slices_sum_kernel(const float *__res
     if (i >= count) return;
     const float *src = partials + i;
     if (i + 4 <= count) {
-        vec_t acc = *reinterpret_cast<const vec_any_t *>(src);
+        vec_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (slices > 0) acc = *reinterpret_cast<const vec_any_t *>(src);
         int s = 1;
         for (; s + 8 <= slices; s += 8) {
             vec_t v[8];
@@ -747,7 +750,7 @@ __global__ __launch_bounds__(64) void sgemm_slices_sum_kernel(const float *__res
         __builtin_nontemporal_store(acc, reinterpret_cast<vec_any_t *>(D + i));
     } else {
         for (int64_t e = i; e < count; ++e) {  // the last one to three outputs
-            float acc = partials[e];
+            float acc = slices > 0 ? partials[e] : 0.0f;
             for (int s = 1; s < slices; ++s) acc += partials[e + s * count];
             acc *= alpha;
             if (C != nullptr && beta != 0.0f) acc += beta * C[e];
@@ -949,9 +952,12 @@ int sgemm(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const fl
     if (m < 0 || n < 0 || k < 0)
         return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
     if (m == 0 || n == 0) return KO_OK;
-    if (k == 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: k must be positive");
     if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30)) return fail(KO_ERR_UNSUPPORTED_SHAPE, "sgemm: dimension too large");
-    if (!A || !B || !D) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
+    if (!D || (k > 0 && (!A || !B))) return fail(KO_ERR_INVALID_ARGUMENT, "sgemm: null A/B/D pointer");
+    if (k == 0) {  // the empty product: D = beta * C (one scale-and-copy launch; A and B are not touched)
+        const Params empty{A, B, C, D, static_cast<int>(m), static_cast<int>(n), 0, alpha, beta, 0, 0, 0, 0};
+        return sum_slices(nullptr, 0, empty, as_stream(stream));
+    }
     Params p{A, B, C, D, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), alpha, beta, 0, 0, static_cast<int>(k), 0};
     hipStream_t s = as_stream(stream);
     const int variant = tuning(knob_sgemm_variant);
@@ -1010,10 +1016,10 @@ KO_EXPORT int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float
     return ko::sgemm(m, n, k, alpha, A, B, beta, C, D, stream, true);
 }
 
-KO_EXPORT int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant) {
+int ko::debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant) {
     using namespace ko;
     if (!slices || !k_slice || !variant || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
-        return fail(KO_ERR_INVALID_ARGUMENT, "ko_debug_sgemm_plan: bad argument");
+        return fail(KO_ERR_INVALID_ARGUMENT, "sgemm_plan: bad argument");
     // operands that the planner takes for 16-byte aligned; nothing is read through them
     const float *aligned = reinterpret_cast<const float *>(uintptr_t{256});
     const Params p{aligned, aligned, nullptr, nullptr, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),

@@ -934,32 +934,3 @@ KO_EXPORT int ko_softmax_16(const void *in, void *out, int64_t rows, int64_t col
     if (dtype == KO_BF16) return ko::entry<ko::IO_BF16>(in, out, rows, cols, valid_len, rows_per_seq, policy, stream);
     return ko::fail(KO_ERR_INVALID_ARGUMENT, "softmax: dtype=%d is neither KO_F16 nor KO_BF16", dtype);
 }
-
-// ---- cross-lane primitive check (see ko.h)
-namespace ko {
-namespace {
-template <int G>
-__global__ void wave_allreduce_kernel(const float *in, float *out, int op) {
-    float v = in[threadIdx.x];
-    out[threadIdx.x] = op == 0 ? wave::allreduce<G, wave::Max>(v) : wave::allreduce<G, wave::Sum>(v);
-}
-}  // namespace
-}  // namespace ko
-
-KO_EXPORT int ko_debug_wave_allreduce(const float *in, float *out, int group, int op,
-                                      ko_stream_t stream) {
-    if (!in || !out) return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: null pointer");
-    if (op != 0 && op != 1) return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: op=%d", op);
-    hipStream_t s = ko::as_stream(stream);
-    switch (group) {
-        case 2: ko::wave_allreduce_kernel<2><<<1, 64, 0, s>>>(in, out, op); break;
-        case 4: ko::wave_allreduce_kernel<4><<<1, 64, 0, s>>>(in, out, op); break;
-        case 8: ko::wave_allreduce_kernel<8><<<1, 64, 0, s>>>(in, out, op); break;
-        case 16: ko::wave_allreduce_kernel<16><<<1, 64, 0, s>>>(in, out, op); break;
-        case 32: ko::wave_allreduce_kernel<32><<<1, 64, 0, s>>>(in, out, op); break;
-        case 64: ko::wave_allreduce_kernel<64><<<1, 64, 0, s>>>(in, out, op); break;
-        default: return ko::fail(KO_ERR_INVALID_ARGUMENT, "wave_allreduce: group=%d", group);
-    }
-    KO_CHECK_LAUNCH();
-    return KO_OK;
-}

@@ -16,28 +16,46 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "kernel_optimization_amd", "bin")
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "ko.h")).read()
+def _declared_symbols(header="ko.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(ko_[a-z0-9_]+)\s*\(", text)))
 
 
+def _exported(path):
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return set(re.findall(r"\sT\s+(ko_[a-z0-9_]+)", out))
+
+
 def test_library_exports_every_declared_symbol():
+    """libko.so exports what ko.h declares - runtime, operators, the entry that allocates nothing - and one door
+    for the harness library; nothing of the harness (fills, probes, knobs, debug views) is in it."""
     names = _declared_symbols()
     assert len(names) >= 30
-    out = subprocess.run(["nm", "-D", "--defined-only", ko.LIB_PATH], capture_output=True, text=True, check=True).stdout
-    exported = set(re.findall(r"\sT\s+(ko_[a-z0-9_]+)", out))
+    exported = _exported(ko.LIB_PATH)
     assert set(names) <= exported, sorted(set(names) - exported)
-    assert exported <= set(names), "exported but not declared in ko.h: %s" % sorted(exported - set(names))
+    assert exported - set(names) == {"ko_harness_hooks"}, sorted(exported - set(names))
     assert set(ko.SIGNATURES) == set(names)
+    assert not [n for n in names if re.match(r"ko_(fill|copy|debug|stream_probe|set_tuning|get_tuning)", n)]
     lib = ko.lib()
     for n in names:
         getattr(lib, n)
 
 
+def test_harness_library_exports_every_declared_symbol():
+    names = set(_declared_symbols("ko_harness.h")) - {"ko_harness_hooks"}
+    exported = _exported(ko.HARNESS_PATH)
+    assert names == exported, sorted(names ^ exported)
+    assert set(ko.HARNESS_SIGNATURES) == names
+    h = ko.harness()
+    for n in names:
+        getattr(h, n)
+
+
 def test_header_is_plain_c(tmp_path):
     src = tmp_path / "t.c"
-    src.write_text('#include "ko.h"\nint main(void) { return (int)KO_OK + (int)sizeof(ko_device_info_t) * 0; }\n')
+    src.write_text('#include "ko.h"\n#include "ko_harness.h"\n'
+                   'int main(void) { return (int)KO_OK + (int)sizeof(ko_device_info_t) * 0; }\n')
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), "-c",
                     str(src), "-o", str(tmp_path / "t.o")], check=True)
 
@@ -54,7 +72,8 @@ def test_status_names_and_argument_errors_without_device():
     assert lib.ko_layernorm_f32(None, None, None, None, None, None, 4, 770, 1e-5, 0, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert lib.ko_sgemm_f32(-1, 1, 1, 1.0, None, None, 0.0, None, None, None) == ko.KO_ERR_INVALID_ARGUMENT
     assert lib.ko_gemm_f16f32acc(8, 8, 12, 1.0, 1, 1, 1, 0.0, None, 1, 0, None) == ko.KO_ERR_UNSUPPORTED_SHAPE
-    assert lib.ko_set_tuning(b"no.such.knob", 1) == ko.KO_ERR_INVALID_ARGUMENT
+    assert ko.harness().ko_set_tuning(b"no.such.knob", 1) == ko.KO_ERR_INVALID_ARGUMENT
+    assert "no.such.knob" in ko.last_error()  # the harness library reports through libko.so's last-error slot
     ko.set_tuning("softmax.lanes_per_row", 16)
     assert ko.get_tuning("softmax.lanes_per_row") == 16
     ko.set_tuning("softmax.lanes_per_row", 0)

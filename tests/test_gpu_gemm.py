@@ -815,3 +815,62 @@ def test_sgemm_shallow_k_is_exact_on_small_integers(ko, m, n, k):
     ref = A.astype(np.float64) @ B.astype(np.float64)
     np.testing.assert_array_equal(ko.sgemm_host(A, B), ref)
     np.testing.assert_array_equal(ko.sgemm_host(A, B, C, 2.0, -1.0), 2.0 * ref - C)
+
+
+@pytest.mark.parametrize("m,n", [(64, 64), (37, 50), (1, 3), (300, 1027)])
+def test_sgemm_empty_product(ko, m, n):
+    """k == 0: the reference's kernel runs no K tile and its epilogue leaves D = C, or zero without a C
+    (simt_gemm.h:325-354).  Here D = beta * C in one launch; A and B are not touched and may be null."""
+    C = inputs.normal_f32((m, n), 5 + m)
+    dC, dD = ko.DeviceBuffer.from_numpy(C), ko.DeviceBuffer(m * n * 4)
+    for c, alpha, beta, want in ((dC, 1.0, 1.0, C), (dC, 3.0, -0.5, np.float32(-0.5) * C), (dC, 1.0, 0.0, np.zeros_like(C)),
+                                 (None, 2.0, 1.0, np.zeros_like(C))):
+        dD.upload(np.full(m * n, np.nan, np.float32))
+        ko.sgemm(m, n, 0, None, None, dD, c, alpha, beta)
+        ko.sgemm_static_scratch(m, n, 0, None, None, dD, c, alpha, beta)
+        ko.synchronize()
+        np.testing.assert_array_equal(dD.download(np.float32, (m, n)), want)
+    ko.sgemm(m, n, 0, None, None, dC, dC, 1.0, 2.0)  # in place
+    ko.synchronize()
+    np.testing.assert_array_equal(dC.download(np.float32, (m, n)), np.float32(2.0) * C)
+    with pytest.raises(ko.KoError):
+        ko.sgemm(m, n, 0, None, None, None)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("m,n", [(64, 64), (37, 50), (5, 3), (130, 1032)])
+def test_gemm16_empty_product(ko, bf16, m, n):
+    """k == 0 on the 16-bit entries: D = activation(beta * C + bias), evaluated in fp32 and rounded once - the
+    oracle's epilogue on an accumulator of zero."""
+    import oracle
+    dt = ko.BF16 if bf16 else ko.F16
+    if bf16:
+        C, bias = inputs.uniform_bf16_bits((m, n), 7 + m, -2.0, 2.0), inputs.uniform_bf16_bits((n,), 8 + m, -1.0, 1.0)
+    else:
+        C = inputs.uniform_f16((m, n), 7 + m, -2.0, 2.0).view(np.uint16)
+        bias = inputs.uniform_f16((n,), 8 + m, -1.0, 1.0).view(np.uint16)
+    c64, b64 = _to_f64(C, bf16), _to_f64(bias, bf16)
+    dC, dB, dD = ko.DeviceBuffer.from_numpy(C), ko.DeviceBuffer.from_numpy(bias), ko.DeviceBuffer(m * n * 2)
+    for use_c, beta, use_bias, act in ((True, 1.0, False, ko.ACT_NONE), (True, -0.5, True, ko.ACT_NONE),
+                                       (False, 0.0, False, ko.ACT_NONE), (True, 1.5, True, ko.ACT_GELU_ERF),
+                                       (False, 0.0, True, ko.ACT_GELU_TANH)):
+        dD.upload(np.full(m * n, 0x7e00, np.uint16))
+        ko.gemm16(m, n, 0, None, None, dD, C=dC if use_c else None, alpha=2.0, beta=beta, dtype=dt,
+                  bias=dB if use_bias else None, act=act)
+        ko.synchronize()
+        got = _to_f64(dD.download(np.uint16, (m, n)), bf16)
+        pre = (np.float32(beta) * c64.astype(np.float32) if use_c else np.zeros((m, n), np.float32)).astype(np.float64)
+        if use_bias:
+            pre = (pre.astype(np.float32) + b64.astype(np.float32)[None, :]).astype(np.float64)
+        if act == ko.ACT_GELU_ERF:
+            from scipy.special import erf
+            want = 0.5 * pre * (1.0 + erf(pre / np.sqrt(2.0)))
+        elif act == ko.ACT_GELU_TANH:
+            want = 0.5 * pre * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (pre + 0.044715 * pre ** 3)))
+        else:
+            want = pre
+        ulp = 2.0 ** -8 if bf16 else 2.0 ** -11
+        assert np.all(np.abs(got - want) <= ulp * np.abs(want) + (1e-5 if act else 1e-6)), (use_c, beta, use_bias, act)
+        if act == ko.ACT_NONE and not use_bias:  # one rounding of an exactly representable product chain: exact
+            exact = pre if use_c else np.zeros((m, n))
+            assert np.all(np.abs(got - exact) <= ulp * np.abs(exact))

@@ -16,7 +16,7 @@ def test_wave_allreduce_primitives(ko):
     dx, dy = ko.DeviceBuffer.from_numpy(x), ko.DeviceBuffer(256)
     for g in (2, 4, 8, 16, 32, 64):
         for op, fn in ((0, np.max), (1, np.sum)):
-            ko.check(ko.lib().ko_debug_wave_allreduce(dx.ptr, dy.ptr, g, op, None))
+            ko.check(ko.harness().ko_debug_wave_allreduce(dx.ptr, dy.ptr, g, op, None))
             ko.synchronize()
             got = dy.download(np.float32, (64,))
             want = np.repeat(fn(x.reshape(64 // g, g), axis=1), g)
@@ -167,8 +167,8 @@ def test_softmax_errors(ko):
     assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE and "mask" in str(e.value)
 
 
-def test_softmax_full_size_cfg1_properties(ko):
-    """[196608,128] at full size, inputs filled on the device: sampled rows against the oracle on the
+def test_softmax_full_size_cfg1(ko):
+    """[196608,128] at full size, inputs filled on the device: the whole output against the oracle on the
     very bytes the kernel read, plus size-independent properties over the whole output."""
     rows, cols = 196608, 128
     n = rows * cols
@@ -181,9 +181,8 @@ def test_softmax_full_size_cfg1_properties(ko):
     assert np.all(np.isfinite(y)) and y.min() >= 0
     assert np.abs(y.sum(1, dtype=np.float64) - 1).max() <= cols * 2.0 ** -24
     assert np.array_equal(y[np.arange(rows), x.argmax(1)], y.max(1))  # order preserved at the top
-    idx = np.random.default_rng(0).choice(rows, 4096, replace=False)
-    idx = np.concatenate([idx, [0, 1, 2, 3, rows - 4, rows - 3, rows - 2, rows - 1]])
-    assert_softmax_close(y[idx], oracle.softmax(x[idx]))
+    for r0 in range(0, rows, 32768):
+        assert_softmax_close(y[r0:r0 + 32768], oracle.softmax(x[r0:r0 + 32768]))
     # the device fill is the same generator as the host one
     host = inputs.normal_f32((64, cols), inputs.tensor_seed(1, 0), 0.0, 4.0)
     assert np.all(np.abs(host - x[:64]) <= 2.0 ** -22 * np.maximum(np.abs(host), 1.0))

@@ -167,6 +167,52 @@ def test_sgemm_whose_first_sliced_call_is_captured_allocates_nothing(ko):
     np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))
 
 
+def _workspaces(ko):
+    n = ctypes.c_int()
+    ko.check(ko.harness().ko_debug_stream_workspace_count(ctypes.byref(n)))
+    return n.value
+
+
+def test_stream_destroy_releases_the_workspace(ko):
+    """ko_stream_destroy frees the 32 MiB workspace a K-sliced call gave the stream: a process that creates and
+    destroys more streams than the workspace table has entries (64) keeps the sliced path - same bits as on the
+    first stream - and holds no more workspaces afterwards than before."""
+    m, n, k = 256, 256, 2048
+    assert ko.gemm_plan(m, n, k)[0] > 1 and ko.gemm_plan(m, n, k, sixteen_bit=True)[0] > 1
+    A, B = inputs.uniform_f32((m, k), 41), inputs.uniform_f32((k, n), 42)
+    dA, dB = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B)
+    A16 = inputs.uniform_f16((m, k), 43).view(np.uint16)
+    B16 = inputs.uniform_f16((n, k), 44).view(np.uint16)
+    dA16, dB16 = ko.DeviceBuffer.from_numpy(A16), ko.DeviceBuffer.from_numpy(B16)
+    ko.set_tuning("sgemm.k_slices", 1)
+    try:
+        unsliced = ko.DeviceBuffer(m * n * 4)
+        ko.sgemm(m, n, k, dA, dB, unsliced)
+        ko.synchronize()
+        unsliced = unsliced.download(np.uint32, (m, n))
+    finally:
+        ko.set_tuning("sgemm.k_slices", 0)
+    base = _workspaces(ko)
+    first = first16 = None
+    for i in range(70):
+        stream = ko.Stream()
+        dD, dD16 = ko.DeviceBuffer(m * n * 4), ko.DeviceBuffer(m * n * 2)
+        ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
+        assert _workspaces(ko) == base + 1, i
+        ko.gemm16(m, n, k, dA16, dB16, dD16, stream=stream)
+        assert _workspaces(ko) == base + 1, i
+        stream.close()  # waits for the work, then frees the workspace
+        assert _workspaces(ko) == base, i
+        got, got16 = dD.download(np.uint32, (m, n)), dD16.download(np.uint16, (m, n))
+        if first is None:
+            first, first16 = got, got16
+            assert not np.array_equal(first, unsliced)  # the sliced sum rounds differently: that path really ran
+        np.testing.assert_array_equal(got, first, err_msg="stream %d" % i)
+        np.testing.assert_array_equal(got16, first16, err_msg="stream %d" % i)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    assert np.abs(first.view(np.float32) - ref).max() <= 2 * k * 2.0 ** -24 * (np.abs(A) @ np.abs(B)).max()
+
+
 def test_operators_from_two_threads_on_two_streams(ko):
     """Thread-compatible entry points: two host threads, each with its own stream and buffers, run the row
     operators and the GEMMs at the same time; every result equals the single-threaded one bit for bit."""

@@ -3,6 +3,9 @@ ABI: the same kernels with the partial products of a K-sliced problem in the lib
 instead of an allocated workspace, so the outputs must be the same bits.  Two calls in a row share the array, the
 second on a smaller problem (what the first left behind must not reach the second's sum); a problem that is not
 sliced takes the same path in both entry points; a slice plan that does not fit the array is refused."""
+import ctypes
+import re
+
 import numpy as np
 import pytest
 
@@ -57,3 +60,85 @@ def test_static_scratch_sgemm_refuses_what_does_not_fit(ko):
     with pytest.raises(ko.KoError) as e:
         ko.sgemm_static_scratch(16, 16, 16, None, buf, out)
     assert e.value.status == ko.KO_ERR_INVALID_ARGUMENT
+
+
+def _hip_runtime():
+    """The libamdhip64 this process already has loaded (through libko.so)."""
+    with open("/proc/self/maps") as f:
+        paths = sorted(set(re.findall(r"(/\S*libamdhip64\.so[\w.]*)", f.read())))
+    assert paths
+    hip = ctypes.CDLL(paths[0])
+    vp = ctypes.c_void_p
+    hip.hipStreamBeginCapture.argtypes = [vp, ctypes.c_int]
+    hip.hipStreamEndCapture.argtypes = [vp, ctypes.POINTER(vp)]
+    hip.hipGraphInstantiate.argtypes = [ctypes.POINTER(vp), vp, vp, vp, ctypes.c_size_t]
+    hip.hipGraphLaunch.argtypes = [vp, vp]
+    hip.hipGraphExecDestroy.argtypes = [vp]
+    hip.hipGraphDestroy.argtypes = [vp]
+    hip.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    return hip
+
+
+def _free_bytes(hip):
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_static_scratch_sgemm_allocates_nothing_and_slices_under_capture(ko):
+    """What the entry point is for.  On a fresh stream, which has no workspace: a sliced call through it leaves
+    the device's free memory and the library's workspace table as they were, and the same call captured into a
+    graph still takes the sliced path (the allocating entry point, captured first on such a stream, falls back to
+    the unsliced kernels): every replay gives the bits of the eager sliced result."""
+    ko.lib()
+    hip = _hip_runtime()
+    m, n, k = 256, 256, 2048
+    assert ko.gemm_plan(m, n, k)[0] > 1
+    A, B = inputs.uniform_f32((m, k), 31), inputs.uniform_f32((k, n), 32)
+    dA, dB = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B)
+    sliced, unsliced, dD = ko.DeviceBuffer(m * n * 4), ko.DeviceBuffer(m * n * 4), ko.DeviceBuffer(m * n * 4)
+    ko.sgemm(m, n, k, dA, dB, sliced)  # default stream: its workspace exists after this call
+    ko.set_tuning("sgemm.k_slices", 1)
+    try:
+        ko.sgemm(m, n, k, dA, dB, unsliced)
+    finally:
+        ko.set_tuning("sgemm.k_slices", 0)
+    ko.sgemm_static_scratch(m, n, k, dA, dB, dD)  # the one-time symbol lookup, outside any capture
+    ko.synchronize()
+    want = sliced.download(np.uint32, (m, n))
+    assert not np.array_equal(want, unsliced.download(np.uint32, (m, n)))  # the two paths round differently
+
+    stream = ko.Stream()
+    count = ctypes.c_int()
+    ko.check(ko.harness().ko_debug_stream_workspace_count(ctypes.byref(count)))
+    before_count, before_free = count.value, _free_bytes(hip)
+    dD.upload(np.zeros(m * n, np.float32))
+    ko.sgemm_static_scratch(m, n, k, dA, dB, dD, stream=stream)
+    stream.synchronize()
+    assert _free_bytes(hip) == before_free
+    ko.check(ko.harness().ko_debug_stream_workspace_count(ctypes.byref(count)))
+    assert count.value == before_count
+    np.testing.assert_array_equal(dD.download(np.uint32, (m, n)), want)
+
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 0) == 0
+    try:
+        ko.sgemm_static_scratch(m, n, k, dA, dB, dD, stream=stream)
+    finally:
+        rc = hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
+    try:
+        for replay in range(3):
+            dD.upload(np.zeros(m * n, np.float32))
+            assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+            stream.synchronize()
+            np.testing.assert_array_equal(dD.download(np.uint32, (m, n)), want, err_msg="replay %d" % replay)
+            ko.sgemm_static_scratch(100, 72, 1300, dA, dB, unsliced)  # eager work on the array between replays
+            ko.synchronize()
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+    ko.check(ko.harness().ko_debug_stream_workspace_count(ctypes.byref(count)))
+    assert count.value == before_count
+    stream.close()
