@@ -412,6 +412,66 @@ def bench_rows16(kind, dtype_name, steps, warmup):
     return res
 
 
+def bench_short_kernels(steps, warmup):
+    """Where the time of the two short configurations goes: the row count of softmax [196608, 128] and LayerNorm
+    [16384, 768] times 1, 2, 4, 8 and 16 next to the plain copy of the same bytes, with the straight line through
+    the five points (intercept: what a launch costs whatever its size; slope: the rate the kernel streams at), the
+    price of gamma and beta, and what a plain copy reaches when a wavefront holds as many bytes as a row."""
+    out = dict(steps=steps, warmup=warmup, lines={}, points=[])
+
+    def median_us(launch):
+        runs = []
+        for _ in range(5):
+            _, dev = _time_steps(launch, steps, warmup)
+            runs.append(dev * 1e6)
+        return float(np.median(runs))
+
+    def sets(nbytes):
+        nsets = max(2, -(-(1 << 30) // (2 * nbytes)))
+        xs = [ko.DeviceBuffer(nbytes) for _ in range(nsets)]
+        ys = [ko.DeviceBuffer(nbytes) for _ in range(nsets)]
+        for x in xs:
+            ko.fill_normal_f32(x, nbytes // 4, 1, 0.5, 2.0)
+        return xs, ys, nsets
+
+    for op, rows0, cols in (("softmax", 196608, 128), ("layernorm", 16384, 768)):
+        g, b = ko.DeviceBuffer(cols * 4), ko.DeviceBuffer(cols * 4)
+        ko.fill_normal_f32(g, cols, 2, 1.0, 0.1)
+        ko.fill_normal_f32(b, cols, 3, 0.0, 0.1)
+        for kind in (op, "copy") + (("layernorm_no_gamma_beta",) if op == "layernorm" else ()):
+            pts = []
+            for mult in (1, 2, 4, 8, 16):
+                rows = rows0 * mult
+                n = rows * cols
+                xs, ys, ns = sets(n * 4)
+                m, r = ko.DeviceBuffer(rows * 4), ko.DeviceBuffer(rows * 4)
+                if kind == "copy":
+                    us = median_us(lambda i: ko.copy_f32(xs[i % ns], ys[i % ns], n))
+                elif kind == "softmax":
+                    us = median_us(lambda i: ko.softmax(xs[i % ns], ys[i % ns], rows, cols))
+                elif kind == "layernorm":
+                    us = median_us(lambda i: ko.layernorm(xs[i % ns], ys[i % ns], rows, cols, m, r, g, b, 1e-5))
+                else:
+                    us = median_us(lambda i: ko.layernorm(xs[i % ns], ys[i % ns], rows, cols, m, r, None, None, 1e-5))
+                pts.append((2 * n * 4, us))
+                out["points"].append(dict(kernel=kind, rows=rows, cols=cols, bytes=2 * n * 4, us=us,
+                                          gbps=2 * n * 4 / us / 1e3))
+                del xs, ys
+            slope, intercept = np.polyfit([p[0] for p in pts], [p[1] for p in pts], 1)
+            out["lines"]["%s_%dcols" % (kind, cols)] = dict(intercept_us=float(intercept), slope_gbps=float(1e-3 / slope))
+    # a plain copy whose wavefronts hold 1, 2 and 4 vectors per lane, and whose workgroups hold 3 KB and 6 KB
+    n = 262144 * 768
+    xs, ys, ns = sets(n * 4)
+    out["copy_by_footprint"] = []
+    for threads, vpt in ((64, 1), (64, 2), (64, 4), (128, 1), (192, 1), (256, 1), (384, 1)):
+        for pad in (0, 10240):
+            us = median_us(lambda i: ko.stream_probe(xs[i % ns], ys[i % ns], n * 4, ko.PROBE_COPY, vectors_per_thread=vpt,
+                                                     threads=threads, load_policy=1, store_policy=3, lds_pad_bytes=pad))
+            out["copy_by_footprint"].append(dict(threads=threads, vectors_per_thread=vpt, lds_pad_bytes=pad, us=us,
+                                                 gbps=2 * n * 4 / us / 1e3))
+    return out
+
+
 def run_workload(cfg, steps, warmup, vendor):
     op = inputs.CONFIGS[cfg]["op"]
     if op == "softmax":
@@ -729,7 +789,7 @@ def main():
                     help="untimed launches before the timed ones; the device takes a few hundred short launches "
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
     ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"],
-                    help="one of %s, copy_f32, hbm_ceilings, softmax_f32_786432x512_unmasked, or a long-row line by name: "
+                    help="one of %s, copy_f32, hbm_ceilings, short_kernels, softmax_f32_786432x512_unmasked, or a long-row line by name: "
                          "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache)" % ", ".join(sorted(WORKLOADS)))
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
@@ -748,6 +808,9 @@ def main():
         return
     if args.workload == "hbm_ceilings":  # the whole streaming sweep, for profiles/
         print(json.dumps(bench_ceilings(min(args.steps, 10), 3, full=True)))
+        return
+    if args.workload == "short_kernels":  # intercept and slope of the two short configurations, for profiles/
+        print(json.dumps(bench_short_kernels(min(args.steps, 30), max(args.warmup, 100))))
         return
     if args.workload == "softmax_f32_786432x512_unmasked":  # for the traffic counters and traces
         res, _ = bench_softmax(5, args.steps, args.warmup, unmasked=True)
