@@ -44,7 +44,10 @@ typedef enum ko_status {
  * AUTO  = chosen from the row length: the first of the three that holds the row.
  * Longest rows: WARP 2048 fp32 / 4096 16-bit columns; BLOCK softmax 135168 fp32 / 172032 16-bit columns
  * (98304 columns with a padding mask), LayerNorm any length (what the chip does not hold is read twice);
- * BLOCK_NOCACHE any length.  A policy asked for explicitly on a longer row returns KO_ERR_UNSUPPORTED_SHAPE. */
+ * BLOCK_NOCACHE any length.  Rows that are walked element by element (a row length that is not a whole number of
+ * 16-byte vectors, or tensors off 16-byte boundaries): WARP 2048 columns, BLOCK softmax 65536 columns, LayerNorm
+ * any length.  A policy asked for explicitly runs that policy's kernel; on a longer row than it holds it returns
+ * KO_ERR_UNSUPPORTED_SHAPE. */
 typedef enum ko_policy {
     KO_POLICY_AUTO = 0,
     KO_POLICY_WARP = 1,

@@ -1048,10 +1048,23 @@ int launch_block_by_element(const Args<IO> &a) {
 // Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
 // 16 or 64 lanes (column j in lane j % lanes, slot j / lanes), up to 65536 in those of a workgroup, and is read
 // once; of longer rows the far end is read twice.
+// An explicit policy is honoured: WARP takes the wavefront kernels (up to 2048 columns here), BLOCK the workgroup
+// kernel, BLOCK_NOCACHE the one that reads every row twice; AUTO the first that holds the row.
 template <int IO>
-int launch_by_element(const Args<IO> &a) {
+int launch_by_element(const Args<IO> &a, int policy) {
     static_assert(Io<IO>::E == 1, "");
     const int cols = a.cols;
+    if (policy == KO_POLICY_BLOCK_NOCACHE) return launch_nocache<IO>(a);
+    if (policy == KO_POLICY_WARP && cols > 2048)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "layernorm: WARP policy holds at most 2048 columns of a row walked "
+                                              "element by element, got %d", cols);
+    if (policy == KO_POLICY_BLOCK) {
+        if (cols <= 4096) return launch_block_by_element<IO, 4, false>(a);
+        if (cols <= 8192) return launch_block_by_element<IO, 8, false>(a);
+        if (cols <= 16384) return launch_block_by_element<IO, 16, false>(a);
+        if (cols <= 32768) return launch_block_by_element<IO, 32, false>(a);
+        return launch_block_by_element<IO, 64, true>(a);
+    }
     if (cols <= 1) return launch_wave_full<IO, 1, 1, false>(a);  // rows of a few columns: as many lanes as columns
     if (cols <= 2) return launch_wave_full<IO, 2, 1, false>(a);
     if (cols <= 4) return launch_wave_full<IO, 4, 1, false>(a);
@@ -1136,7 +1149,7 @@ int entry(const void *in, void *out, float *mean, float *rstd, const void *gamma
         Args<BY_ELEMENT> a1{static_cast<const elem *>(in), static_cast<elem *>(out), mean, rstd,
                             static_cast<const elem *>(gamma), static_cast<const elem *>(beta), rows,
                             static_cast<int>(cols), eps, static_cast<float>(1.0 / denom), as_stream(stream)};
-        return launch_by_element<BY_ELEMENT>(a1);
+        return launch_by_element<BY_ELEMENT>(a1, policy);
     }
     Args<IO> a{static_cast<const elem *>(in), static_cast<elem *>(out), mean, rstd, static_cast<const elem *>(gamma),
                static_cast<const elem *>(beta), rows, static_cast<int>(cols), eps, static_cast<float>(1.0 / denom),

@@ -811,6 +811,12 @@ int run(Params p, hipStream_t s, int variant) {
         const bool aligned = ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&
                              p.lda % 4 == 0 && p.N % 4 == 0 && p.K % 4 == 0;
         if (!aligned && variant == 40) variant = 36;
+        // a slice of K (a forced slice count can bring one here with any depth): only the direct-to-LDS kernels
+        // take slices, so the register pipeline's shapes go to the direct-to-LDS kernel of the same tile
+        if (p.k_slice > 0) {
+            if (variant == 13) variant = 33;
+            if (variant == 16) variant = 36;
+        }
     }
     switch (variant) {
         case 13: return launch<64, 64, 64, 2, 2, 4, true>(p, s);

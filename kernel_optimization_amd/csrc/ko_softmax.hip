@@ -787,10 +787,25 @@ int launch_block_by_element(const Args<IO> &a) {
 // Rows walked element by element (IO is one of the *_1 kinds): up to 2048 columns a row sits in the registers of
 // 16 or 64 lanes (column j in lane j % lanes, slot j / lanes), up to 65536 in those of a workgroup, and is read
 // once; longer rows are read twice.
+// An explicit policy is honoured: WARP takes the wavefront kernels (up to 2048 columns here), BLOCK the workgroup
+// kernel (up to 65536 columns), BLOCK_NOCACHE the one that reads twice; AUTO the first that holds the row.
 template <int IO, bool MASKED>
-int launch_by_element(const Args<IO> &a) {
+int launch_by_element(const Args<IO> &a, int policy) {
     static_assert(Io<IO>::E == 1, "");
     const int cols = a.cols;
+    if (policy == KO_POLICY_BLOCK_NOCACHE) return launch_nocache<IO, MASKED>(a);
+    if (policy == KO_POLICY_WARP && cols > 2048)
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: WARP policy holds at most 2048 columns of a row walked element "
+                                              "by element, got %d", cols);
+    if (policy == KO_POLICY_BLOCK) {
+        if (cols <= 4096) return launch_block_by_element<IO, 4, MASKED>(a);
+        if (cols <= 8192) return launch_block_by_element<IO, 8, MASKED>(a);
+        if (cols <= 16384) return launch_block_by_element<IO, 16, MASKED>(a);
+        if (cols <= 32768) return launch_block_by_element<IO, 32, MASKED>(a);
+        if (cols <= 65536) return launch_block_by_element<IO, 64, MASKED>(a);
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "softmax: BLOCK policy holds at most 65536 columns of a row walked "
+                                              "element by element, got %d", cols);
+    }
     if constexpr (!MASKED) {  // rows of a few columns: as many lanes as columns, up to 64 rows per wavefront
         if (cols <= 1) return launch_wave<IO, 1, 1, false, true>(a);
         if (cols <= 2) return launch_wave<IO, 2, 1, false, true>(a);
@@ -907,7 +922,7 @@ int entry(const void *in, void *out, int64_t rows, int64_t cols, const int32_t *
                         (valid_len ? 1024 * (96 / E) : kBlockMaxVecs<IO>) * E, valid_len ? " with a mask" : "", (long long)cols);
         Args<BY_ELEMENT> a{static_cast<const typename Io<IO>::elem *>(in), static_cast<typename Io<IO>::elem *>(out), rows,
                            static_cast<int>(cols), valid_len, rows_per_seq, as_stream(stream)};
-        return valid_len ? launch_by_element<BY_ELEMENT, true>(a) : launch_by_element<BY_ELEMENT, false>(a);
+        return valid_len ? launch_by_element<BY_ELEMENT, true>(a, policy) : launch_by_element<BY_ELEMENT, false>(a, policy);
     }
     Args<IO> a{static_cast<const typename Io<IO>::elem *>(in), static_cast<typename Io<IO>::elem *>(out), rows,
                static_cast<int>(cols), valid_len, rows_per_seq, as_stream(stream)};

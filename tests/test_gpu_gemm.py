@@ -874,3 +874,24 @@ def test_gemm16_empty_product(ko, bf16, m, n):
         if act == ko.ACT_NONE and not use_bias:  # one rounding of an exactly representable product chain: exact
             exact = pre if use_c else np.zeros((m, n))
             assert np.all(np.abs(got - exact) <= ulp * np.abs(exact))
+
+
+def test_sgemm_forced_slices_keep_a_kernel_that_takes_them(ko):
+    """A slice count forced through the knob with the tiling left to the shape: 1024 x 2048 x 512 in two slices is a
+    shallow K on many small tiles, the shape class of the register pipeline, which takes no slices - the sliced
+    launch has to go to the direct-to-LDS kernel of the same tile instead of being refused."""
+    m, n, k = 1024, 2048, 512
+    rng = np.random.default_rng(5)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    dA, dB, dD = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B), ko.DeviceBuffer(m * n * 4)
+    for slices in (2, 4):
+        ko.set_tuning("sgemm.k_slices", slices)
+        try:
+            assert ko.gemm_plan(m, n, k)[0] == slices
+            dD.upload(np.full(m * n, np.nan, np.float32))
+            ko.sgemm(m, n, k, dA, dB, dD)
+            ko.synchronize()
+        finally:
+            ko.set_tuning("sgemm.k_slices", 0)
+        np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))

@@ -33,7 +33,7 @@ def test_softmax_rows_of_any_length(ko, rows, cols):
     x = inputs.normal_f32((rows, cols), 700 + cols, 0.0, 4.0)
     ref = oracle.softmax(x)
     for policy in (0, 1, 2, 3):
-        if (policy == 1 and cols > 2048) or (policy == 2 and cols > 135168):
+        if (policy == 1 and cols > 2048) or (policy == 2 and cols > 65536):  # what the policies hold element by element
             with pytest.raises(ko.KoError) as e:
                 ko.softmax_host(x, policy=policy)
             assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
@@ -66,7 +66,12 @@ def test_softmax16_rows_of_any_length(ko, rows, cols, bf16):
     dt = ko.BF16 if bf16 else ko.F16
     xb = _bits(inputs.normal_f32((rows, cols), 720 + cols, 0.0, 4.0), bf16)
     _, ref64 = oracle.softmax16(xb, bf16=bf16)
-    for policy in (0, 3):
+    for policy in (0, 1, 2, 3):
+        if (policy == 1 and cols > 2048) or (policy == 2 and cols > 65536):
+            with pytest.raises(ko.KoError) as e:
+                ko.softmax16_host(xb, dtype=dt, policy=policy)
+            assert e.value.status == ko.KO_ERR_UNSUPPORTED_SHAPE
+            continue
         assert_softmax16_close(_to64(ko.softmax16_host(xb, dtype=dt, policy=policy), bf16), ref64, bf16)
     rps = 2
     vl = np.random.default_rng(cols).integers(0, cols + 1, (rows + rps - 1) // rps).astype(np.int32)
