@@ -472,6 +472,45 @@ def bench_short_kernels(steps, warmup):
     return out
 
 
+MIDSIZE_ROWS = (100, 256, 512, 1000, 2048, 3000, 4096, 6000, 8192, 12000, 20000)
+MIDSIZE_WEIGHTS = ((3072, 768), (768, 3072), (2304, 768), (4096, 4096), (1024, 1024), (4096, 1024), (1024, 4096))
+
+
+def bench_gemm16_midsize(steps, warmup, vendor):
+    """The 16-bit GEMM on token counts from 100 to 20000 against transformer weight shapes (N x K), next to
+    hipBLASLt on the same buffers: time, ratio, and what the host-side planner decided (K slices and their tiling)."""
+    rows = []
+    for n, k in MIDSIZE_WEIGHTS:
+        for m in MIDSIZE_ROWS:
+            res, _ = bench_gemm16(4, steps, warmup, vendor, shape=(m, n, k))
+            slices, k_slice, tile = ko.gemm_plan(m, n, k, sixteen_bit=True)
+            rows.append(dict(m=m, n=n, k=k, us=res["kernel_us"], tflops=res["roofline"]["achieved"]
+                             if res["roofline"]["unit"] == "TFLOP/s" else res["flops"] / res["kernel_us"] / 1e6,
+                             hipblaslt_us=res["flops"] / res["hipblaslt_tflops"] / 1e6 if "hipblaslt_tflops" in res else None,
+                             vs_hipblaslt=res.get("vs_hipblaslt"), k_slices=slices, k_slice=k_slice, slice_tile=tile,
+                             tiles_256=-(-m // 256) * -(-n // 256)))
+    ratios = sorted(r["vs_hipblaslt"] for r in rows if r["vs_hipblaslt"])
+    return dict(steps=steps, warmup=warmup, shapes=len(rows), median_vs_hipblaslt=ratios[len(ratios) // 2] if ratios else None,
+                min_vs_hipblaslt=ratios[0] if ratios else None, max_vs_hipblaslt=ratios[-1] if ratios else None, rows=rows)
+
+
+def bench_gemm16_active_cus(steps, warmup):
+    """Time per K tile of the 256 x 256 kernel of the 16-bit GEMM by how many compute units have a tile: K = 4096
+    (64 K tiles per output tile), N = 3072 (12 tile columns), M from 256 to 16384."""
+    out = []
+    for m in (256, 512, 1024, 2048, 4096, 5376, 10752, 16384):
+        n, k = 3072, 4096
+        res, _ = bench_gemm16(4, steps, warmup, None, shape=(m, n, k))
+        tiles = (m // 256) * (n // 256)
+        cus = ko.device_info()["compute_units"]
+        rounds = -(-tiles // cus)
+        slices = ko.gemm_plan(m, n, k, sixteen_bit=True)[0]
+        out.append(dict(m=m, n=n, k=k, tiles=tiles, busy_compute_units=min(tiles, cus), tiles_per_compute_unit=rounds,
+                        k_slices=slices, us=res["kernel_us"], us_per_k_tile=res["kernel_us"] / (rounds * k / 64),
+                        tflops=res["flops"] / res["kernel_us"] / 1e6))
+    return dict(steps=steps, warmup=warmup, rows=out)
+
+
 def run_workload(cfg, steps, warmup, vendor):
     op = inputs.CONFIGS[cfg]["op"]
     if op == "softmax":
@@ -789,7 +828,7 @@ def main():
                     help="untimed launches before the timed ones; the device takes a few hundred short launches "
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
     ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"],
-                    help="one of %s, copy_f32, hbm_ceilings, short_kernels, softmax_f32_786432x512_unmasked, or a long-row line by name: "
+                    help="one of %s, copy_f32, hbm_ceilings, short_kernels, gemm16_midsize, gemm16_active_cus, softmax_f32_786432x512_unmasked, or a long-row line by name: "
                          "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache)" % ", ".join(sorted(WORKLOADS)))
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
@@ -808,6 +847,12 @@ def main():
         return
     if args.workload == "hbm_ceilings":  # the whole streaming sweep, for profiles/
         print(json.dumps(bench_ceilings(min(args.steps, 10), 3, full=True)))
+        return
+    if args.workload == "gemm16_midsize":  # the sweep behind profiles/gemm16_midsize.md
+        print(json.dumps(bench_gemm16_midsize(min(args.steps, 30), max(args.warmup, 100), vendor)))
+        return
+    if args.workload == "gemm16_active_cus":  # time per K tile by the number of busy compute units, for profiles/
+        print(json.dumps(bench_gemm16_active_cus(min(args.steps, 30), max(args.warmup, 100))))
         return
     if args.workload == "short_kernels":  # intercept and slope of the two short configurations, for profiles/
         print(json.dumps(bench_short_kernels(min(args.steps, 30), max(args.warmup, 100))))

@@ -202,7 +202,9 @@ __device__ __forceinline__ void tile_of(const Params &p, int b, int grid, int t,
 // only WTM * WTN * 2 / PARTS bytes of LDS.
 // WAIT_VM: wait for this wave's outstanding vector memory operations right before the first global store
 // (the caller has loads in flight that it wants confirmed while they are still the only ones outstanding).
-template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1, bool WAIT_VM = false>
+// GUARD_M (full-tile form): the tile may reach past row M - rows at or past M hold the products of rows fetched from
+// elsewhere in A: they take no C and are not stored.
+template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1, bool WAIT_VM = false, bool GUARD_M = false>
 __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
                                            int lane, int row0, int col0) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -250,7 +252,9 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 // C of this 32-row block: all loads first, so that their latencies overlap
                 u32x2 c_q[TN][4];
                 if (use_c) {
-                    const uint16_t *crow = p.C + (row0 + i * 32 + frow) * ldd + col0 + 4 * fhalf;
+                    // (a row at or past M reads the matrix's last row instead: a valid address, a value never stored)
+                    const int crow_index = GUARD_M && row0 + i * 32 + frow >= M ? M - 1 : row0 + i * 32 + frow;
+                    const uint16_t *crow = p.C + crow_index * ldd + col0 + 4 * fhalf;
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -288,7 +292,7 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int gn = col0 + c * 8;
                 // streaming store: D is written once and not read again by this kernel (`sc1 nt`, which helps the
                 // row kernels, measured no different here: 74.3 against 73.8 us)
-                __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
+                if (!GUARD_M || gm < M) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
             }
         }
         return;
@@ -770,6 +774,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        // The zeroes are written by vector-ALU moves, and the matrix instructions that read them as their addend
+        // are inline assembly: the compiler does not know them for what they are and keeps no distance between
+        // such a move and the instruction that reads its register (it is free to sink the moves down to right in
+        // front of the first of them).  Pin the moves here and put the wait states behind them.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
+        asm volatile("s_nop 7");
     };
     clear_acc();
 
@@ -884,7 +897,10 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
 // EDGE_K: K is any multiple of 8 and is padded with zeros up to the next multiple of 128 - a lane whose
 // 16-byte chunk (or, for a row-major B, whose row) lies at or past K fetches 16 zero bytes instead, chosen per
 // load with a compare and two selects, so nothing is read past the end of a row or of the matrix.
-template <class T, bool BF16, bool B_ROW, bool EDGE_K = false>
+// EDGE_M: M is any multiple of 8; the last row of tiles may reach past it.  A wave-level load covers eight rows of A,
+// so a load whose rows lie at or past M is pointed - a wave-uniform choice, made once per output tile - at the last
+// eight rows of A instead: valid addresses, whose products land in rows of the tile that the epilogue does not store.
+template <class T, bool BF16, bool B_ROW, bool EDGE_K = false, bool EDGE_M = false>
 __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -949,15 +965,25 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // scalar 64-bit add, the lane offset and the LDS address in M0 - no multiplication per load.
     int ld_kt = 0, ld_t = 0;
     const char *cur_a, *cur_b;
+    const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
+    int64_t a_off[A_LOADS];  // load i of A: bytes from the cursor to its eight rows (wave-uniform)
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = i * group_stride;
     auto set_cursor = [&]() {
         int m0, n0;
         tile_origin(ld_t, m0, n0);
+        if constexpr (EDGE_M) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const int first = m0 + 8 * (wave + WAVES * i);  // first of the load's eight rows
+                a_off[i] = static_cast<int64_t>((first < p.M ? first : p.M - 8) - (m0 + 8 * wave)) * K * 2;
+            }
+        }
         cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
         if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(2 * wave) * p.ldb + n0);
         else cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
     };
     set_cursor();
-    const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
     const int64_t group_stride_b = B_ROW ? static_cast<int64_t>(2 * WAVES) * p.ldb * 2 : group_stride;
     const int64_t ktile_step_b = B_ROW ? static_cast<int64_t>(kBK) * p.ldb * 2 : kBK * 2;  // bytes from a K tile to the next
     auto advance_cursor = [&]() {
@@ -975,7 +1001,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // EDGE_K: where load I of the cursor's K tile reads from - its place in A or B, or the zero chunk when the
     // lane's k lies at or past K (for a row-major B the k is the row the load fetches)
     auto source_a = [&](int i) {
-        const char *at = cur_a + i * group_stride + lane_off;
+        const char *at = cur_a + a_off[i] + lane_off;
         if constexpr (EDGE_K) at = ld_kt * kBK + lane_k < K ? at : zeros;
         return at;
     };
@@ -1041,6 +1067,15 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        // The zeroes are written by vector-ALU moves, and the matrix instructions that read them as their addend
+        // are inline assembly: the compiler does not know them for what they are and keeps no distance between
+        // such a move and the instruction that reads its register (it is free to sink the moves down to right in
+        // front of the first of them).  Pin the moves here and put the wait states behind them.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
+        asm volatile("s_nop 7");
     };
     clear_acc();
 
@@ -1106,6 +1141,11 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 bf[slot][j] = u32x4{b_lo[slot][j][0], b_lo[slot][j][1], b_hi[slot][j][0], b_hi[slot][j][1]};
+            // where the halves did not land in adjacent registers the line above is vector-ALU moves, and the matrix
+            // instructions that read bf are inline assembly the compiler keeps no distance to (see clear_acc)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bf[slot][j]));
+            asm volatile("s_nop 3");
         } else if constexpr (TM == 4 && TN == 2) {
             asm volatile("s_waitcnt lgkmcnt(0)"
                          : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]),
@@ -1181,8 +1221,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             if constexpr (SPARE) {
                 constexpr int REGION = WTM * WTN * 2 / 4;  // bytes per wave and pass
                 char *region = lds_bytes + 2 * (A_BYTES + B_BYTES) + wave * REGION;
-                store_tile<WTM, WTN, 1, BF16, false, 4, true>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
-                                                              m0 + wm * WTM, n0 + wn * WTN);
+                store_tile<WTM, WTN, 1, BF16, false, 4, true, EDGE_M>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                                                                      m0 + wm * WTM, n0 + wn * WTN);
                 clear_acc();
                 stores_in_flight = true;
             } else {
@@ -1190,8 +1230,8 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
                 static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
                 char *region = wave < WAVES / 2 ? lds_bytes + S * A_BYTES + wave * REGION
                                                 : lds_bytes + 2 * A_BYTES + S * B_BYTES + (wave - WAVES / 2) * REGION;
-                store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
-                                                                m0 + wm * WTM, n0 + wn * WTN);
+                store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS, false, EDGE_M>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                                                                               m0 + wm * WTM, n0 + wn * WTN);
                 clear_acc();
                 lds_barrier();  // every wave is done with its transpose region in stage S
                 if (step + 2 < total) issue_next(S);
@@ -1222,18 +1262,19 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     }
 }
 
-template <class T, bool BF16, bool B_ROW = false>
+// EDGE_M: M may be any multiple of 8 from 8 on (the last row of tiles then reaches past M, see the kernel).
+template <class T, bool BF16, bool B_ROW = false, bool EDGE_M = false>
 int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
-    if ((p.M % T::BM) != 0 || (p.N % T::BN) != 0 || (p.K % 8) != 0)
+    if ((p.M % (EDGE_M ? 8 : T::BM)) != 0 || p.M < 8 || (p.N % T::BN) != 0 || (p.K % 8) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 8 == 0");
     const bool edge_k = p.K % (2 * kBK) != 0;  // padded with zeros up to a pair of K tiles inside the kernel
-    auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true> : gemm16_pinned_kernel<T, BF16, B_ROW, false>;
+    auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true, EDGE_M> : gemm16_pinned_kernel<T, BF16, B_ROW, false, EDGE_M>;
     static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge_k]); st != KO_OK)
         return st;
     p.tiles_n = p.N / T::BN;
-    const int tiles_m = p.M / T::BM;
+    const int tiles_m = (p.M + T::BM - 1) / T::BM;
     p.nblocks = tiles_m * p.tiles_n;
     int grid = compute_units() / 8 * 8;
     if (grid > p.nblocks) grid = p.nblocks;
@@ -1511,10 +1552,16 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // x 256 81 / 71 (58); 4880 x 7768 x 256 52 / 60 (41), x 512 82 / 82; 1351 x 18488 x 256 41 / 45, x 512 65 / 60;
         // 8148 x 1800 x 512 30 / 37 (27); 3000 x 5000 x 256 22 / 29 (22), x 512 34 / 38 (28); 4071 x 2328 x 768
         // (160 big tiles) 32 / 41 (24), 12521 x 989 x 768 40 / 52 (30), 3000 x 5000 x 768 (240) 46 / 48.
+        // A row count that is a multiple of 8 but not of the tile height, on whole tile columns: the pinned kernel
+        // takes it as it is (its last row of tiles fetches rows it has, and stores what lies inside the matrix),
+        // so such a shape is neither cut nor taken off that kernel.  3000 x 3072 x 768: 30.0 -> 22.1 us (hipBLASLt
+        // 19.5), 12000 x 768 x 3072 84 -> 73, 3000 x 4096 x 4096 112 -> 93, 16000 x 3072 x 768 82 -> 76; on
+        // 128 x 256 tiles 6000 x 1024 x 1024 25.5 -> 18.0 (17.8), 6000 x 768 x 3072 55 -> 44.
+        const bool m_edge = p.M % 256 != 0 && p.M % 8 == 0 && p.M >= 8 && p.N % 256 == 0 && p.K >= 2 * kBK;
         {
             const int64_t cu = compute_units();
             const bool ragged = p.M % 256 != 0 || p.N % 256 != 0;
-            if (ragged && split_knob != 1 && 2 * big_tiles >= cu &&
+            if (ragged && split_knob != 1 && 2 * big_tiles >= cu && !(m_edge && p.K > 512) &&
                 (p.K <= 128 || (p.K <= 256 && 2 * big_tiles <= 5 * cu) || (p.K <= 512 && 4 * big_tiles <= 5 * cu) ||
                  (p.K <= 768 && 5 * big_tiles <= 4 * cu)))
                 return launch<TileSmall, BF16, B_ROW_MAJOR>(p, stream);
@@ -1542,12 +1589,13 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // 128 go out as a launch of their own.
         if (split_knob != 1 && p.N % 256 == 0 && p.K >= 256) {
             const int64_t cu = compute_units();
-            const int64_t rows128 = p.M / 128;
+            const int64_t rows128 = m_edge ? (p.M + 127) / 128 : p.M / 128;
             const int64_t half_tiles = rows128 * (p.N / 256);
             // (the second launch costs about 2 us: 2000 x 3072 x 768 22 us whole on 128 x 128 tiles, 24 cut; from
             // K = 1536 on the first one gains more than that - 7000 x 768 x 3072 66 -> 58, 2000 x 4096 x 4096 117 -> 103)
-            if (20 * half_tiles >= 11 * cu && half_tiles <= cu && (p.M % 128 == 0 || (row_cuts > 0 && p.K >= 1536))) {
+            if (20 * half_tiles >= 11 * cu && half_tiles <= cu && (p.M % 128 == 0 || m_edge || (row_cuts > 0 && p.K >= 1536))) {
                 if (p.M % 128 == 0) return launch_pinned<TileHalf, BF16, B_ROW_MAJOR>(p, stream);
+                if (m_edge) return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
                 const int64_t m1 = rows128 * 128;
                 Params top = p, bottom = p;
                 top.M = static_cast<int>(m1);
@@ -1563,7 +1611,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             const int64_t cu = compute_units();
             const int64_t tn = (p.N + 255) / 256;
             const bool pinned_ok = p.N % 256 == 0 && p.K >= 2 * kBK;
-            int64_t rows_top = p.M % 256 != 0 && pinned_ok ? p.M / 256 : (p.M + 255) / 256;  // in tile rows
+            int64_t rows_top = p.M % 256 != 0 && pinned_ok && !m_edge ? p.M / 256 : (p.M + 255) / 256;  // in tile rows
             const int64_t tiles = rows_top * tn, rounds = tiles / cu;
             if (rounds >= 1 && tiles % cu != 0) {
                 const int64_t rows1 = rounds * cu / tn;  // whole tile rows within the full rounds
@@ -1588,6 +1636,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // the two are level).
         if (2 * big_tiles >= compute_units() && p.M % 256 == 0 && p.N % 256 == 0 && p.K >= 2 * kBK)
             return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR>(p, stream);
+        if (2 * big_tiles >= compute_units() && m_edge) return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
         // at most 32 rows and tiles for every compute unit: one matrix instruction's worth of rows per tile, 256
         // columns wide (64 x 64 tiles load 64 rows of A per tile and multiply most of them for nothing); with
         // fewer tiles the smaller tilings below put more workgroups to work (8 x 3072 x 768: 8 us against 13 us)
@@ -1623,6 +1672,8 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
         case 53: return launch_direct<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
         case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // M any multiple of 8
+        case 61: return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }

@@ -895,3 +895,56 @@ def test_sgemm_forced_slices_keep_a_kernel_that_takes_them(ko):
         finally:
             ko.set_tuning("sgemm.k_slices", 0)
         np.testing.assert_array_equal(dD.download(np.float32, (m, n)), A.astype(np.float64) @ B.astype(np.float64))
+
+
+@pytest.mark.parametrize("variant", [60, 61])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k", [(8, 256, 128), (136, 512, 256), (264, 256, 200), (1000, 768, 384), (3000, 512, 1032)])
+def test_gemm16_pinned_kernel_takes_any_multiple_of_8_rows(ko, variant, bf16, b_col_major, m, n, k):
+    """The pinned kernel with a last row of tiles that reaches past M (M a multiple of 8): its loads of rows at or past M
+    fetch the last eight rows of A instead and its epilogue leaves those rows of the tile alone.  Against the oracle,
+    on 256 x 256 and 128 x 256 tiles, both layouts of B, K that is and is not whole K tiles, with C and beta, and with a
+    guard area behind D that must come back untouched."""
+    dt = ko.BF16 if bf16 else ko.F16
+    A = _bits16((m, k), 31 + m, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 33 + n, bf16)
+    C = _bits16((m, n), 35 + k, bf16)
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    guard = 4096
+    dA, dB, dC = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B), ko.DeviceBuffer.from_numpy(C)
+    dD = ko.DeviceBuffer((m * n + guard) * 2)
+    ko.set_tuning("gemm16.variant", variant)
+    try:
+        for use_c in (False, True):
+            dD.upload(np.full(m * n + guard, 0x7b7b, np.uint16))
+            ko.gemm16(m, n, k, dA, dB, dD, C=dC if use_c else None, alpha=0.5 if use_c else 1.0,
+                      beta=-1.5 if use_c else 0.0, b_layout=layout, dtype=dt)
+            ko.synchronize()
+            out = dD.download(np.uint16, (m * n + guard,))
+            assert np.all(out[m * n:] == 0x7b7b), "rows past M were written"
+            if use_c:
+                _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, C_bits=C, alpha=0.5, beta=-1.5, bf16=bf16)
+                ap = 0.5 * ap + 1.5 * np.abs(_to_f64(C, bf16))
+            else:
+                _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bf16=bf16)
+            assert_gemm16_close(_to_f64(out[:m * n].reshape(m, n), bf16), ref64, ap, k, bf16=bf16)
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+
+
+@pytest.mark.parametrize("m,n,k", [(3000, 3072, 768), (6000, 1024, 1024), (1240, 2304, 3072), (16000, 3072, 768)])
+def test_gemm16_ragged_rows_through_the_default_dispatch_are_exact(ko, m, n, k):
+    """Row counts that are multiples of 8 but not of the tile height, on the shapes the dispatch sends to the pinned
+    kernel as they are (256 x 256 tiles, and 128 x 256 tiles): small integers make every sum exact, so any row fetched
+    from the wrong place or stored where it does not belong shows."""
+    rng = np.random.default_rng(m + k)
+    A = rng.integers(-3, 4, (m, k)).astype(np.float16)
+    B = rng.integers(-3, 4, (n, k)).astype(np.float16)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float16)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert np.abs(want).max() < 2048 - 8  # exactly representable in binary16
+    got = ko.gemm16_host(A.view(np.uint16), B.view(np.uint16), m, n, k)
+    np.testing.assert_array_equal(got.view(np.float16).astype(np.float64), want)
+    got = ko.gemm16_host(A.view(np.uint16), B.view(np.uint16), m, n, k, bias_bits=bias.view(np.uint16))
+    np.testing.assert_array_equal(got.view(np.float16).astype(np.float64), want + bias.astype(np.float64)[None, :])
