@@ -498,16 +498,17 @@ def bench_gemm16_active_cus(steps, warmup):
     """Time per K tile of the 256 x 256 kernel of the 16-bit GEMM by how many compute units have a tile: K = 4096
     (64 K tiles per output tile), N = 3072 (12 tile columns), M from 256 to 16384."""
     out = []
+    ko.set_tuning("gemm16.variant", 53)  # the 256 x 256 pinned kernel whatever the dispatch would pick
     for m in (256, 512, 1024, 2048, 4096, 5376, 10752, 16384):
         n, k = 3072, 4096
         res, _ = bench_gemm16(4, steps, warmup, None, shape=(m, n, k))
         tiles = (m // 256) * (n // 256)
         cus = ko.device_info()["compute_units"]
         rounds = -(-tiles // cus)
-        slices = ko.gemm_plan(m, n, k, sixteen_bit=True)[0]
         out.append(dict(m=m, n=n, k=k, tiles=tiles, busy_compute_units=min(tiles, cus), tiles_per_compute_unit=rounds,
-                        k_slices=slices, us=res["kernel_us"], us_per_k_tile=res["kernel_us"] / (rounds * k / 64),
+                        us=res["kernel_us"], us_per_k_tile=res["kernel_us"] / (rounds * k / 64),
                         tflops=res["flops"] / res["kernel_us"] / 1e6))
+    ko.set_tuning("gemm16.variant", 0)
     return dict(steps=steps, warmup=warmup, rows=out)
 
 
