@@ -29,7 +29,7 @@ int hip_fail(hipError_t err, const char *expr, const char *file, int line);
     X(softmax_nontemporal, "softmax.nontemporal") X(softmax_block_threads, "softmax.block_threads")         \
     X(softmax_wave_threads, "softmax.wave_threads") X(layernorm_lanes_per_row, "layernorm.lanes_per_row")   \
     X(layernorm_blocks_per_cu, "layernorm.blocks_per_cu") X(layernorm_block_threads, "layernorm.block_threads") \
-    X(layernorm_wave_threads, "layernorm.wave_threads") X(softmax_wave_lds, "softmax.wave_lds") X(rows_block_grid, "rows.block_grid") X(layernorm_wave_lds, "layernorm.wave_lds")           \
+    X(layernorm_wave_threads, "layernorm.wave_threads") X(softmax_wave_lds, "softmax.wave_lds") X(rows_block_grid, "rows.block_grid") X(layernorm_wave_lds, "layernorm.wave_lds") X(layernorm_affine_lds, "layernorm.affine_lds")           \
     X(sgemm_variant, "sgemm.variant") X(sgemm_mapping, "sgemm.mapping") X(sgemm_split_rows, "sgemm.split_rows") \
     X(sgemm_k_slices, "sgemm.k_slices") X(gemm16_k_slices, "gemm16.k_slices") X(layernorm_block_rows, "layernorm.block_rows") X(sgemm_slice_variant, "sgemm.slice_variant") X(sgemm_unaligned, "sgemm.unaligned")                                                                     \
     X(gemm16_variant, "gemm16.variant") X(gemm16_mapping, "gemm16.mapping")                                 \

@@ -93,7 +93,10 @@ struct Args {
 // other and its values ignored - because loads inside `if (gamma)` branches leave the compiler unable to count
 // the loads in flight: it then makes the statistics wait for all but the last two of them, gamma and beta
 // included, instead of for the row alone.
-template <int IO, int LPR, int VPL, bool FULL, bool AFFINE>
+// AFFINE_LDS (with AFFINE, FULL rows, one row per wavefront, four wavefronts per workgroup, rows a multiple of four):
+// gamma and beta come into LDS once per workgroup, straight from global memory, and every wavefront reads its
+// lanes' vectors from there.  Fetched per wavefront they are 6 KB of L1 traffic next to a 3 KB row.
+template <int IO, int LPR, int VPL, bool FULL, bool AFFINE, bool AFFINE_LDS = false>
 __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<IO>::elem *in,
                                                              typename Io<IO>::elem *out,
                                                              float *__restrict__ mean_out,
@@ -121,7 +124,21 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     // four and six resident waves per SIMD at 768 columns) and converted where they are used.
     typename Io<IO>::raw g_raw[VPL], b_raw[VPL];
     const typename Io<IO>::elem *g_from = gamma ? gamma : beta, *b_from = beta ? beta : gamma;
+    extern __shared__ __attribute__((aligned(16))) char affine_lds[];  // AFFINE_LDS: raw gamma[nvec], then raw beta[nvec]
     auto load_affine = [&]() {
+        if constexpr (AFFINE_LDS) {
+            // thread t brings vector t of gamma and of beta in: a wavefront's 64 vectors land, 16 bytes per lane, behind
+            // a wave-uniform LDS address
+            typedef const __attribute__((address_space(1))) void *gptr_t;
+            typedef __attribute__((address_space(3))) void *lptr_t;
+            for (int j0 = static_cast<int>(threadIdx.x & ~63u); j0 < nvec; j0 += blockDim.x) {
+                if (j0 + lane < nvec) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(g_from + E * (j0 + lane)), (lptr_t)(affine_lds + 16 * j0), 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((gptr_t)(b_from + E * (j0 + lane)), (lptr_t)(affine_lds + 16 * (nvec + j0)), 16, 0, 0);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
             const int j = l + k * LPR;
@@ -152,7 +169,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
         for (int k = 0; k < VPL; ++k) Io<IO>::unpack(loaded[k], v[k]);
     };
 
-    auto finish_rows = [&](float (&v)[VPL][E], int64_t row) {
+    auto finish_rows = [&](float (&v)[VPL][E], int64_t row, auto between) {
         const bool row_ok = row < rows;
         const float x0 = wave::broadcast_group_first<LPR>(v[0][0]);
         wave::Welford w{0.0f, 0.0f, 0.0f};
@@ -206,6 +223,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
 
         const float mean = w.mean;  // of the shifted row
         const float rstd = rsqrt_1ulp(w.m2 * inv_denominator + eps);
+        between();
 
         // streaming stores: wave-uniform base (the wavefront's first row) + per-lane byte offset
         // (written through at once only when rows are whole 64-byte lines: see store_row_vec)
@@ -252,10 +270,22 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const typename Io<I
     float v[VPL][E];
     load_rows(v, row0 + sub);
     load_affine();
-    finish_rows(v, row0 + sub);
+    finish_rows(v, row0 + sub, [&]() {
+        if constexpr (AFFINE_LDS) {
+            // every wavefront of the workgroup has a row (rows are a multiple of the wavefronts per workgroup), so
+            // all of them arrive here; the statistics above have covered the latency of the fetch
+            __syncthreads();
+            const typename Io<IO>::raw *g_lds = reinterpret_cast<const typename Io<IO>::raw *>(affine_lds);
+#pragma unroll
+            for (int k = 0; k < VPL; ++k) {
+                g_raw[k] = g_lds[l + k * LPR];
+                b_raw[k] = g_lds[nvec + l + k * LPR];
+            }
+        }
+    });
     for (row0 += stride; row0 < rows; row0 += stride) {
         load_rows(v, row0 + sub);
-        finish_rows(v, row0 + sub);
+        finish_rows(v, row0 + sub, []() {});
     }
 }
 
@@ -818,6 +848,35 @@ int launch_wave_full(const Args<IO> &a) {
     if (lds == 0 && threads == 64)
         lds = lds_pad_for_residency(static_cast<int64_t>(RPW) * a.cols * sizeof(typename Io<IO>::elem), 72 * 1024);
     if (lds < 0) lds = 0;
+    if constexpr (FULL && LPR == 64 && sizeof(typename Io<IO>::raw) == 16 && VPL >= 2) {
+        // gamma and beta through LDS, four rows per workgroup: from two vectors per lane on, where fetching them per
+        // wavefront is a third or more of its L1 traffic.  Knob layernorm.affine_lds: 1 never, 2 whenever the shape allows.
+        const int knob = tuning(knob_layernorm_affine_lds);
+        if ((a.gamma || a.beta) && knob != 1 && a.rows % 4 == 0 && per_cu <= 0 &&
+            (knob == 2 || tuning(knob_layernorm_wave_threads) == 0)) {
+            const int64_t wgrid = a.rows / 4;
+            if (wgrid <= 0x7fffffff) {
+                const int need = 2 * (a.cols / Io<IO>::E) * 16;
+                // Residency cap (see lds_pad_for_residency): workgroups of four rows, about 56 KB of rows in flight per
+                // compute unit but never fewer than three workgroups.  Interleaved runs, workgroups per CU 8 / 6 / 5 / 4 / 3,
+                // us: [16384, 768] 18.7 / 18.5 / 18.3 / 18.2 / 19.2 (gamma and beta per wavefront: 18.7), [262144, 768]
+                // 258 / 257 / 254 / 254 / 257 (265), [196608, 1024] 259 / 259 / 253 / 253 / 253 (260), [65536, 1536]
+                // 130 / 130 / 130 / 130 / 127 (138), [32768, 512] 23.4 / 23.1 / 23.8 / 23.8 / 25.8 (23.5).
+                // Knob layernorm.wave_lds: bytes per workgroup, or -1 for no cap.
+                const int64_t wg_bytes = 4 * static_cast<int64_t>(a.cols) * sizeof(typename Io<IO>::elem);
+                int64_t wgs = (56 * 1024 + wg_bytes / 2) / wg_bytes;
+                wgs = wgs < 3 ? 3 : (wgs > 8 ? 8 : wgs);
+                // (a KB short of an even share of the 160 KB, so that the count fits whatever the allocation rounds to)
+                int pad = wgs >= 8 ? 0 : static_cast<int>((160 * 1024 / wgs - 1024) & ~int64_t{511});
+                if (tuning(knob_layernorm_wave_lds) != 0) pad = tuning(knob_layernorm_wave_lds) > 0 ? tuning(knob_layernorm_wave_lds) : 0;
+                layernorm_wave_kernel<IO, LPR, VPL, FULL, true, true>
+                    <<<dim3(static_cast<unsigned>(wgrid)), dim3(256), static_cast<size_t>(pad > need ? pad : need), a.stream>>>(
+                        a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
+                KO_CHECK_LAUNCH();
+                return KO_OK;
+            }
+        }
+    }
     if (a.gamma || a.beta)
         layernorm_wave_kernel<IO, LPR, VPL, FULL, true><<<dim3(static_cast<unsigned>(grid)), dim3(threads), lds, a.stream>>>(
             a.in, a.out, a.mean, a.rstd, a.gamma, a.beta, a.rows, a.cols, a.eps, a.inv_denominator);
