@@ -24,7 +24,7 @@ typedef struct ko_harness_hooks_t {
     int (*set_tuning)(const char *name, int value);
     int (*get_tuning)(const char *name, int *value);
     int (*sgemm_plan)(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
-    int (*gemm16_plan)(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
+    int (*gemm16_plan)(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile);
     int (*stream_workspace_count)(void);
     int (*set_last_error)(int status, const char *message); /* returns status */
 } ko_harness_hooks_t;
@@ -76,9 +76,12 @@ int ko_debug_stream_workspace_count(int *count);
 /* What the GEMMs' host-side planners decide for a shape (16-byte aligned operands, 256 compute units when no
  * device is visible): the number of K slices (1 = the problem goes out whole), the depth of every slice but the
  * last, and the tiling of the sliced launch (SGEMM: the kernel variant number, 0 = chosen as for the whole
- * problem; 16-bit GEMM: 128 or 64, the tile edge, or 32 for 32 x 256 tiles).  Touches no device memory and launches nothing. */
+ * problem; 16-bit GEMM: 128 or 64, the tile edge, or 32 for 32 x 256 tiles).  The 16-bit GEMM with B in layout
+ * b_layout (KO_ROW_MAJOR / KO_COL_MAJOR) has one more answer for a problem of few tiles: slices = 1 and tile = 3232,
+ * 3264 or 6464 - one launch whose workgroups own a 32 x 32, 32 x 64 or 64 x 64 output tile and split K over their
+ * waves (tile = 0: none of this).  Touches no device memory and launches nothing. */
 int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
-int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
+int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile);
 
 #ifdef __cplusplus
 }

@@ -89,7 +89,7 @@ HARNESS_SIGNATURES = {
     "ko_debug_stream_workspace_count": (_int, [ctypes.POINTER(_int)]),
     "ko_debug_sgemm_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
                                    ctypes.POINTER(ctypes.c_int)]),
-    "ko_debug_gemm16_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+    "ko_debug_gemm16_plan": (_int, [_i64, _i64, _i64, _int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
                                     ctypes.POINTER(ctypes.c_int)]),
 }
 
@@ -307,11 +307,14 @@ def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
     check(lib().ko_sgemm_f32(m, n, k, alpha, _p(A), _p(B), beta, _p(C), _p(D), _h(stream)))
 
 
-def gemm_plan(m, n, k, sixteen_bit=False):
-    """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM decides for a shape."""
+def gemm_plan(m, n, k, sixteen_bit=False, b_layout=COL_MAJOR):
+    """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM (with B in b_layout) decides
+    for a shape; (1, 0, 3232 | 3264 | 6464) is the 16-bit GEMM's one launch that splits K over the waves of a workgroup."""
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    fn = harness().ko_debug_gemm16_plan if sixteen_bit else harness().ko_debug_sgemm_plan
-    check(fn(m, n, k, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    if sixteen_bit:
+        check(harness().ko_debug_gemm16_plan(m, n, k, b_layout, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    else:
+        check(harness().ko_debug_sgemm_plan(m, n, k, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
     return a.value, b.value, c.value
 
 

@@ -1309,6 +1309,228 @@ int launch_pinned(Params p, hipStream_t stream) {
     return KO_OK;
 }
 
+// K split over the waves of a workgroup, for a problem of few output tiles (a few hundred rows against a weight
+// matrix): every kernel above walks K in steps that all waves of a workgroup take together - a barrier per K tile,
+// one or two K tiles in flight per workgroup - and with a workgroup or less per compute unit such a step costs its
+// latencies (0.4 us per 64 k on 64 x 64 tiles, whatever the arithmetic).  Here a workgroup owns one (32 TM) x (32 TN)
+// output tile and wave w multiplies K tiles w, w + WAVES, ... of it: the whole tile over its own share of K, out of two
+// LDS stages of its own that it fills with direct-to-LDS loads (eight rows of 128 bytes per wave-level load, as
+// in the kernels above) - no barrier in the loop, WAVES times fewer steps in a row, and two K tiles per wave in
+// flight.  At the end the waves leave their fp32 tiles in LDS and the workgroup adds them in wave order (the same
+// bits from call to call) and applies alpha, beta * C, the bias and the activation once.
+// Any M, N and any K that is a multiple of 8: a row at or past M (N) is fetched from the last row instead and its
+// results are not stored; a 16-byte chunk at or past K - in the last K tile, or in a K tile past the end that a
+// wave's second stage asks for - is fetched from sixteen zero bytes, chosen per load with a compare and two selects.
+// B column-major ([N][K], K contiguous) only.
+template <int TM, int TN, int WAVES, bool BF16>
+__global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params p) {
+    constexpr int WTM = 32 * TM, WTN = 32 * TN;
+    constexpr int KS = kBK / 16;
+    constexpr int A_LOADS = WTM / 8, B_LOADS = WTN / 8, LOADS = A_LOADS + B_LOADS;
+    constexpr int A_BYTES = WTM * kBK * 2, STAGE_BYTES = (WTM + WTN) * kBK * 2, WAVE_BYTES = 2 * STAGE_BYTES;
+    constexpr int LDP = WTN + 4;  // floats between the rows of a wave's fp32 tile in LDS
+    static_assert(KS == 4 && LOADS <= 31, "two K tiles of loads must fit the 6-bit counter");
+    static_assert(WTM * LDP * 4 <= WAVE_BYTES && WAVES * WAVE_BYTES <= 160 * 1024, "");
+    static_assert((TM == 1 || TM == 2) && (TN == 1 || TN == 2), "");
+
+    extern __shared__ u32x4 lds[];
+    char *const lds_bytes = reinterpret_cast<char *>(lds);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = static_cast<int>(blockIdx.x);
+    const int m0 = (tile / p.tiles_n) * WTM, n0 = (tile % p.tiles_n) * WTN;
+    const int M = p.M, N = p.N, K = p.K;
+    const int64_t ldk = p.ldk;
+    const int KT = (K + kBK - 1) / kBK;
+    const int my_tiles = wave < KT ? (KT - wave + WAVES - 1) / WAVES : 0;
+
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    const char *const zeros = reinterpret_cast<const char *>(&zero_chunk16);
+
+    // Lane l of a wave-level load fills the l-th 16-byte slot of eight LDS rows: row l / 8, slot l % 8, which holds
+    // chunk (l % 8) ^ swz(row) of the row.  The row within the tile is 8 i + l / 8 for load i, so the swizzle term
+    // takes two values, by the parity of i.
+    const int row_in = lane >> 3;
+    int lane_k[2];  // first k, within a K tile, of the chunk this lane fetches in an even / odd load
+#pragma unroll
+    for (int par = 0; par < 2; ++par) lane_k[par] = ((lane & 7) ^ ((4 * par + (row_in >> 1)) & 7)) << 3;
+    const char *src_a[A_LOADS], *src_b[B_LOADS];  // this lane's chunk of load i in the K tile to fetch next
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int r = m0 + 8 * i + row_in;
+        src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + wave * kBK + lane_k[i & 1]);
+    }
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) {
+        const int r = n0 + 8 * j + row_in;
+        src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + wave * kBK + lane_k[j & 1]);
+    }
+    int ld_k0 = wave * kBK;  // first k of the K tile to fetch next
+    char *const wave_lds = lds_bytes + wave * WAVE_BYTES;
+    auto issue = [&](int stage) {
+        const bool in0 = ld_k0 + lane_k[0] < K, in1 = ld_k0 + lane_k[1] < K;
+        char *dst = wave_lds + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            __builtin_amdgcn_global_load_lds((gptr_t)((i & 1 ? in1 : in0) ? src_a[i] : zeros), (lptr_t)(dst + 1024 * i), 16, 0, 0);
+            src_a[i] += WAVES * kBK * 2;
+        }
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j) {
+            __builtin_amdgcn_global_load_lds((gptr_t)((j & 1 ? in1 : in0) ? src_b[j] : zeros), (lptr_t)(dst + A_BYTES + 1024 * j), 16, 0, 0);
+            src_b[j] += WAVES * kBK * 2;
+        }
+        ld_k0 += WAVES * kBK;
+    };
+
+    // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int sw = (frow >> 1) & 7;
+    const uint32_t frag_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wave_lds));
+    uint32_t off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) off[ks] = frag_base + static_cast<uint32_t>(frow * 128 + (((2 * ks + fhalf) ^ sw) << 4));
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    u32x4 af[2][TM], bf[2][TN];
+    auto read_frags = [&](auto ks_c, auto slot_c, auto stage_c) {
+        constexpr int KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value, S = decltype(stage_c)::value;
+        static_for<TM>([&](auto i_c) {
+            constexpr int I = decltype(i_c)::value;
+            lds_read16<S * STAGE_BYTES + I * 4096>(af[SLOT][I], off[KSTEP]);
+        });
+        static_for<TN>([&](auto j_c) {
+            constexpr int J = decltype(j_c)::value;
+            lds_read16<S * STAGE_BYTES + A_BYTES + J * 4096>(bf[SLOT][J], off[KSTEP]);
+        });
+    };
+    // every read issued so far has landed; the operands keep the matrix instructions that use them behind this point
+    auto wait_frags = [&](int slot) {
+        if constexpr (TM == 2 && TN == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
+        else if constexpr (TM == 1 && TN == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
+        else if constexpr (TM == 2 && TN == 1)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0])::"memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0])::"memory");
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<BF16>(bf[slot][j], af[slot][i], acc[i][j]);
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+    // One K tile out of stage S; the loads of the K tile after next go out as soon as the stage's last fragments
+    // are in registers.  Loads complete in order: with two K tiles' worth in flight, all but the last LOADS done
+    // means that this stage has landed.
+    auto k_tile = [&](auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+        read_frags(C0{}, C0{}, stage_c);
+        read_frags(C1{}, C1{}, stage_c);
+        wait_frags(0);
+        wait_frags(1);
+        multiply(0);
+        read_frags(C2{}, C0{}, stage_c);
+        multiply(1);
+        read_frags(C3{}, C1{}, stage_c);
+        wait_frags(0);
+        wait_frags(1);
+        issue(S);
+        multiply(0);
+        multiply(1);
+    };
+    issue(0);
+    issue(1);
+    for (int t = 0; t < my_tiles; t += 2) {
+        k_tile(C0{});
+        k_tile(C1{});  // past this wave's last K tile: a stage of zeros
+    }
+    // the loads still in flight (K tiles past the end: zeros) must land before the stages are written over
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // this wave's tile as fp32 into its own LDS; a lane holds, of row frow of each 32 x 32 block, columns 8 q + 4 fhalf .. + 3
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    float *const mine = reinterpret_cast<float *>(wave_lds);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                *reinterpret_cast<float4v *>(mine + (i * 32 + frow) * LDP + j * 32 + 8 * q + 4 * fhalf) = v;
+            }
+    __syncthreads();
+    // one thread per four consecutive columns of a row; the waves' tiles are added in wave order
+    constexpr int GROUPS = WTN / 4, ROWS_PER_PASS = 64 * WAVES / GROUPS;
+    static_assert(64 * WAVES % GROUPS == 0, "");
+    const bool use_c = p.C != nullptr && p.beta != 0.0f;
+    const int g = tid % GROUPS;
+    const int n = n0 + 4 * g;
+    for (int r = tid / GROUPS; r < WTM; r += ROWS_PER_PASS) {
+        const int m = m0 + r;
+        if (m >= M || n >= N) continue;
+        float4v sum = *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(lds_bytes) + r * LDP + 4 * g);
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w)
+            sum += *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(lds_bytes + w * WAVE_BYTES) + r * LDP + 4 * g);
+        float v[4] = {sum[0], sum[1], sum[2], sum[3]};
+        const int64_t at = static_cast<int64_t>(m) * p.ldd + n;
+        u32x2 c2 = {0, 0}, b2 = {0, 0};
+        if (n + 3 < N) {
+            if (use_c) c2 = *reinterpret_cast<const u32x2_rows *>(p.C + at);
+            if (p.bias) b2 = *reinterpret_cast<const u32x2_rows *>(p.bias + n);
+            finish4<BF16>(p, v, c2, b2, use_c);
+            u32x2 o;
+            o[0] = pack2<BF16>(v[0], v[1]);
+            o[1] = pack2<BF16>(v[2], v[3]);
+            *reinterpret_cast<u32x2_rows *>(p.D + at) = o;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e >= N) continue;
+                if (use_c) c2[e >> 1] |= static_cast<uint32_t>(p.C[at + e]) << ((e & 1) * 16);
+                if (p.bias) b2[e >> 1] |= static_cast<uint32_t>(p.bias[n + e]) << ((e & 1) * 16);
+            }
+            finish4<BF16>(p, v, c2, b2, use_c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) p.D[at + e] = from_float<BF16>(v[e]);
+        }
+    }
+}
+
+template <int TM, int TN, int WAVES, bool BF16>
+int launch_wave_k(Params p, hipStream_t stream) {
+    constexpr size_t lds_bytes = static_cast<size_t>(WAVES) * 2 * (32 * TM + 32 * TN) * kBK * 2;
+    if (p.K % 8 != 0 || p.k_slice != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variant takes a whole K that is a multiple of 8");
+    auto kernel = gemm16_wave_k_kernel<TM, TN, WAVES, BF16>;
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK) return st;
+    p.tiles_n = (p.N + 32 * TN - 1) / (32 * TN);
+    const int64_t tiles = static_cast<int64_t>((p.M + 32 * TM - 1) / (32 * TM)) * p.tiles_n;
+    if (tiles > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: too many tiles for the wave-K variant");
+    p.nblocks = static_cast<int>(tiles);
+    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(64 * WAVES), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 template <class T, bool BF16>
 int launch_persistent(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
@@ -1505,6 +1727,26 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
     return KO_OK;
 }
 
+// Which problems go to the kernel that splits K over the waves of a workgroup (gemm16_wave_k_kernel; B column-major):
+// those whose output is at most one workgroup per compute unit of its tiles - the smallest of 32 x 32 (K over eight
+// waves), 32 x 64 and 64 x 64 (over four) that the problem does not exceed that with - and whose K is neither so
+// shallow that the other kernels' few steps cost nothing, nor so deep that the bytes a small tile draws from the
+// L2s per flop outweigh the steps saved (a compute unit takes in some 85 GB/s this way: 768 x 768 x 16384 on
+// 64 x 64 tiles 47 us, in K slices of 128 x 128 tiles 42).  Measured against the dispatch below (hipBLASLt), us:
+// 100 x 1024 x 1024 9.0 -> 5.7 (5.5), 256 x 768 x 3072 12.5 -> 8.1 (8.6), 512 x 1024 x 4096 17.7 -> 12.3 (13.6),
+// 100 x 4096 x 4096 19.5 -> 11.7 (14.4), 1000 x 1024 x 4096 24.4 -> 18.3 (18.0), 768 x 768 x 4096 19.8 -> 16.0 (16.2),
+// 32 x 768 x 3072 11.4 -> 6.5 (7.1); with more tiles than compute units it loses (512 x 3072 x 768: 10.3 against 14.1).
+// Returns 0, or 3232, 3264, 6464.
+int wave_k_tile(int64_t m, int64_t n, int64_t k) {
+    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k > 8192) return 0;
+    const int64_t cu = compute_units();
+    const int64_t m32 = (m + 31) / 32, m64 = (m + 63) / 64, n32 = (n + 31) / 32, n64 = (n + 63) / 64;
+    if (m32 * n32 <= cu) return k >= 128 ? 3232 : 0;
+    if (m32 * n64 <= cu) return k >= 256 ? 3264 : 0;
+    if (m64 * n64 <= cu) return k >= 1024 ? 6464 : 0;
+    return 0;
+}
+
 // One call becomes at most five launches: one column cut (left, right), then at most two row cuts in the left
 // part (the rows below the last full round, and of those the rows below the last full tile row) and one in the
 // right part.  col_cut / row_cuts are what a (sub-)problem may still spend; the knobs are read once per call.
@@ -1515,6 +1757,17 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         variant = tuning(knob_gemm16_variant);
         split_knob = tuning(knob_gemm16_split_rows);
         if (variant < 0) variant = 0;
+    }
+    if constexpr (!B_ROW_MAJOR) {
+        if (variant <= 0 && p.k_slice == 0) {
+            // the whole problem, or a part cut off it, when it is small
+            switch (wave_k_tile(p.M, p.N, p.K)) {
+                case 3232: return launch_wave_k<1, 1, 8, BF16>(p, stream);
+                case 3264: return launch_wave_k<1, 2, 4, BF16>(p, stream);
+                case 6464: return launch_wave_k<2, 2, 4, BF16>(p, stream);
+                default: break;
+            }
+        }
     }
     if (variant <= 0 && p.k_slice == 0) {
         // the whole problem, or a part cut off it (the launches of one call follow each other on the stream and may
@@ -1674,6 +1927,18 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // M any multiple of 8
         case 61: return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 70:
+        case 71:
+        case 72:
+        case 73:
+            if constexpr (B_ROW_MAJOR) {
+                return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variants need column-major B");
+            } else {
+                if (variant == 70) return launch_wave_k<2, 2, 4, BF16>(p, stream);  // 64 x 64 tiles, K over 4 waves
+                if (variant == 71) return launch_wave_k<1, 2, 4, BF16>(p, stream);  // 32 x 64
+                if (variant == 72) return launch_wave_k<1, 1, 8, BF16>(p, stream);  // 32 x 32, K over 8 waves
+                return launch_wave_k<1, 2, 6, BF16>(p, stream);                     // 32 x 64, K over 6 waves
+            }
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
@@ -1728,10 +1993,19 @@ KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, co
                                       stream);
 }
 
-int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile) {
+int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile) {
     using namespace ko;
-    if (!slices || !k_slice || !tile || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
+    if (!slices || !k_slice || !tile || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30) ||
+        (b_layout != KO_ROW_MAJOR && b_layout != KO_COL_MAJOR))
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16_plan: bad argument");
+    if (b_layout == KO_COL_MAJOR && k % 8 == 0) {
+        if (const int wave_k = wave_k_tile(m, n, k); wave_k != 0) {
+            *slices = 1;
+            *k_slice = 0;
+            *tile = wave_k;
+            return KO_OK;
+        }
+    }
     Params p{};
     p.M = static_cast<int>(m);
     p.N = static_cast<int>(n);

@@ -33,7 +33,7 @@ int hip_fail(hipError_t err, const char *expr, const char *file, int line);
     X(sgemm_variant, "sgemm.variant") X(sgemm_mapping, "sgemm.mapping") X(sgemm_split_rows, "sgemm.split_rows") \
     X(sgemm_k_slices, "sgemm.k_slices") X(gemm16_k_slices, "gemm16.k_slices") X(layernorm_block_rows, "layernorm.block_rows") X(sgemm_slice_variant, "sgemm.slice_variant") X(sgemm_unaligned, "sgemm.unaligned")                                                                     \
     X(gemm16_variant, "gemm16.variant") X(gemm16_mapping, "gemm16.mapping")                                 \
-    X(gemm16_split_rows, "gemm16.split_rows") X(copy_blocks_per_cu, "copy.blocks_per_cu")                   \
+    X(gemm16_split_rows, "gemm16.split_rows") X(gemm16_wave_k, "gemm16.wave_k") X(copy_blocks_per_cu, "copy.blocks_per_cu")                   \
     X(copy_nontemporal, "copy.nontemporal")
 enum Knob {
 #define KO_KNOB_ENUM(id, name) knob_##id,
@@ -83,7 +83,7 @@ int stream_workspace_count();
 
 // What the GEMM planners decide for a shape, for the harness (ko_harness_hooks_t::sgemm_plan, gemm16_plan).
 int debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
-int debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile);
+int debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile);
 
 }  // namespace ko
 

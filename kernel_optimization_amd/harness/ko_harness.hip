@@ -82,8 +82,8 @@ KO_EXPORT int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, 
     return ko::hooks()->sgemm_plan(m, n, k, slices, k_slice, variant);
 }
 
-KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *tile) {
-    return ko::hooks()->gemm16_plan(m, n, k, slices, k_slice, tile);
+KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile) {
+    return ko::hooks()->gemm16_plan(m, n, k, b_layout, slices, k_slice, tile);
 }
 
 KO_EXPORT int ko_debug_stream_workspace_count(int *count) {

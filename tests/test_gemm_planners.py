@@ -37,14 +37,26 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
             assert plan[2] != 40 or (n % 4 == 0 and k % 4 == 0), plan   # not with four-byte operand loads
 
 
+@pytest.mark.parametrize("b_layout", [ko.COL_MAJOR, ko.ROW_MAJOR])
 @pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
-def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n):
+def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
     for k in DEPTHS:
-        plan = ko.gemm_plan(m, n, k, sixteen_bit=True)
+        plan = ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=b_layout)
         _check(m, n, k, plan, k_tile=64, min_k=1536, row_pad=4)   # rows of partial products: whole groups of 4
-        assert plan[2] in ((128, 64, 32) if plan[0] > 1 else (0,))
-        if plan[2] == 32:
-            assert m <= 32
+        if plan[0] > 1:
+            assert plan[2] in (128, 64, 32)
+            if plan[2] == 32:
+                assert m <= 32
+            continue
+        # one launch: whole, or K split over the waves of workgroups that own one small output tile each - a
+        # column-major B only, a multiple of 8 deep (as every K the operator takes), at most one such tile per
+        # compute unit, and the smallest tile for which that holds
+        assert plan[1] == 0 and plan[2] in (0, 3232, 3264, 6464)
+        if plan[2]:
+            tm, tn = divmod(plan[2], 100)
+            assert b_layout == ko.COL_MAJOR and k % 8 == 0 and 128 <= k <= 8192
+            assert -(-m // tm) * -(-n // tn) <= 256
+            assert plan[2] == 3232 or -(-m // 32) * -(-n // 32) > 256
 
 
 def test_measured_decisions_stay_put():
@@ -55,7 +67,15 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(4096, 4096, 4096)[0] == 1
     assert ko.gemm_plan(256, 256, 512)[0] == 1
     assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (7, 2368, 128)
-    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (4, 2048, 64)
+    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (4, 2048, 64)
+    # few tiles, column-major B, K up to 8192: one launch that splits K over the waves of a workgroup
+    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (1, 0, 3232)
+    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 3232)
+    assert ko.gemm_plan(512, 1024, 4096, sixteen_bit=True) == (1, 0, 3264)
+    assert ko.gemm_plan(1000, 1024, 4096, sixteen_bit=True) == (1, 0, 6464)
+    assert ko.gemm_plan(1000, 1024, 768, sixteen_bit=True) == (1, 0, 0)       # 64 x 64 tiles only from K = 1024 on
+    assert ko.gemm_plan(512, 3072, 768, sixteen_bit=True) == (1, 0, 0)        # more tiles than compute units
+    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)
     assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
     assert ko.gemm_plan(16384, 3072, 768, sixteen_bit=True)[0] == 1
     # operand rows off 16-byte boundaries are sliced like the others
