@@ -309,7 +309,8 @@ def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
 
 def gemm_plan(m, n, k, sixteen_bit=False, b_layout=COL_MAJOR):
     """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM (with B in b_layout) decides
-    for a shape; (1, 0, 3232 | 3264 | 6464) is the 16-bit GEMM's one launch that splits K over the waves of a workgroup."""
+    for a shape; (1, 0, 1000 * rows + columns) is the 16-bit GEMM's one launch whose workgroups own one output tile of
+    that size (32 x 32 to 128 x 64) and split K over their waves."""
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     if sixteen_bit:
         check(harness().ko_debug_gemm16_plan(m, n, k, b_layout, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))

@@ -1313,7 +1313,7 @@ int launch_pinned(Params p, hipStream_t stream) {
 // matrix): every kernel above walks K in steps that all waves of a workgroup take together - a barrier per K tile,
 // one or two K tiles in flight per workgroup - and with a workgroup or less per compute unit such a step costs its
 // latencies (0.4 us per 64 k on 64 x 64 tiles, whatever the arithmetic).  Here a workgroup owns one (32 TM) x (32 TN)
-// output tile and wave w multiplies K tiles w, w + WAVES, ... of it: the whole tile over its own share of K, out of two
+// output tile (32 x 32 to 128 x 64) and wave w multiplies K tiles w, w + WAVES, ... of it: the whole tile over its own share of K, out of two
 // LDS stages of its own that it fills with direct-to-LDS loads (eight rows of 128 bytes per wave-level load, as
 // in the kernels above) - no barrier in the loop, WAVES times fewer steps in a row, and two K tiles per wave in
 // flight.  At the end the waves leave their fp32 tiles in LDS and the workgroup adds them in wave order (the same
@@ -1331,13 +1331,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
     constexpr int LDP = WTN + 4;  // floats between the rows of a wave's fp32 tile in LDS
     static_assert(KS == 4 && LOADS <= 31, "two K tiles of loads must fit the 6-bit counter");
     static_assert(WTM * LDP * 4 <= WAVE_BYTES && WAVES * WAVE_BYTES <= 160 * 1024, "");
-    static_assert((TM == 1 || TM == 2) && (TN == 1 || TN == 2), "");
+    static_assert(TM * TN <= 8 && TM + TN <= 6, "");
 
     extern __shared__ u32x4 lds[];
     char *const lds_bytes = reinterpret_cast<char *>(lds);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Tiles in row-major order, workgroup b on XCD b % 8: the tiles of one row of tiles - which share their rows of
+    // A - are spread over the XCDs.  (One contiguous range of the tile list per XCD, along the smaller operand, so
+    // that the larger one is shared out between the L2s, was slower: 256 x 4096 x 4096 18.1 -> 20.2 us, 1000 x 1024 x
+    // 4096 18.6 -> 20.5, 100 x 4096 x 4096 11.7 -> 13.0 - the workgroups of an XCD then ask for the same few blocks
+    // at the same moment.)
     const int tile = static_cast<int>(blockIdx.x);
     const int m0 = (tile / p.tiles_n) * WTM, n0 = (tile % p.tiles_n) * WTN;
     const int M = p.M, N = p.N, K = p.K;
@@ -1421,8 +1426,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
         else if constexpr (TM == 2 && TN == 1)
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0])::"memory");
-        else
+        else if constexpr (TM == 4 && TN == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
+        else if constexpr (TM == 2 && TN == 4)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1]), "+v"(bf[slot][2]), "+v"(bf[slot][3])::"memory");
+        else {
+            static_assert(TM == 1 && TN == 1, "");
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0])::"memory");
+        }
     };
     auto multiply = [&](int slot) {
 #pragma unroll
@@ -1736,14 +1749,19 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
 // 100 x 1024 x 1024 9.0 -> 5.7 (5.5), 256 x 768 x 3072 12.5 -> 8.1 (8.6), 512 x 1024 x 4096 17.7 -> 12.3 (13.6),
 // 100 x 4096 x 4096 19.5 -> 11.7 (14.4), 1000 x 1024 x 4096 24.4 -> 18.3 (18.0), 768 x 768 x 4096 19.8 -> 16.0 (16.2),
 // 32 x 768 x 3072 11.4 -> 6.5 (7.1); with more tiles than compute units it loses (512 x 3072 x 768: 10.3 against 14.1).
-// Returns 0, or 3232, 3264, 6464.
+// Beyond that, 64 x 128 or 128 x 64 tiles over three waves (all the LDS stages that fit) from K = 2048 on: 512 x
+// 4096 x 4096 38.0 -> 31.7 (25.7), 2048 x 768 x 3072 27.6 -> 24.9 (18.1), 2048 x 1024 x 4096 37.4 -> 33.8 (25.0).
+// Returns 0, or 1000 * rows + columns of the tile: 32032, 32064, 64064, 64128, 128064.
 int wave_k_tile(int64_t m, int64_t n, int64_t k) {
     if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k > 8192) return 0;
     const int64_t cu = compute_units();
     const int64_t m32 = (m + 31) / 32, m64 = (m + 63) / 64, n32 = (n + 31) / 32, n64 = (n + 63) / 64;
-    if (m32 * n32 <= cu) return k >= 128 ? 3232 : 0;
-    if (m32 * n64 <= cu) return k >= 256 ? 3264 : 0;
-    if (m64 * n64 <= cu) return k >= 1024 ? 6464 : 0;
+    if (m32 * n32 <= cu) return k >= 128 ? 32032 : 0;
+    if (m32 * n64 <= cu) return k >= 256 ? 32064 : 0;
+    if (m64 * n64 <= cu) return k >= 1024 ? 64064 : 0;
+    if (k < 2048) return 0;
+    if (m64 * ((n + 127) / 128) <= cu) return 64128;
+    if (((m + 127) / 128) * n64 <= cu) return 128064;
     return 0;
 }
 
@@ -1762,9 +1780,11 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         if (variant <= 0 && p.k_slice == 0) {
             // the whole problem, or a part cut off it, when it is small
             switch (wave_k_tile(p.M, p.N, p.K)) {
-                case 3232: return launch_wave_k<1, 1, 8, BF16>(p, stream);
-                case 3264: return launch_wave_k<1, 2, 4, BF16>(p, stream);
-                case 6464: return launch_wave_k<2, 2, 4, BF16>(p, stream);
+                case 32032: return launch_wave_k<1, 1, 8, BF16>(p, stream);
+                case 32064: return launch_wave_k<1, 2, 4, BF16>(p, stream);
+                case 64064: return launch_wave_k<2, 2, 4, BF16>(p, stream);
+                case 64128: return launch_wave_k<2, 4, 3, BF16>(p, stream);
+                case 128064: return launch_wave_k<4, 2, 3, BF16>(p, stream);
                 default: break;
             }
         }
@@ -1931,13 +1951,17 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 71:
         case 72:
         case 73:
+        case 74:
+        case 75:
             if constexpr (B_ROW_MAJOR) {
                 return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variants need column-major B");
             } else {
                 if (variant == 70) return launch_wave_k<2, 2, 4, BF16>(p, stream);  // 64 x 64 tiles, K over 4 waves
                 if (variant == 71) return launch_wave_k<1, 2, 4, BF16>(p, stream);  // 32 x 64
                 if (variant == 72) return launch_wave_k<1, 1, 8, BF16>(p, stream);  // 32 x 32, K over 8 waves
-                return launch_wave_k<1, 2, 6, BF16>(p, stream);                     // 32 x 64, K over 6 waves
+                if (variant == 73) return launch_wave_k<1, 2, 6, BF16>(p, stream);  // 32 x 64, K over 6 waves
+                if (variant == 74) return launch_wave_k<4, 2, 3, BF16>(p, stream);  // 128 x 64, K over 3 waves
+                return launch_wave_k<2, 4, 3, BF16>(p, stream);                     // 64 x 128, K over 3 waves
             }
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }

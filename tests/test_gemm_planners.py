@@ -51,12 +51,12 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
         # one launch: whole, or K split over the waves of workgroups that own one small output tile each - a
         # column-major B only, a multiple of 8 deep (as every K the operator takes), at most one such tile per
         # compute unit, and the smallest tile for which that holds
-        assert plan[1] == 0 and plan[2] in (0, 3232, 3264, 6464)
+        assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064)
         if plan[2]:
-            tm, tn = divmod(plan[2], 100)
+            tm, tn = divmod(plan[2], 1000)
             assert b_layout == ko.COL_MAJOR and k % 8 == 0 and 128 <= k <= 8192
             assert -(-m // tm) * -(-n // tn) <= 256
-            assert plan[2] == 3232 or -(-m // 32) * -(-n // 32) > 256
+            assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
 
 
 def test_measured_decisions_stay_put():
@@ -69,10 +69,12 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (7, 2368, 128)
     assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (4, 2048, 64)
     # few tiles, column-major B, K up to 8192: one launch that splits K over the waves of a workgroup
-    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (1, 0, 3232)
-    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 3232)
-    assert ko.gemm_plan(512, 1024, 4096, sixteen_bit=True) == (1, 0, 3264)
-    assert ko.gemm_plan(1000, 1024, 4096, sixteen_bit=True) == (1, 0, 6464)
+    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (1, 0, 32032)
+    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 32032)
+    assert ko.gemm_plan(512, 1024, 4096, sixteen_bit=True) == (1, 0, 32064)
+    assert ko.gemm_plan(1000, 1024, 4096, sixteen_bit=True) == (1, 0, 64064)
+    assert ko.gemm_plan(2048, 768, 3072, sixteen_bit=True) == (1, 0, 64128)
+    assert ko.gemm_plan(9000, 192, 2048, sixteen_bit=True) == (1, 0, 128064)
     assert ko.gemm_plan(1000, 1024, 768, sixteen_bit=True) == (1, 0, 0)       # 64 x 64 tiles only from K = 1024 on
     assert ko.gemm_plan(512, 3072, 768, sixteen_bit=True) == (1, 0, 0)        # more tiles than compute units
     assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)

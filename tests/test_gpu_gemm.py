@@ -951,8 +951,8 @@ def test_gemm16_ragged_rows_through_the_default_dispatch_are_exact(ko, m, n, k):
 
 
 # K split over the waves of a workgroup (few output tiles, column-major B): 70 = 64 x 64 tiles over 4 waves,
-# 71 = 32 x 64 over 4, 72 = 32 x 32 over 8, 73 = 32 x 64 over 6
-WAVE_K_VARIANTS = [70, 71, 72, 73]
+# 71 = 32 x 64 over 4, 72 = 32 x 32 over 8, 73 = 32 x 64 over 6, 74 = 128 x 64 over 3, 75 = 64 x 128 over 3
+WAVE_K_VARIANTS = [70, 71, 72, 73, 74, 75]
 
 
 @pytest.mark.parametrize("variant", WAVE_K_VARIANTS)
@@ -1003,8 +1003,9 @@ def test_gemm16_wave_k_variants_are_exact_on_small_integers(ko, variant):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("m,n,k,tile", [(100, 1024, 1024, 3232), (512, 768, 3072, 3264), (1000, 1024, 4096, 6464),
-                                        (8, 4096, 4096, 3232), (200, 2304, 768, 3264), (750, 1000, 1032, 6464)])
+@pytest.mark.parametrize("m,n,k,tile", [(100, 1024, 1024, 32032), (512, 768, 3072, 32064), (1000, 1024, 4096, 64064),
+                                        (8, 4096, 4096, 32032), (200, 2304, 768, 32064), (750, 1000, 1032, 64064),
+                                        (2040, 700, 2056, 64128), (9000, 192, 2048, 128064)])
 def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, bf16):
     """A few hundred rows against a weight matrix (column-major B): the dispatch sends them to the kernel that splits K
     over the waves of a workgroup - the plan query says which tile - and the whole output agrees with the oracle,
