@@ -239,7 +239,7 @@ def bench_sgemm(cfg, steps, warmup, vendor, shape=None):
     return res, keep
 
 
-def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
+def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None, c_loop=False):
     """Configuration 4 (B column-major, both operands K-contiguous) or, with b_row_major, the same product with B
     handed over as [K][N], the layout of the reference's own tensor-core kernel (tensor_core_gemm.h:178)."""
     c = inputs.CONFIGS[cfg]
@@ -255,6 +255,10 @@ def bench_gemm16(cfg, steps, warmup, vendor, b_row_major=False, shape=None):
     layout = ko.ROW_MAJOR if b_row_major else ko.COL_MAJOR
     wall, dev = _time_steps(lambda i: ko.gemm16(m, n, k, As[i % nsets], Bs[i % nsets], Ds[i % nsets], b_layout=layout),
                             steps, warmup)
+    if c_loop:
+        # kernels of a few microseconds: launched from a loop in C, as the vendor library's are below (a Python loop
+        # launches one every 4-8 us); the median of three batches
+        dev = ko.time_gemm16_sets(m, n, k, As, Bs, Ds, b_layout=layout, warmup=warmup, reps=steps, batches=3) * 1e-6
     name = c["name"] if shape is None else "gemm_f16_%dx%dx%d" % (m, n, k)
     if b_row_major:
         name = name.replace("gemm_f16_", "gemm_f16_rowmajorB_")
@@ -482,7 +486,7 @@ def bench_gemm16_midsize(steps, warmup, vendor):
     rows = []
     for n, k in MIDSIZE_WEIGHTS:
         for m in MIDSIZE_ROWS:
-            res, _ = bench_gemm16(4, steps, warmup, vendor, shape=(m, n, k))
+            res, _ = bench_gemm16(4, steps, warmup, vendor, shape=(m, n, k), c_loop=True)
             slices, k_slice, tile = ko.gemm_plan(m, n, k, sixteen_bit=True)
             rows.append(dict(m=m, n=n, k=k, us=res["kernel_us"], tflops=res["roofline"]["achieved"]
                              if res["roofline"]["unit"] == "TFLOP/s" else res["flops"] / res["kernel_us"] / 1e6,

@@ -63,6 +63,12 @@ int ko_copy_f32(const float *in, float *out, int64_t n, ko_stream_t stream);
 int ko_stream_probe(const void *in, void *out, int64_t nbytes, int mode, int vectors_per_thread,
                     int threads, int blocks_per_cu, int load_policy, int store_policy, int read_of_128,
                     int lds_pad_bytes, ko_stream_t stream);
+/* Times ko_gemm_f16f32acc (alpha 1, no C) from a host loop in C, as the vendor library's kernels are timed by the
+ * comparison harness: `warmup` launches, then `batches` batches of `reps` launches between two events on the
+ * default stream, launch i on operand set i % nsets (A, B, D: arrays of nsets device pointers); *median_us is the
+ * median batch's time per launch.  For kernels of a few microseconds a Python loop cannot launch fast enough. */
+int ko_time_gemm16_sets(int64_t m, int64_t n, int64_t k, const void *const *A, const void *const *B, void *const *D,
+                        int nsets, int b_layout, int dtype, int warmup, int reps, int batches, float *median_us);
 /* Integer tuning knobs by name ("softmax.lanes_per_row", ...); value 0 restores the default.
  * Unknown names return KO_ERR_INVALID_ARGUMENT. */
 int ko_set_tuning(const char *name, int value);

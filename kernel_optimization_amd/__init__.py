@@ -87,6 +87,8 @@ HARNESS_SIGNATURES = {
     "ko_get_tuning": (_int, [ctypes.c_char_p, ctypes.POINTER(_int)]),
     "ko_debug_wave_allreduce": (_int, [_vp, _vp, _int, _int, _vp]),
     "ko_debug_stream_workspace_count": (_int, [ctypes.POINTER(_int)]),
+    "ko_time_gemm16_sets": (_int, [_i64, _i64, _i64, ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp), _int,
+                                   _int, _int, _int, _int, _int, ctypes.POINTER(ctypes.c_float)]),
     "ko_debug_sgemm_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
                                    ctypes.POINTER(ctypes.c_int)]),
     "ko_debug_gemm16_plan": (_int, [_i64, _i64, _i64, _int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
@@ -317,6 +319,16 @@ def gemm_plan(m, n, k, sixteen_bit=False, b_layout=COL_MAJOR):
     else:
         check(harness().ko_debug_sgemm_plan(m, n, k, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
     return a.value, b.value, c.value
+
+
+def time_gemm16_sets(m, n, k, As, Bs, Ds, b_layout=COL_MAJOR, dtype=F16, warmup=100, reps=30, batches=3):
+    """Microseconds per ko_gemm_f16f32acc launch, timed from a host loop in C (the median of `batches` batches of
+    `reps` launches after `warmup` launches), launch i on the operand set i % len(As)."""
+    arr = lambda bufs: (ctypes.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+    us = ctypes.c_float()
+    check(harness().ko_time_gemm16_sets(m, n, k, arr(As), arr(Bs), arr(Ds), len(As), b_layout, dtype, warmup, reps,
+                                        batches, ctypes.byref(us)))
+    return us.value
 
 
 def sgemm_static_scratch(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):

@@ -5,6 +5,7 @@
 #include "ko_internal.h"
 #include "wave64.h"
 
+#include <algorithm>
 #include <cstring>
 
 namespace ko {
@@ -84,6 +85,43 @@ KO_EXPORT int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, 
 
 KO_EXPORT int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile) {
     return ko::hooks()->gemm16_plan(m, n, k, b_layout, slices, k_slice, tile);
+}
+
+KO_EXPORT int ko_time_gemm16_sets(int64_t m, int64_t n, int64_t k, const void *const *A, const void *const *B,
+                                  void *const *D, int nsets, int b_layout, int dtype, int warmup, int reps, int batches,
+                                  float *median_us) {
+    if (!A || !B || !D || !median_us || nsets <= 0 || warmup < 0 || reps <= 0 || batches <= 0 || batches > 64)
+        return ko::fail(KO_ERR_INVALID_ARGUMENT, "ko_time_gemm16_sets: bad argument");
+    auto call = [&](int i) {
+        const int s = i % nsets;
+        return ko_gemm_f16f32acc(m, n, k, 1.0f, A[s], B[s], b_layout, 0.0f, nullptr, D[s], dtype, nullptr);
+    };
+    for (int i = 0; i < warmup; ++i)
+        if (const int st = call(i); st != KO_OK) return st;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    KO_HIP(hipEventCreate(&e0));
+    if (const hipError_t e = hipEventCreate(&e1); e != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return ko::hip_fail(e, "hipEventCreate", __FILE__, __LINE__);
+    }
+    float us[64];
+    int st = KO_OK;
+    for (int b = 0; b < batches && st == KO_OK; ++b) {
+        (void)hipEventRecord(e0, nullptr);
+        for (int r = 0; r < reps && st == KO_OK; ++r) st = call(warmup + b * reps + r);
+        (void)hipEventRecord(e1, nullptr);
+        if (const hipError_t e = hipEventSynchronize(e1); e != hipSuccess && st == KO_OK)
+            st = ko::hip_fail(e, "hipEventSynchronize", __FILE__, __LINE__);
+        float ms = 0.0f;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        us[b] = ms * 1e3f / reps;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (st != KO_OK) return st;
+    std::sort(us, us + batches);
+    *median_us = us[batches / 2];
+    return KO_OK;
 }
 
 KO_EXPORT int ko_debug_stream_workspace_count(int *count) {
