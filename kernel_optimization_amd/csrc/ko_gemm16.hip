@@ -1321,8 +1321,12 @@ int launch_pinned(Params p, hipStream_t stream) {
 // Any M, N and any K that is a multiple of 8: a row at or past M (N) is fetched from the last row instead and its
 // results are not stored; a 16-byte chunk at or past K - in the last K tile, or in a K tile past the end that a
 // wave's second stage asks for - is fetched from sixteen zero bytes, chosen per load with a compare and two selects.
-// B column-major ([N][K], K contiguous) only.
-template <int TM, int TN, int WAVES, bool BF16>
+// B_ROW: B as [K][N] (rows ldb apart, N and ldb multiples of 8).  A wave's K tile of B is 64 rows of 32 TN values and
+// stays row-major in LDS; a wave-level load covers 1 KB of it (16, 8 or 4 rows), the 16-byte chunk a lane fetches
+// is permuted with the row number modulo 4 - as far as the row has chunks for it - and the fragments come out of
+// transposing LDS reads as in the pinned kernel (read_b_transposed has the lane arithmetic); a chunk at or past N
+// or a row at or past K is fetched from the zeros.
+template <int TM, int TN, int WAVES, bool BF16, bool B_ROW = false>
 __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params p) {
     constexpr int WTM = 32 * TM, WTN = 32 * TN;
     constexpr int KS = kBK / 16;
@@ -1367,13 +1371,27 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
         const int r = m0 + 8 * i + row_in;
         src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + wave * kBK + lane_k[i & 1]);
     }
+    // row-major B: NCH chunks per LDS row, RPL rows per wave-level load; lane l fills position l % NCH of row
+    // l / NCH of its load's rows, with chunk (l % NCH) ^ b_swz(row) of that row of the tile
+    constexpr int NCH = WTN / 8, RPL = 64 / NCH, B_ROW_BYTES = WTN * 2;
+    auto b_swz = [](int k) { return ((k & 3) << 2) & (NCH - 1); };
+    const int b_krow = lane / NCH;  // + RPL * j: the row, within the K tile, that this lane fetches in load j
+    bool b_inside = true;           // row-major B: this lane's chunk lies inside N (the same chunk in every load: RPL % 4 == 0)
 #pragma unroll
     for (int j = 0; j < B_LOADS; ++j) {
-        const int r = n0 + 8 * j + row_in;
-        src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + wave * kBK + lane_k[j & 1]);
+        if constexpr (B_ROW) {
+            static_assert(RPL % 4 == 0, "");
+            const int c = n0 + 8 * ((lane % NCH) ^ b_swz(b_krow));
+            b_inside = c < N;
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(wave * kBK + RPL * j + b_krow) * p.ldb + (b_inside ? c : 0));
+        } else {
+            const int r = n0 + 8 * j + row_in;
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + wave * kBK + lane_k[j & 1]);
+        }
     }
     int ld_k0 = wave * kBK;  // first k of the K tile to fetch next
     char *const wave_lds = lds_bytes + wave * WAVE_BYTES;
+    const int64_t b_tile_step = B_ROW ? static_cast<int64_t>(WAVES * kBK) * p.ldb * 2 : WAVES * kBK * 2;  // bytes to this wave's next K tile
     auto issue = [&](int stage) {
         const bool in0 = ld_k0 + lane_k[0] < K, in1 = ld_k0 + lane_k[1] < K;
         char *dst = wave_lds + stage * STAGE_BYTES;
@@ -1384,8 +1402,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
         }
 #pragma unroll
         for (int j = 0; j < B_LOADS; ++j) {
-            __builtin_amdgcn_global_load_lds((gptr_t)((j & 1 ? in1 : in0) ? src_b[j] : zeros), (lptr_t)(dst + A_BYTES + 1024 * j), 16, 0, 0);
-            src_b[j] += WAVES * kBK * 2;
+            bool in = j & 1 ? in1 : in0;
+            if constexpr (B_ROW) in = b_inside && ld_k0 + RPL * j + b_krow < K;
+            __builtin_amdgcn_global_load_lds((gptr_t)(in ? src_b[j] : zeros), (lptr_t)(dst + A_BYTES + 1024 * j), 16, 0, 0);
+            src_b[j] += b_tile_step;
         }
         ld_k0 += WAVES * kBK;
     };
@@ -1407,6 +1427,19 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     u32x4 af[2][TM], bf[2][TN];
+    // row-major B: the two halves of a B fragment as the transposing reads deliver them (k .. k+3 and k+4 .. k+7 of
+    // this lane's column), and where the lane reads them (K step 0 of stage 0): lane i of a group of 16 points at row
+    // i / 4 of the K step's rows, columns 4 (i % 4) .. + 3 of the group's 16
+    u32x2 b_lo[2][B_ROW ? TN : 1], b_hi[2][B_ROW ? TN : 1];
+    uint32_t off_br[B_ROW ? TN : 1];
+    if constexpr (B_ROW) {
+        const int i = lane & 15, g = (lane >> 4) & 1, kq = i >> 2;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int chunk = ((j * 32 + g * 16 + 4 * (i & 3)) >> 3) ^ b_swz(kq);
+            off_br[j] = frag_base + A_BYTES + (fhalf * 8 + kq) * B_ROW_BYTES + chunk * 16 + (i & 1) * 8;
+        }
+    }
     auto read_frags = [&](auto ks_c, auto slot_c, auto stage_c) {
         constexpr int KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value, S = decltype(stage_c)::value;
         static_for<TM>([&](auto i_c) {
@@ -1415,26 +1448,29 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
         });
         static_for<TN>([&](auto j_c) {
             constexpr int J = decltype(j_c)::value;
-            lds_read16<S * STAGE_BYTES + A_BYTES + J * 4096>(bf[SLOT][J], off[KSTEP]);
+            if constexpr (B_ROW) {
+                constexpr int IMM = S * STAGE_BYTES + KSTEP * 16 * B_ROW_BYTES;
+                lds_read_tr<IMM>(b_lo[SLOT][J], off_br[J]);
+                lds_read_tr<IMM + 4 * B_ROW_BYTES>(b_hi[SLOT][J], off_br[J]);
+            } else {
+                lds_read16<S * STAGE_BYTES + A_BYTES + J * 4096>(bf[SLOT][J], off[KSTEP]);
+            }
         });
     };
-    // every read issued so far has landed; the operands keep the matrix instructions that use them behind this point
+    // every read issued so far has landed; each register the reads wrote passes through an empty statement behind the
+    // wait, which keeps the matrix instructions that use it behind this point
     auto wait_frags = [&](int slot) {
-        if constexpr (TM == 2 && TN == 2)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
-        else if constexpr (TM == 1 && TN == 2)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
-        else if constexpr (TM == 2 && TN == 1)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0])::"memory");
-        else if constexpr (TM == 4 && TN == 2)
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(af[slot][2]), "+v"(af[slot][3]), "+v"(bf[slot][0]), "+v"(bf[slot][1])::"memory");
-        else if constexpr (TM == 2 && TN == 4)
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(af[slot][0]), "+v"(af[slot][1]), "+v"(bf[slot][0]), "+v"(bf[slot][1]), "+v"(bf[slot][2]), "+v"(bf[slot][3])::"memory");
-        else {
-            static_assert(TM == 1 && TN == 1, "");
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[slot][0]), "+v"(bf[slot][0])::"memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(af[slot][i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (B_ROW) {
+                asm volatile("" : "+v"(b_lo[slot][j]), "+v"(b_hi[slot][j]));
+                bf[slot][j] = u32x4{b_lo[slot][j][0], b_lo[slot][j][1], b_hi[slot][j][0], b_hi[slot][j][1]};
+            } else {
+                asm volatile("" : "+v"(bf[slot][j]));
+            }
         }
     };
     auto multiply = [&](int slot) {
@@ -1528,11 +1564,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
     }
 }
 
-template <int TM, int TN, int WAVES, bool BF16>
+template <int TM, int TN, int WAVES, bool BF16, bool B_ROW = false>
 int launch_wave_k(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = static_cast<size_t>(WAVES) * 2 * (32 * TM + 32 * TN) * kBK * 2;
     if (p.K % 8 != 0 || p.k_slice != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variant takes a whole K that is a multiple of 8");
-    auto kernel = gemm16_wave_k_kernel<TM, TN, WAVES, BF16>;
+    if (B_ROW && (p.N % 8 != 0 || p.ldb % 8 != 0))
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variant takes a row-major B whose N and row stride are multiples of 8");
+    auto kernel = gemm16_wave_k_kernel<TM, TN, WAVES, BF16, B_ROW>;
     static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK) return st;
     p.tiles_n = (p.N + 32 * TN - 1) / (32 * TN);
@@ -1740,7 +1778,7 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
     return KO_OK;
 }
 
-// Which problems go to the kernel that splits K over the waves of a workgroup (gemm16_wave_k_kernel; B column-major):
+// Which problems go to the kernel that splits K over the waves of a workgroup (gemm16_wave_k_kernel; timings with B column-major):
 // those whose output is at most one workgroup per compute unit of its tiles - the smallest of 32 x 32 (K over eight
 // waves), 32 x 64 and 64 x 64 (over four) that the problem does not exceed that with - and whose K is neither so
 // shallow that the other kernels' few steps cost nothing, nor so deep that the bytes a small tile draws from the
@@ -1776,17 +1814,15 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         split_knob = tuning(knob_gemm16_split_rows);
         if (variant < 0) variant = 0;
     }
-    if constexpr (!B_ROW_MAJOR) {
-        if (variant <= 0 && p.k_slice == 0) {
-            // the whole problem, or a part cut off it, when it is small
-            switch (wave_k_tile(p.M, p.N, p.K)) {
-                case 32032: return launch_wave_k<1, 1, 8, BF16>(p, stream);
-                case 32064: return launch_wave_k<1, 2, 4, BF16>(p, stream);
-                case 64064: return launch_wave_k<2, 2, 4, BF16>(p, stream);
-                case 64128: return launch_wave_k<2, 4, 3, BF16>(p, stream);
-                case 128064: return launch_wave_k<4, 2, 3, BF16>(p, stream);
-                default: break;
-            }
+    if (variant <= 0 && p.k_slice == 0 && (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0))) {
+        // the whole problem, or a part cut off it, when it is small
+        switch (wave_k_tile(p.M, p.N, p.K)) {
+            case 32032: return launch_wave_k<1, 1, 8, BF16, B_ROW_MAJOR>(p, stream);
+            case 32064: return launch_wave_k<1, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
+            case 64064: return launch_wave_k<2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
+            case 64128: return launch_wave_k<2, 4, 3, BF16, B_ROW_MAJOR>(p, stream);
+            case 128064: return launch_wave_k<4, 2, 3, BF16, B_ROW_MAJOR>(p, stream);
+            default: break;
         }
     }
     if (variant <= 0 && p.k_slice == 0) {
@@ -1953,16 +1989,12 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 73:
         case 74:
         case 75:
-            if constexpr (B_ROW_MAJOR) {
-                return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the wave-K variants need column-major B");
-            } else {
-                if (variant == 70) return launch_wave_k<2, 2, 4, BF16>(p, stream);  // 64 x 64 tiles, K over 4 waves
-                if (variant == 71) return launch_wave_k<1, 2, 4, BF16>(p, stream);  // 32 x 64
-                if (variant == 72) return launch_wave_k<1, 1, 8, BF16>(p, stream);  // 32 x 32, K over 8 waves
-                if (variant == 73) return launch_wave_k<1, 2, 6, BF16>(p, stream);  // 32 x 64, K over 6 waves
-                if (variant == 74) return launch_wave_k<4, 2, 3, BF16>(p, stream);  // 128 x 64, K over 3 waves
-                return launch_wave_k<2, 4, 3, BF16>(p, stream);                     // 64 x 128, K over 3 waves
-            }
+            if (variant == 70) return launch_wave_k<2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);  // 64 x 64 tiles, K over 4 waves
+            if (variant == 71) return launch_wave_k<1, 2, 4, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 64
+            if (variant == 72) return launch_wave_k<1, 1, 8, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 32, K over 8 waves
+            if (variant == 73) return launch_wave_k<1, 2, 6, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 64, K over 6 waves
+            if (variant == 74) return launch_wave_k<4, 2, 3, BF16, B_ROW_MAJOR>(p, stream);  // 128 x 64, K over 3 waves
+            return launch_wave_k<2, 4, 3, BF16, B_ROW_MAJOR>(p, stream);                     // 64 x 128, K over 3 waves
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
@@ -2022,7 +2054,7 @@ int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *sl
     if (!slices || !k_slice || !tile || m <= 0 || n <= 0 || k <= 0 || m > (1 << 30) || n > (1 << 30) || k > (1 << 30) ||
         (b_layout != KO_ROW_MAJOR && b_layout != KO_COL_MAJOR))
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16_plan: bad argument");
-    if (b_layout == KO_COL_MAJOR && k % 8 == 0) {
+    if ((b_layout == KO_COL_MAJOR || n % 8 == 0) && k % 8 == 0) {  // (a row-major B: rows of whole 16-byte chunks)
         if (const int wave_k = wave_k_tile(m, n, k); wave_k != 0) {
             *slices = 1;
             *k_slice = 0;

@@ -48,13 +48,13 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
             if plan[2] == 32:
                 assert m <= 32
             continue
-        # one launch: whole, or K split over the waves of workgroups that own one small output tile each - a
-        # column-major B only, a multiple of 8 deep (as every K the operator takes), at most one such tile per
-        # compute unit, and the smallest tile for which that holds
+        # one launch: whole, or K split over the waves of workgroups that own one small output tile each - B
+        # column-major, or row-major with rows of whole 16-byte chunks; a multiple of 8 deep (as every K the operator
+        # takes); at most one such tile per compute unit, and the smallest tile for which that holds
         assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064)
         if plan[2]:
             tm, tn = divmod(plan[2], 1000)
-            assert b_layout == ko.COL_MAJOR and k % 8 == 0 and 128 <= k <= 8192
+            assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and k % 8 == 0 and 128 <= k <= 8192
             assert -(-m // tm) * -(-n // tn) <= 256
             assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
 
@@ -67,7 +67,7 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(4096, 4096, 4096)[0] == 1
     assert ko.gemm_plan(256, 256, 512)[0] == 1
     assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (7, 2368, 128)
-    assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (4, 2048, 64)
+    assert ko.gemm_plan(512, 520, 16384, sixteen_bit=True, b_layout=ko.ROW_MAJOR)[0] > 1
     # few tiles, column-major B, K up to 8192: one launch that splits K over the waves of a workgroup
     assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (1, 0, 32032)
     assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 32032)
@@ -77,7 +77,8 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(9000, 192, 2048, sixteen_bit=True) == (1, 0, 128064)
     assert ko.gemm_plan(1000, 1024, 768, sixteen_bit=True) == (1, 0, 0)       # 64 x 64 tiles only from K = 1024 on
     assert ko.gemm_plan(512, 3072, 768, sixteen_bit=True) == (1, 0, 0)        # more tiles than compute units
-    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)
+    assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 32032)
+    assert ko.gemm_plan(100, 1028, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)  # rows of B off 16 bytes
     assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
     assert ko.gemm_plan(16384, 3072, 768, sixteen_bit=True)[0] == 1
     # operand rows off 16-byte boundaries are sliced like the others

@@ -957,25 +957,30 @@ WAVE_K_VARIANTS = [70, 71, 72, 73, 74, 75]
 
 @pytest.mark.parametrize("variant", WAVE_K_VARIANTS)
 @pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k", [(1, 1, 8), (33, 36, 8), (64, 64, 64), (100, 200, 1032), (31, 67, 136), (130, 75, 4104),
-                                   (256, 256, 2048), (65, 129, 72), (96, 128, 448), (8, 520, 1544)])
-def test_gemm16_wave_k_variants_match_oracle(ko, variant, bf16, m, n, k):
+                                   (256, 256, 2048), (65, 129, 72), (96, 128, 448), (8, 520, 1544), (70, 8, 264),
+                                   (40, 328, 200)])
+def test_gemm16_wave_k_variants_match_oracle(ko, variant, bf16, b_col_major, m, n, k):
     """Every wave of a workgroup multiplies its own K tiles (w, w + WAVES, ...) of the workgroup's one output tile and
     the partial tiles are added in wave order: against the oracle, plain and with the whole epilogue (beta C, bias,
     activation), bit-stable from call to call - ragged M and N, row lengths of D off 8 bytes, a K that ends inside
-    a K tile, fewer K tiles than waves, more K tiles than one round of the waves' two stages."""
+    a K tile, fewer K tiles than waves, more K tiles than one round of the waves' two stages.  B as [N][K], or as
+    [K][N] when N is a multiple of 8 (rows of whole 16-byte chunks)."""
+    if not b_col_major and n % 8:
+        pytest.skip("a row-major B off 16-byte rows does not go to these kernels")
     A = _bits16((m, k), 91 + m, bf16)
-    B = _bits16((n, k), 93 + n, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 93 + n, bf16)
     C = _bits16((m, n), 95, bf16)
     bias = _bits16((n,), 97, bf16)
-    kw = dict(dtype=ko.BF16 if bf16 else ko.F16)
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
     ko.set_tuning("gemm16.variant", variant)
     try:
-        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major)
         got = ko.gemm16_host(A, B, m, n, k, **kw)
         assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
         np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, **kw), got)
-        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, C_bits=C, beta=0.5, bias_bits=bias, act=2)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major, C_bits=C, beta=0.5, bias_bits=bias, act=2)
         got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
         assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap + 2.0, k, bf16=bf16)
     finally:
@@ -990,14 +995,18 @@ def test_gemm16_wave_k_variants_are_exact_on_small_integers(ko, variant):
     rng = np.random.default_rng(variant)
     ko.set_tuning("gemm16.variant", variant)
     try:
-        for m, n, k in ((96, 200, 128), (70, 90, 456), (33, 64, 1992), (128, 32, 72), (257, 100, 328)):
+        for m, n, k in ((96, 200, 128), (70, 90, 456), (33, 64, 1992), (128, 32, 72), (257, 100, 328), (100, 328, 520)):
             Ai = rng.integers(-2, 3, (m, k)).astype(np.float16)
             Bi = rng.integers(-2, 3, (n, k)).astype(np.float16)  # [n][k]
             scale = 64.0 / k if k > 64 else 1.0  # keeps |sum| below 2^11: thin out the non-zeros of A
             Ai[rng.random((m, k)) > scale] = 0
+            want = Ai.astype(np.float64) @ Bi.astype(np.float64).T
             got = ko.gemm16_host(Ai.view(np.uint16), Bi.view(np.uint16), m, n, k).view(np.float16)
-            np.testing.assert_array_equal(got.astype(np.float64), Ai.astype(np.float64) @ Bi.astype(np.float64).T,
-                                          err_msg="%dx%dx%d" % (m, n, k))
+            np.testing.assert_array_equal(got.astype(np.float64), want, err_msg="%dx%dx%d" % (m, n, k))
+            if n % 8 == 0:  # the same product with B handed over as [K][N]
+                got = ko.gemm16_host(Ai.view(np.uint16), np.ascontiguousarray(Bi.T).view(np.uint16), m, n, k,
+                                     b_layout=ko.ROW_MAJOR).view(np.float16)
+                np.testing.assert_array_equal(got.astype(np.float64), want, err_msg="%dx%dx%d, B row-major" % (m, n, k))
     finally:
         ko.set_tuning("gemm16.variant", 0)
 
@@ -1005,19 +1014,21 @@ def test_gemm16_wave_k_variants_are_exact_on_small_integers(ko, variant):
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("m,n,k,tile", [(100, 1024, 1024, 32032), (512, 768, 3072, 32064), (1000, 1024, 4096, 64064),
                                         (8, 4096, 4096, 32032), (200, 2304, 768, 32064), (750, 1000, 1032, 64064),
-                                        (2040, 700, 2056, 64128), (9000, 192, 2048, 128064)])
-def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, bf16):
-    """A few hundred rows against a weight matrix (column-major B): the dispatch sends them to the kernel that splits K
-    over the waves of a workgroup - the plan query says which tile - and the whole output agrees with the oracle,
-    plain and with bias + GELU; with that kernel switched off (gemm16.wave_k = 1) the older paths give the same
-    result to the same bound."""
-    assert ko.gemm_plan(m, n, k, sixteen_bit=True) == (1, 0, tile)
+                                        (2040, 704, 2056, 64128), (9000, 192, 2048, 128064)])
+@pytest.mark.parametrize("b_col_major", [True, False])
+def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, bf16, b_col_major):
+    """A few hundred rows against a weight matrix: the dispatch sends them to the kernel that splits K over the waves
+    of a workgroup - the plan query says which tile - and the whole output agrees with the oracle, plain and with
+    bias + GELU; with that kernel switched off (gemm16.wave_k = 1) the older paths give the same result to the same
+    bound."""
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout) == (1, 0, tile)
     A = _bits16((m, k), 101 + m, bf16)
-    B = _bits16((n, k), 103 + n, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 103 + n, bf16)
     bias = _bits16((n,), 105, bf16)
-    kw = dict(dtype=ko.BF16 if bf16 else ko.F16)
-    _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16)
-    _, ref64b, apb = oracle.gemm16(A, B, m, n, k, bf16=bf16, bias_bits=bias, act=1)
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16, b_layout=layout)
+    _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major)
+    _, ref64b, apb = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major, bias_bits=bias, act=1)
     try:
         for off in (0, 1):
             ko.set_tuning("gemm16.wave_k", off)
@@ -1027,4 +1038,3 @@ def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, b
             assert_gemm16_act_close(_to_f64(got, bf16), ref64b, apb + 2.0, k, bf16=bf16)
     finally:
         ko.set_tuning("gemm16.wave_k", 0)
-    assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=ko.ROW_MAJOR)[2] in (0, 128, 64, 32)

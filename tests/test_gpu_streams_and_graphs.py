@@ -53,7 +53,7 @@ def test_operators_replay_from_a_hip_graph(ko):
     a4, b4, d4 = ko.DeviceBuffer(m4 * k4 * 4), ko.DeviceBuffer(k4 * n4 * 4), ko.DeviceBuffer(m4 * n4 * 4)
     ko.fill_uniform_f32(a4, m4 * k4, 511)
     ko.fill_uniform_f32(b4, k4 * n4, 512)
-    m5, n5, k5 = 256, 384, 4096  # 16-bit, few tiles and a deep K, B as [K][N]: slices of K as well
+    m5, n5, k5 = 256, 384, 4096  # 16-bit, few tiles and a deep K: slices of K as well (with gemm16.wave_k = 1)
     a5, b5, d5 = ko.DeviceBuffer(m5 * k5 * 2), ko.DeviceBuffer(n5 * k5 * 2), ko.DeviceBuffer(m5 * n5 * 2)
     ko.fill_uniform_16(a5, m5 * k5, 513)
     ko.fill_uniform_16(b5, n5 * k5, 514)
@@ -78,7 +78,9 @@ def test_operators_replay_from_a_hip_graph(ko):
         ko.gemm16(m2, n2, k2, a2, b2, d2, stream=stream)
         ko.gemm16(m3, n3, k3, a3, b3, d3, stream=stream)
         ko.sgemm(m4, n4, k4, a4, b4, d4, stream=stream)
-        ko.gemm16(m5, n5, k5, a5, b5, d5, stream=stream, b_layout=ko.ROW_MAJOR)
+        ko.set_tuning("gemm16.wave_k", 1)
+        ko.gemm16(m5, n5, k5, a5, b5, d5, stream=stream)
+        ko.set_tuning("gemm16.wave_k", 0)
         ko.softmax(x6, s6, rows6, cols6, stream=stream)
         ko.layernorm(s6, l6, rows6, cols6, stream=stream)
 
@@ -177,12 +179,20 @@ def test_stream_destroy_releases_the_workspace(ko):
     """ko_stream_destroy frees the 32 MiB workspace a K-sliced call gave the stream: a process that creates and
     destroys more streams than the workspace table has entries (64) keeps the sliced path - same bits as on the
     first stream - and holds no more workspaces afterwards than before."""
+    ko.set_tuning("gemm16.wave_k", 1)  # (by default the 16-bit GEMM splits K over the waves of a workgroup here, in one launch)
+    try:
+        _stream_destroy_releases_the_workspace(ko)
+    finally:
+        ko.set_tuning("gemm16.wave_k", 0)
+
+
+def _stream_destroy_releases_the_workspace(ko):
     m, n, k = 256, 256, 2048
-    assert ko.gemm_plan(m, n, k)[0] > 1 and ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=ko.ROW_MAJOR)[0] > 1
+    assert ko.gemm_plan(m, n, k)[0] > 1 and ko.gemm_plan(m, n, k, sixteen_bit=True)[0] > 1
     A, B = inputs.uniform_f32((m, k), 41), inputs.uniform_f32((k, n), 42)
     dA, dB = ko.DeviceBuffer.from_numpy(A), ko.DeviceBuffer.from_numpy(B)
     A16 = inputs.uniform_f16((m, k), 43).view(np.uint16)
-    B16 = inputs.uniform_f16((k, n), 44).view(np.uint16)  # [K][N]: with a column-major B this shape takes no K slices
+    B16 = inputs.uniform_f16((n, k), 44).view(np.uint16)
     dA16, dB16 = ko.DeviceBuffer.from_numpy(A16), ko.DeviceBuffer.from_numpy(B16)
     ko.set_tuning("sgemm.k_slices", 1)
     try:
@@ -199,7 +209,7 @@ def test_stream_destroy_releases_the_workspace(ko):
         dD, dD16 = ko.DeviceBuffer(m * n * 4), ko.DeviceBuffer(m * n * 2)
         ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
         assert _workspaces(ko) == base + 1, i
-        ko.gemm16(m, n, k, dA16, dB16, dD16, stream=stream, b_layout=ko.ROW_MAJOR)
+        ko.gemm16(m, n, k, dA16, dB16, dD16, stream=stream)
         assert _workspaces(ko) == base + 1, i
         stream.close()  # waits for the work, then frees the workspace
         assert _workspaces(ko) == base, i
