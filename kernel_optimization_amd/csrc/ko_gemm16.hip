@@ -1789,15 +1789,17 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
 // 32 x 768 x 3072 11.4 -> 6.5 (7.1); with more tiles than compute units it loses (512 x 3072 x 768: 10.3 against 14.1).
 // Beyond that, 64 x 128 or 128 x 64 tiles over three waves (all the LDS stages that fit) from K = 2048 on: 512 x
 // 4096 x 4096 38.0 -> 31.7 (25.7), 2048 x 768 x 3072 27.6 -> 24.9 (18.1), 2048 x 1024 x 4096 37.4 -> 33.8 (25.0).
+// With B as [K][N] the small tiles gain as much (100 x 1024 x 1024 12.2 -> 4.4 us, 1000 x 1024 x 4096 30.4 -> 20.4;
+// hipBLASLt 5.7 and 17.3), the two large ones lose (2048 x 768 x 3072 25.6 -> 29.3) and are left out.
 // Returns 0, or 1000 * rows + columns of the tile: 32032, 32064, 64064, 64128, 128064.
-int wave_k_tile(int64_t m, int64_t n, int64_t k) {
+int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k > 8192) return 0;
     const int64_t cu = compute_units();
     const int64_t m32 = (m + 31) / 32, m64 = (m + 63) / 64, n32 = (n + 31) / 32, n64 = (n + 63) / 64;
     if (m32 * n32 <= cu) return k >= 128 ? 32032 : 0;
     if (m32 * n64 <= cu) return k >= 256 ? 32064 : 0;
     if (m64 * n64 <= cu) return k >= 1024 ? 64064 : 0;
-    if (k < 2048) return 0;
+    if (k < 2048 || b_row_major) return 0;
     if (m64 * ((n + 127) / 128) <= cu) return 64128;
     if (((m + 127) / 128) * n64 <= cu) return 128064;
     return 0;
@@ -1816,7 +1818,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
     }
     if (variant <= 0 && p.k_slice == 0 && (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0))) {
         // the whole problem, or a part cut off it, when it is small
-        switch (wave_k_tile(p.M, p.N, p.K)) {
+        switch (wave_k_tile(p.M, p.N, p.K, B_ROW_MAJOR)) {
             case 32032: return launch_wave_k<1, 1, 8, BF16, B_ROW_MAJOR>(p, stream);
             case 32064: return launch_wave_k<1, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
             case 64064: return launch_wave_k<2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
@@ -2055,7 +2057,7 @@ int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *sl
         (b_layout != KO_ROW_MAJOR && b_layout != KO_COL_MAJOR))
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16_plan: bad argument");
     if ((b_layout == KO_COL_MAJOR || n % 8 == 0) && k % 8 == 0) {  // (a row-major B: rows of whole 16-byte chunks)
-        if (const int wave_k = wave_k_tile(m, n, k); wave_k != 0) {
+        if (const int wave_k = wave_k_tile(m, n, k, b_layout == KO_ROW_MAJOR); wave_k != 0) {
             *slices = 1;
             *k_slice = 0;
             *tile = wave_k;

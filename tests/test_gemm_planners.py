@@ -57,6 +57,7 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
             assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and k % 8 == 0 and 128 <= k <= 8192
             assert -(-m // tm) * -(-n // tn) <= 256
             assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
+            assert b_layout == ko.COL_MAJOR or plan[2] in (32032, 32064, 64064)
 
 
 def test_measured_decisions_stay_put():

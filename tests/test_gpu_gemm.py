@@ -1022,6 +1022,8 @@ def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, b
     bias + GELU; with that kernel switched off (gemm16.wave_k = 1) the older paths give the same result to the same
     bound."""
     layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    if not b_col_major and tile in (64128, 128064):
+        pytest.skip("the two large tiles take a column-major B only")
     assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout) == (1, 0, tile)
     A = _bits16((m, k), 101 + m, bf16)
     B = _bits16((n, k) if b_col_major else (k, n), 103 + n, bf16)
