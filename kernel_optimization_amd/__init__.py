@@ -312,7 +312,8 @@ def sgemm(m, n, k, A, B, D, C=None, alpha=1.0, beta=0.0, stream=None):
 def gemm_plan(m, n, k, sixteen_bit=False, b_layout=COL_MAJOR):
     """(slices, k_slice, tiling) the host-side planner of the SGEMM or the 16-bit GEMM (with B in b_layout) decides
     for a shape; (1, 0, 1000 * rows + columns) is the 16-bit GEMM's one launch whose workgroups own one output tile of
-    that size (32 x 32 to 128 x 64) and split K over their waves."""
+    that size and split K over their waves (32 x 32 to 64 x 64) or walk it through a deep ring of LDS stages (64 x 128
+    to 128 x 128)."""
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     if sixteen_bit:
         check(harness().ko_debug_gemm16_plan(m, n, k, b_layout, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))

@@ -1582,6 +1582,233 @@ int launch_wave_k(Params p, hipStream_t stream) {
     return KO_OK;
 }
 
+// A deep ring of LDS stages for mid-size problems (a few thousand rows against a weight matrix: tens to a few
+// hundred tiles of 128 x 128).  What a compute unit takes in through direct-to-LDS loads is the bytes it has in flight
+// over a latency of 1 - 1.5 us, and the bytes in flight are LDS stages: two stages of a 256 x 256 tile (or of any
+// other) give a K tile that takes one latency whatever its size.  Here the tile is small enough (BM + BN rows of
+// 128 bytes per stage) for STAGES - 1 K tiles to be on their way while one is multiplied: the loads of K tile
+// t + STAGES - 1 go out right behind the barrier that publishes K tile t, into the stage that K tile t - 1 was read
+// from; a wave waits only for its own loads of K tile t (loads complete in order: all but the last (STAGES - 2) K
+// tiles' worth done) and one barrier per K tile publishes them.  The waves share the stages as in the kernels
+// above (WAVES_M x WAVES_N wave tiles of 32 TM x 32 TN, eight rows of 128 bytes per wave-level load, the same
+// swizzle, inline-assembly fragment reads two K steps deep); the stage is a compile-time number (the loop is
+// unrolled by STAGES and K is padded with K tiles of zeros up to a multiple of that - at most STAGES - 1 K tiles
+// of multiplying zeros).  One workgroup per tile and per compute unit; the epilogue is store_tile's, through the
+// stages once the last K tile has been read.  Any M and N (rows past the end are fetched from the last row, edge tiles take the
+// element-wise epilogue), K a multiple of 8 (chunks at or past K come from sixteen zero bytes); B column-major.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(const Params p) {
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    constexpr int KS = kBK / 16;
+    constexpr int A_BYTES = BM * kBK * 2, B_BYTES = BN * kBK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
+    constexpr int A_LOADS = BM / 8 / WAVES, B_LOADS = BN / 8 / WAVES, LOADS = A_LOADS + B_LOADS;  // per wave and K tile
+    constexpr int EPILOGUE_BYTES = WTM * WTN * 2;                                                 // per wave
+    static_assert(KS == 4 && WAVES % 2 == 0 && (BM / 8) % WAVES == 0 && (BN / 8) % WAVES == 0, "");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && STAGES >= 3 && (STAGES - 1) * LOADS <= 63, "");
+    static_assert(STAGES * STAGE_BYTES <= 160 * 1024 && WAVES * EPILOGUE_BYTES <= STAGES * STAGE_BYTES, "");
+    constexpr int OFFSET_SETS = ((STAGES - 1) * STAGE_BYTES) / 65536 + 1;  // fragment addresses 64 KB apart (see off_a)
+    static_assert(STAGE_BYTES + (TM > TN ? TM : TN) * 4096 <= 65536, "");
+
+    extern __shared__ u32x4 lds[];
+    char *const lds_bytes = reinterpret_cast<char *>(lds);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int tile = xcd_remap(static_cast<int>(blockIdx.x), p.nblocks);
+    const int m0 = (tile / p.tiles_n) * BM, n0 = (tile % p.tiles_n) * BN;
+    const int M = p.M, N = p.N, K = p.K;
+    const int64_t ldk = p.ldk;
+    const int KT = (K + kBK - 1) / kBK;
+    const int KT_padded = (KT + STAGES - 1) / STAGES * STAGES;
+
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    const char *const zeros = reinterpret_cast<const char *>(&zero_chunk16);
+
+    // wave w issues the wave-level loads w, w + WAVES, ... of a K tile (eight tile rows each); lane l fills slot
+    // l % 8 of row l / 8 with chunk (l % 8) ^ swz(row) - the same for all of a wave's loads, as 8 WAVES rows apart
+    // the swizzle repeats
+    const int row_in = lane >> 3;
+    const int lane_k = ((lane & 7) ^ swz<1>(8 * wave + row_in)) << 3;  // first k, within a K tile, of this lane's chunk
+    const char *src_a[A_LOADS], *src_b[B_LOADS];  // this lane's chunk of this wave's load i in the K tile to fetch next
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int r = m0 + 8 * (wave + WAVES * i) + row_in;
+        src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + lane_k);
+    }
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) {
+        const int r = n0 + 8 * (wave + WAVES * j) + row_in;
+        src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + lane_k);
+    }
+    int ld_k0 = 0;     // first k of the K tile to fetch next
+    bool ld_in = lane_k < K;  // this lane's chunk of that K tile lies inside K
+    // load number L (the A loads first, then the B loads) of the K tile to fetch next, into stage `stage`; the last
+    // one moves on to the next K tile
+    auto issue_one = [&](int stage, auto l_c) {
+        constexpr int L = decltype(l_c)::value;
+        char *dst = lds_bytes + stage * STAGE_BYTES + 1024 * wave;
+        if constexpr (L < A_LOADS) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(ld_in ? src_a[L] : zeros), (lptr_t)(dst + 1024 * WAVES * L), 16, 0, 0);
+            src_a[L] += kBK * 2;
+        } else {
+            constexpr int J = L - A_LOADS;
+            __builtin_amdgcn_global_load_lds((gptr_t)(ld_in ? src_b[J] : zeros), (lptr_t)(dst + A_BYTES + 1024 * WAVES * J), 16, 0, 0);
+            src_b[J] += kBK * 2;
+        }
+        if constexpr (L == LOADS - 1) {
+            ld_k0 += kBK;
+            ld_in = ld_k0 + lane_k < K;
+        }
+    };
+
+    // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps; further sets 64 KB up
+    // each, for the stages that the 16-bit offset field of the read does not reach from the first
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int sw = (frow >> 1) & 7;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_bytes));
+    uint32_t off_a[OFFSET_SETS][KS], off_b[OFFSET_SETS][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const uint32_t o = lds_base + static_cast<uint32_t>(frow * 128 + (((2 * ks + fhalf) ^ sw) << 4));
+#pragma unroll
+        for (int set = 0; set < OFFSET_SETS; ++set) {
+            off_a[set][ks] = o + wm * WTM * 128 + set * 65536;
+            off_b[set][ks] = o + A_BYTES + wn * WTN * 128 + set * 65536;
+        }
+    }
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    // the matrix instructions are inline assembly: pin the moves that zero their addends and keep the distance the
+    // compiler does not know it has to keep (see gemm16_pinned_kernel)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
+    asm volatile("s_nop 7");
+
+    constexpr int READS = TM + TN, MFMAS = TM * TN;
+    u32x4 af[2][TM], bf[2][TN];
+    // read number R (the A blocks first, then the B blocks) of K step KSTEP out of stage S into fragment set SLOT
+    auto read_one = [&](auto r_c, auto ks_c, auto slot_c, auto stage_c) {
+        constexpr int R = decltype(r_c)::value, KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value,
+                      S = decltype(stage_c)::value;
+        constexpr int HI = S * STAGE_BYTES / 65536, BASE = S * STAGE_BYTES - HI * 65536;
+        static_assert(BASE + ((TM > TN ? TM : TN) - 1) * 4096 < 65536, "");
+        if constexpr (R < TM) lds_read16<BASE + R * 4096>(af[SLOT][R], off_a[HI][KSTEP]);
+        else lds_read16<BASE + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[HI][KSTEP]);
+    };
+    // every read issued so far has landed; each register the reads wrote passes through an empty statement behind the
+    // wait, which keeps the matrix instructions that use it behind this point
+    auto wait_frags = [&](int slot) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(af[slot][i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bf[slot][j]));
+    };
+    // The matrix instructions of one K step out of fragment set SLOT; behind the IDX-th of them go its share of the
+    // step's fragment reads (reader(R), R = 0 .. READS - 1) and of the step's loads (loader(L), L = FIRST_LOAD ..
+    // FIRST_LOAD + STEP_LOADS - 1), so that a wave held at the issue of a read or a load has a matrix instruction running.
+    // (the reads go out behind the first matrix instructions of the step, two behind each, so that the rest of the
+    // step covers their latency; with one read behind each of four the last one's latency lay open: 0.31 us per K
+    // tile without any loads, against 0.21 us of matrix instructions)
+    constexpr int RPM = MFMAS >= 2 * READS ? 1 : 2;                  // reads behind one matrix instruction
+    constexpr int STEP_LOADS = (LOADS + 1) / 2, LPM = (STEP_LOADS + MFMAS - 1) / MFMAS;
+    auto mfma_step = [&](auto slot_c, auto reader, auto first_load_c, auto loader) {
+        constexpr int SLOT = decltype(slot_c)::value, FIRST_LOAD = decltype(first_load_c)::value;
+        static_for<MFMAS>([&](auto idx_c) {
+            constexpr int IDX = decltype(idx_c)::value;
+            mfma_asm<BF16>(acc[IDX / TN][IDX % TN], bf[SLOT][IDX % TN], af[SLOT][IDX / TN]);
+            static_for<RPM>([&](auto r_c) {
+                constexpr int R = IDX * RPM + decltype(r_c)::value;
+                if constexpr (R < READS) reader(std::integral_constant<int, R>{});
+            });
+            static_for<LPM>([&](auto l_c) {
+                constexpr int L = IDX * LPM + decltype(l_c)::value;
+                if constexpr (FIRST_LOAD >= 0 && L < STEP_LOADS && FIRST_LOAD + L < LOADS) loader(std::integral_constant<int, FIRST_LOAD + L>{});
+            });
+        });
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+    using NoLoads = std::integral_constant<int, -1>;
+    auto nothing = [](auto) {};
+    // One K tile, held in stage S, its K step 0 already in fragment set 0.  Per K step the matrix instructions run out
+    // of one fragment set while the next step's fragments are read into the other.  Between steps 1 and 2: this wave's
+    // loads of the next K tile have landed (loads complete in order; those of the STAGES - 3 K tiles behind it may
+    // still be on their way) - and behind the barrier every wave's have, and every wave has left the stage before S,
+    // which the loads of the K tile STAGES - 1 ahead, one behind each matrix instruction of steps 2 and 3, fill
+    // next.  Step 3 reads step 0 of the next K tile out of the next stage.
+    auto k_tile = [&](auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        using Next = std::integral_constant<int, (S + 1) % STAGES>;
+        constexpr int FREE = (S + STAGES - 1) % STAGES;
+        mfma_step(C0{}, [&](auto r) { read_one(r, C1{}, C1{}, stage_c); }, NoLoads{}, nothing);
+        wait_frags(1);
+        mfma_step(C1{}, [&](auto r) { read_one(r, C2{}, C0{}, stage_c); }, NoLoads{}, nothing);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 3) * LOADS) : "memory");
+        lds_barrier();
+        wait_frags(0);
+        mfma_step(C0{}, [&](auto r) { read_one(r, C3{}, C1{}, stage_c); }, C0{}, [&](auto l) { issue_one(FREE, l); });
+        wait_frags(1);
+        mfma_step(C1{}, [&](auto r) { read_one(r, C0{}, C0{}, Next{}); }, std::integral_constant<int, STEP_LOADS>{},
+                  [&](auto l) { issue_one(FREE, l); });
+        wait_frags(0);
+    };
+    // Prologue: K tiles 0 .. STAGES - 2 on their way into stages 0 .. STAGES - 2; K tile 0 landed and published; its
+    // K step 0 in fragment set 0.
+    static_for<STAGES - 1>([&](auto s_c) {
+        static_for<LOADS>([&](auto l_c) { issue_one(decltype(s_c)::value, l_c); });
+    });
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * LOADS) : "memory");
+    lds_barrier();
+    static_for<READS>([&](auto r) { read_one(r, C0{}, C0{}, C0{}); });
+    wait_frags(0);
+    for (int kt = 0; kt < KT_padded; kt += STAGES) static_for<STAGES>([&](auto s_c) { k_tile(s_c); });
+    // matrix-instruction results are read by vector-ALU instructions next: cover the issue-to-write latency
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // the loads still in flight (K tiles past the end: zeros) land, and every wave is done reading, before the
+    // stages are written over by the epilogue's transposes
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+
+    // whole tiles, and tiles that only reach past M, take the coalesced epilogue (rows at or past M are not stored)
+    u32x4 *region = reinterpret_cast<u32x4 *>(lds_bytes + wave * EPILOGUE_BYTES);
+    if (n0 + BN > N)
+        store_tile<WTM, WTN, 1, BF16, true>(p, acc, region, lane, m0 + wm * WTM, n0 + wn * WTN);
+    else if (m0 + BM <= M)
+        store_tile<WTM, WTN, 1, BF16, false>(p, acc, region, lane, m0 + wm * WTM, n0 + wn * WTN);
+    else
+        store_tile<WTM, WTN, 1, BF16, false, 1, false, true>(p, acc, region, lane, m0 + wm * WTM, n0 + wn * WTN);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16>
+int launch_ring(Params p, hipStream_t stream) {
+    constexpr size_t lds_bytes = static_cast<size_t>(STAGES) * (BM + BN) * kBK * 2;
+    if (p.K % 8 != 0 || p.k_slice != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a whole K that is a multiple of 8");
+    auto kernel = gemm16_ring_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, BF16>;
+    static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
+    if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK) return st;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * p.tiles_n;
+    if (tiles > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: too many tiles for the ring variant");
+    p.nblocks = static_cast<int>(tiles);
+    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, stream>>>(p);
+    KO_CHECK_LAUNCH();
+    return KO_OK;
+}
+
 template <class T, bool BF16>
 int launch_persistent(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
@@ -1787,11 +2014,10 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
 // 100 x 1024 x 1024 9.0 -> 5.7 (5.5), 256 x 768 x 3072 12.5 -> 8.1 (8.6), 512 x 1024 x 4096 17.7 -> 12.3 (13.6),
 // 100 x 4096 x 4096 19.5 -> 11.7 (14.4), 1000 x 1024 x 4096 24.4 -> 18.3 (18.0), 768 x 768 x 4096 19.8 -> 16.0 (16.2),
 // 32 x 768 x 3072 11.4 -> 6.5 (7.1); with more tiles than compute units it loses (512 x 3072 x 768: 10.3 against 14.1).
-// Beyond that, 64 x 128 or 128 x 64 tiles over three waves (all the LDS stages that fit) from K = 2048 on: 512 x
-// 4096 x 4096 38.0 -> 31.7 (25.7), 2048 x 768 x 3072 27.6 -> 24.9 (18.1), 2048 x 1024 x 4096 37.4 -> 33.8 (25.0).
-// With B as [K][N] the small tiles gain as much (100 x 1024 x 1024 12.2 -> 4.4 us, 1000 x 1024 x 4096 30.4 -> 20.4;
-// hipBLASLt 5.7 and 17.3), the two large ones lose (2048 x 768 x 3072 25.6 -> 29.3) and are left out.
-// Returns 0, or 1000 * rows + columns of the tile: 32032, 32064, 64064, 64128, 128064.
+// (64 x 128 and 128 x 64 tiles over three waves gained less - 512 x 4096 x 4096 38.0 -> 31.7, 2048 x 768 x 3072 27.6 ->
+// 24.9 - than the ring kernel below does on those problems, and are gone.)
+// With B as [K][N] the tiles gain as much (100 x 1024 x 1024 12.2 -> 4.4 us, 1000 x 1024 x 4096 30.4 -> 20.4; hipBLASLt
+// 5.7 and 17.3).  Returns 0, or 1000 * rows + columns of the tile: 32032, 32064, 64064.
 int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k > 8192) return 0;
     const int64_t cu = compute_units();
@@ -1799,9 +2025,25 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     if (m32 * n32 <= cu) return k >= 128 ? 32032 : 0;
     if (m32 * n64 <= cu) return k >= 256 ? 32064 : 0;
     if (m64 * n64 <= cu) return k >= 1024 ? 64064 : 0;
-    if (k < 2048 || b_row_major) return 0;
-    if (m64 * ((n + 127) / 128) <= cu) return 64128;
-    if (((m + 127) / 128) * n64 <= cu) return 128064;
+    return 0;
+}
+
+// Which problems go to the kernel with the deep ring of LDS stages (gemm16_ring_kernel; B column-major): those that
+// are at most one tile of 128 x 128 per compute unit - of 128 x 64 or 64 x 128 when that still holds with those (the
+// short side of the tile along the longer side of the output: fewer distinct panels of A and B per XCD) - and too
+// many small tiles for the kernel above.  Measured against the dispatch below (hipBLASLt), us: 4096 x 1024 x 4096
+// 59.5 -> 36.8 (36.8), 3000 x 1024 x 4096 51.3 -> 33.0 (30.1), 1000 x 4096 x 4096 62.9 -> 45.3 (37.7), 4096 x 768 x
+// 3072 37.1 -> 26.4 (25.0), 3000 x 768 x 3072 35.9 -> 25.3 (21.9), 4096 x 1024 x 1024 16.2 -> 13.2 (13.4); on the half
+// tiles 2048 x 768 x 3072 23.7 -> 17.7 (17.3), 2048 x 1024 x 4096 33.2 -> 25.9 (24.4), 512 x 4096 x 4096 31.4 -> 27.4
+// (24.5), 512 x 4096 x 1024 13.1 -> 10.4 (9.8); with more tiles than compute units the pinned kernel wins (6000 x 768
+// x 3072: 43.4 us against 48.6).  Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128.
+int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
+    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || b_row_major || k < 512) return 0;
+    const int64_t cu = compute_units();
+    const int64_t m64 = (m + 63) / 64, m128 = (m + 127) / 128, n64 = (n + 63) / 64, n128 = (n + 127) / 128;
+    if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above, or (a K beyond its range: 768 x 768 x 16384) K slices
+    if (n > m ? m128 * n64 <= cu : m64 * n128 <= cu) return n > m ? 128064 : 64128;
+    if (m128 * n128 <= cu) return 128128;
     return 0;
 }
 
@@ -1822,9 +2064,17 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             case 32032: return launch_wave_k<1, 1, 8, BF16, B_ROW_MAJOR>(p, stream);
             case 32064: return launch_wave_k<1, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
             case 64064: return launch_wave_k<2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
-            case 64128: return launch_wave_k<2, 4, 3, BF16, B_ROW_MAJOR>(p, stream);
-            case 128064: return launch_wave_k<4, 2, 3, BF16, B_ROW_MAJOR>(p, stream);
             default: break;
+        }
+    }
+    if constexpr (!B_ROW_MAJOR) {
+        if (variant <= 0 && p.k_slice == 0) {
+            switch (ring_tile(p.M, p.N, p.K, false)) {
+                case 64128: return launch_ring<64, 128, 2, 2, 6, BF16>(p, stream);
+                case 128064: return launch_ring<128, 64, 2, 2, 6, BF16>(p, stream);
+                case 128128: return launch_ring<128, 128, 2, 2, 4, BF16>(p, stream);
+                default: break;
+            }
         }
     }
     if (variant <= 0 && p.k_slice == 0) {
@@ -1985,18 +2235,26 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // M any multiple of 8
         case 61: return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 80:
+        case 81:
+        case 82:
+        case 83:
+            if constexpr (B_ROW_MAJOR) {
+                return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variants need column-major B");
+            } else {
+                if (variant == 80) return launch_ring<128, 128, 2, 2, 4, BF16>(p, stream);  // 4 stages of 32 KB
+                if (variant == 81) return launch_ring<128, 64, 2, 2, 6, BF16>(p, stream);   // 6 stages of 24 KB
+                if (variant == 82) return launch_ring<64, 128, 2, 2, 6, BF16>(p, stream);
+                return launch_ring<128, 128, 2, 4, 5, BF16>(p, stream);  // 8 waves of 64 x 32, 5 stages
+            }
         case 70:
         case 71:
         case 72:
         case 73:
-        case 74:
-        case 75:
             if (variant == 70) return launch_wave_k<2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);  // 64 x 64 tiles, K over 4 waves
             if (variant == 71) return launch_wave_k<1, 2, 4, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 64
             if (variant == 72) return launch_wave_k<1, 1, 8, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 32, K over 8 waves
-            if (variant == 73) return launch_wave_k<1, 2, 6, BF16, B_ROW_MAJOR>(p, stream);  // 32 x 64, K over 6 waves
-            if (variant == 74) return launch_wave_k<4, 2, 3, BF16, B_ROW_MAJOR>(p, stream);  // 128 x 64, K over 3 waves
-            return launch_wave_k<2, 4, 3, BF16, B_ROW_MAJOR>(p, stream);                     // 64 x 128, K over 3 waves
+            return launch_wave_k<1, 2, 6, BF16, B_ROW_MAJOR>(p, stream);                     // 32 x 64, K over 6 waves
         default: return fail(KO_ERR_INVALID_ARGUMENT, "gemm16: unknown variant %d", variant);
     }
 }
@@ -2057,10 +2315,12 @@ int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *sl
         (b_layout != KO_ROW_MAJOR && b_layout != KO_COL_MAJOR))
         return fail(KO_ERR_INVALID_ARGUMENT, "gemm16_plan: bad argument");
     if ((b_layout == KO_COL_MAJOR || n % 8 == 0) && k % 8 == 0) {  // (a row-major B: rows of whole 16-byte chunks)
-        if (const int wave_k = wave_k_tile(m, n, k, b_layout == KO_ROW_MAJOR); wave_k != 0) {
+        int one_launch = wave_k_tile(m, n, k, b_layout == KO_ROW_MAJOR);
+        if (one_launch == 0) one_launch = ring_tile(m, n, k, b_layout == KO_ROW_MAJOR);
+        if (one_launch != 0) {
             *slices = 1;
             *k_slice = 0;
-            *tile = wave_k;
+            *tile = one_launch;
             return KO_OK;
         }
     }

@@ -51,13 +51,16 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
         # one launch: whole, or K split over the waves of workgroups that own one small output tile each - B
         # column-major, or row-major with rows of whole 16-byte chunks; a multiple of 8 deep (as every K the operator
         # takes); at most one such tile per compute unit, and the smallest tile for which that holds
-        assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064)
+        assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064, 128128)
         if plan[2]:
             tm, tn = divmod(plan[2], 1000)
-            assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and k % 8 == 0 and 128 <= k <= 8192
-            assert -(-m // tm) * -(-n // tn) <= 256
-            assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
-            assert b_layout == ko.COL_MAJOR or plan[2] in (32032, 32064, 64064)
+            assert -(-m // tm) * -(-n // tn) <= 256 and k % 8 == 0
+            if plan[2] in (32032, 32064, 64064):   # K over the waves of a workgroup
+                assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and 128 <= k <= 8192
+                assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
+            else:                                   # a deep ring of LDS stages: when the small tiles are too many
+                assert b_layout == ko.COL_MAJOR and k >= 512
+                assert -(-m // 64) * -(-n // 64) > 256
 
 
 def test_measured_decisions_stay_put():
@@ -74,10 +77,13 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 32032)
     assert ko.gemm_plan(512, 1024, 4096, sixteen_bit=True) == (1, 0, 32064)
     assert ko.gemm_plan(1000, 1024, 4096, sixteen_bit=True) == (1, 0, 64064)
+    # too many small tiles for that, at most one tile of 128 x 128 (or half of one) per compute unit: the ring kernel
     assert ko.gemm_plan(2048, 768, 3072, sixteen_bit=True) == (1, 0, 64128)
-    assert ko.gemm_plan(9000, 192, 2048, sixteen_bit=True) == (1, 0, 128064)
+    assert ko.gemm_plan(512, 4096, 4096, sixteen_bit=True) == (1, 0, 128064)
+    assert ko.gemm_plan(4096, 1024, 4096, sixteen_bit=True) == (1, 0, 128128)
+    assert ko.gemm_plan(6000, 768, 3072, sixteen_bit=True) == (1, 0, 0)
     assert ko.gemm_plan(1000, 1024, 768, sixteen_bit=True) == (1, 0, 0)       # 64 x 64 tiles only from K = 1024 on
-    assert ko.gemm_plan(512, 3072, 768, sixteen_bit=True) == (1, 0, 0)        # more tiles than compute units
+    assert ko.gemm_plan(512, 3072, 768, sixteen_bit=True) == (1, 0, 128064)   # more 64 x 64 tiles than compute units
     assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 32032)
     assert ko.gemm_plan(100, 1028, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)  # rows of B off 16 bytes
     assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
