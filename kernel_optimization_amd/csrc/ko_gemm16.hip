@@ -1595,8 +1595,11 @@ int launch_wave_k(Params p, hipStream_t stream) {
 // unrolled by STAGES and K is padded with K tiles of zeros up to a multiple of that - at most STAGES - 1 K tiles
 // of multiplying zeros).  One workgroup per tile and per compute unit; the epilogue is store_tile's, through the
 // stages once the last K tile has been read.  Any M and N (rows past the end are fetched from the last row, edge tiles take the
-// element-wise epilogue), K a multiple of 8 (chunks at or past K come from sixteen zero bytes); B column-major.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16>
+// element-wise epilogue), K a multiple of 8 (chunks at or past K come from sixteen zero bytes).
+// B_ROW: B as [K][N] (rows ldb apart, N and ldb multiples of 8): the K tile of B is 64 rows of BN values and stays
+// row-major in LDS, a wave-level load covers four or eight of its rows with the 16-byte chunks permuted by the row
+// number modulo 4, and the fragments come out of pairs of transposing reads - as in gemm16_wave_k_kernel.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16, bool B_ROW = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(const Params p) {
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -1607,8 +1610,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
     static_assert(KS == 4 && WAVES % 2 == 0 && (BM / 8) % WAVES == 0 && (BN / 8) % WAVES == 0, "");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && STAGES >= 3 && (STAGES - 1) * LOADS <= 63, "");
     static_assert(STAGES * STAGE_BYTES <= 160 * 1024 && WAVES * EPILOGUE_BYTES <= STAGES * STAGE_BYTES, "");
-    constexpr int OFFSET_SETS = ((STAGES - 1) * STAGE_BYTES) / 65536 + 1;  // fragment addresses 64 KB apart (see off_a)
-    static_assert(STAGE_BYTES + (TM > TN ? TM : TN) * 4096 <= 65536, "");
+    constexpr int SET_BYTES = 32768;                                       // fragment address registers this far apart (see off_a)
+    constexpr int OFFSET_SETS = ((STAGES - 1) * STAGE_BYTES) / SET_BYTES + 1;
+    constexpr int NCH = BN / 8, RPL = 64 / NCH, B_ROW_BYTES = BN * 2;      // row-major B: chunks per LDS row, rows per wave-level load
+    static_assert(SET_BYTES + (TM > TN ? TM : TN) * 4096 <= 65536 && SET_BYTES + 52 * B_ROW_BYTES < 65536 && RPL % 4 == 0, "");
 
     extern __shared__ u32x4 lds[];
     char *const lds_bytes = reinterpret_cast<char *>(lds);
@@ -1638,11 +1643,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         const int r = m0 + 8 * (wave + WAVES * i) + row_in;
         src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + lane_k);
     }
+    // row-major B: lane l fills position l % NCH of row l / NCH of its load's RPL rows with chunk (l % NCH) ^ b_swz(row)
+    auto b_swz = [](int k) { return ((k & 3) << 2) & (NCH - 1); };
+    const int b_krow = lane / NCH;  // + RPL * (wave + WAVES * j): the row, within the K tile, this lane fetches in load j
+    bool b_inside = true;           // row-major B: this lane's chunk lies inside N (the same chunk in every load)
 #pragma unroll
     for (int j = 0; j < B_LOADS; ++j) {
-        const int r = n0 + 8 * (wave + WAVES * j) + row_in;
-        src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + lane_k);
+        if constexpr (B_ROW) {
+            const int c = n0 + 8 * ((lane % NCH) ^ b_swz(b_krow));
+            b_inside = c < N;
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(RPL * (wave + WAVES * j) + b_krow) * p.ldb + (b_inside ? c : 0));
+        } else {
+            const int r = n0 + 8 * (wave + WAVES * j) + row_in;
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + lane_k);
+        }
     }
+    const int64_t b_tile_step = B_ROW ? static_cast<int64_t>(kBK) * p.ldb * 2 : kBK * 2;  // bytes from a K tile to the next
     int ld_k0 = 0;     // first k of the K tile to fetch next
     bool ld_in = lane_k < K;  // this lane's chunk of that K tile lies inside K
     // load number L (the A loads first, then the B loads) of the K tile to fetch next, into stage `stage`; the last
@@ -1655,8 +1671,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
             src_a[L] += kBK * 2;
         } else {
             constexpr int J = L - A_LOADS;
-            __builtin_amdgcn_global_load_lds((gptr_t)(ld_in ? src_b[J] : zeros), (lptr_t)(dst + A_BYTES + 1024 * WAVES * J), 16, 0, 0);
-            src_b[J] += kBK * 2;
+            bool in = ld_in;
+            if constexpr (B_ROW) in = b_inside && ld_k0 + RPL * (wave + WAVES * J) + b_krow < K;
+            __builtin_amdgcn_global_load_lds((gptr_t)(in ? src_b[J] : zeros), (lptr_t)(dst + A_BYTES + 1024 * WAVES * J), 16, 0, 0);
+            src_b[J] += b_tile_step;
         }
         if constexpr (L == LOADS - 1) {
             ld_k0 += kBK;
@@ -1664,7 +1682,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         }
     };
 
-    // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps; further sets 64 KB up
+    // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps; further sets 32 KB up
     // each, for the stages that the 16-bit offset field of the read does not reach from the first
     const int frow = lane & 31, fhalf = lane >> 5;
     const int sw = (frow >> 1) & 7;
@@ -1675,8 +1693,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         const uint32_t o = lds_base + static_cast<uint32_t>(frow * 128 + (((2 * ks + fhalf) ^ sw) << 4));
 #pragma unroll
         for (int set = 0; set < OFFSET_SETS; ++set) {
-            off_a[set][ks] = o + wm * WTM * 128 + set * 65536;
-            off_b[set][ks] = o + A_BYTES + wn * WTN * 128 + set * 65536;
+            off_a[set][ks] = o + wm * WTM * 128 + set * SET_BYTES;
+            off_b[set][ks] = o + A_BYTES + wn * WTN * 128 + set * SET_BYTES;
+        }
+    }
+    // row-major B: where this lane's transposing reads of K step 0 start (lane i of a group of 16: row i / 4 of the
+    // step's rows, columns 4 (i % 4) .. + 3 of the group's 16), and the halves of a fragment as the reads deliver them
+    uint32_t off_br[OFFSET_SETS][B_ROW ? TN : 1];
+    u32x2 b_lo[2][B_ROW ? TN : 1], b_hi[2][B_ROW ? TN : 1];
+    if constexpr (B_ROW) {
+        const int i = lane & 15, g = (lane >> 4) & 1, kq = i >> 2;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int chunk = ((wn * WTN + j * 32 + g * 16 + 4 * (i & 3)) >> 3) ^ b_swz(kq);
+#pragma unroll
+            for (int set = 0; set < OFFSET_SETS; ++set)
+                off_br[set][j] = lds_base + A_BYTES + (fhalf * 8 + kq) * B_ROW_BYTES + chunk * 16 + (i & 1) * 8 + set * SET_BYTES;
         }
     }
 
@@ -1695,16 +1727,23 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
     asm volatile("s_nop 7");
 
-    constexpr int READS = TM + TN, MFMAS = TM * TN;
+    constexpr int READS = B_ROW ? TM + 2 * TN : TM + TN, MFMAS = TM * TN;
     u32x4 af[2][TM], bf[2][TN];
-    // read number R (the A blocks first, then the B blocks) of K step KSTEP out of stage S into fragment set SLOT
+    // read number R (the A blocks first, then the B blocks - row-major B: their halves) of K step KSTEP out of stage S
+    // into fragment set SLOT
     auto read_one = [&](auto r_c, auto ks_c, auto slot_c, auto stage_c) {
         constexpr int R = decltype(r_c)::value, KSTEP = decltype(ks_c)::value, SLOT = decltype(slot_c)::value,
                       S = decltype(stage_c)::value;
-        constexpr int HI = S * STAGE_BYTES / 65536, BASE = S * STAGE_BYTES - HI * 65536;
-        static_assert(BASE + ((TM > TN ? TM : TN) - 1) * 4096 < 65536, "");
-        if constexpr (R < TM) lds_read16<BASE + R * 4096>(af[SLOT][R], off_a[HI][KSTEP]);
-        else lds_read16<BASE + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[HI][KSTEP]);
+        constexpr int HI = S * STAGE_BYTES / SET_BYTES, BASE = S * STAGE_BYTES - HI * SET_BYTES;
+        if constexpr (R < TM) {
+            lds_read16<BASE + R * 4096>(af[SLOT][R], off_a[HI][KSTEP]);
+        } else if constexpr (!B_ROW) {
+            lds_read16<BASE + (R - TM) * 4096>(bf[SLOT][R - TM], off_b[HI][KSTEP]);
+        } else {
+            constexpr int J = (R - TM) / 2, IMM = BASE + KSTEP * 16 * B_ROW_BYTES;
+            if constexpr ((R - TM) % 2 == 0) lds_read_tr<IMM>(b_lo[SLOT][J], off_br[HI][J]);
+            else lds_read_tr<IMM + 4 * B_ROW_BYTES>(b_hi[SLOT][J], off_br[HI][J]);
+        }
     };
     // every read issued so far has landed; each register the reads wrote passes through an empty statement behind the
     // wait, which keeps the matrix instructions that use it behind this point
@@ -1712,8 +1751,21 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(af[slot][i]));
+        if constexpr (B_ROW) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bf[slot][j]));
+            for (int j = 0; j < TN; ++j) {
+                asm volatile("" : "+v"(b_lo[slot][j]), "+v"(b_hi[slot][j]));
+                bf[slot][j] = u32x4{b_lo[slot][j][0], b_lo[slot][j][1], b_hi[slot][j][0], b_hi[slot][j][1]};
+            }
+            // where the halves did not land in adjacent registers the line above is vector-ALU moves, and the matrix
+            // instructions that read bf are inline assembly the compiler keeps no distance to
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bf[slot][j]));
+            asm volatile("s_nop 3");
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bf[slot][j]));
+        }
     };
     // The matrix instructions of one K step out of fragment set SLOT; behind the IDX-th of them go its share of the
     // step's fragment reads (reader(R), R = 0 .. READS - 1) and of the step's loads (loader(L), L = FIRST_LOAD ..
@@ -1721,7 +1773,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
     // (the reads go out behind the first matrix instructions of the step, two behind each, so that the rest of the
     // step covers their latency; with one read behind each of four the last one's latency lay open: 0.31 us per K
     // tile without any loads, against 0.21 us of matrix instructions)
-    constexpr int RPM = MFMAS >= 2 * READS ? 1 : 2;                  // reads behind one matrix instruction
+    constexpr int RPM = MFMAS >= 2 * READS ? 1 : (READS > 2 * MFMAS ? (READS + MFMAS - 1) / MFMAS : 2);  // reads behind one matrix instruction
+    static_assert(RPM * MFMAS >= READS, "");
     constexpr int STEP_LOADS = (LOADS + 1) / 2, LPM = (STEP_LOADS + MFMAS - 1) / MFMAS;
     auto mfma_step = [&](auto slot_c, auto reader, auto first_load_c, auto loader) {
         constexpr int SLOT = decltype(slot_c)::value, FIRST_LOAD = decltype(first_load_c)::value;
@@ -1793,11 +1846,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
         store_tile<WTM, WTN, 1, BF16, false, 1, false, true>(p, acc, region, lane, m0 + wm * WTM, n0 + wn * WTN);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16, bool B_ROW = false>
 int launch_ring(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = static_cast<size_t>(STAGES) * (BM + BN) * kBK * 2;
     if (p.K % 8 != 0 || p.k_slice != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a whole K that is a multiple of 8");
-    auto kernel = gemm16_ring_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, BF16>;
+    if (B_ROW && (p.N % 8 != 0 || p.ldb % 8 != 0))
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a row-major B whose N and row stride are multiples of 8");
+    auto kernel = gemm16_ring_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, BF16, B_ROW>;
     static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK) return st;
     p.tiles_n = (p.N + BN - 1) / BN;
@@ -2036,13 +2091,21 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
 // 3072 37.1 -> 26.4 (25.0), 3000 x 768 x 3072 35.9 -> 25.3 (21.9), 4096 x 1024 x 1024 16.2 -> 13.2 (13.4); on the half
 // tiles 2048 x 768 x 3072 23.7 -> 17.7 (17.3), 2048 x 1024 x 4096 33.2 -> 25.9 (24.4), 512 x 4096 x 4096 31.4 -> 27.4
 // (24.5), 512 x 4096 x 1024 13.1 -> 10.4 (9.8); with more tiles than compute units the pinned kernel wins (6000 x 768
-// x 3072: 43.4 us against 48.6).  Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128.
+// x 3072: 43.4 us against 48.6).  With B as [K][N] (hipBLASLt on that layout in brackets): 3000 x 768 x 3072 45.2 -> 24.2
+// (26.0), 4096 x 1024 x 4096 56.2 -> 40.3 (40.8), 1000 x 4096 x 4096 74.2 -> 43.4 (40.4), 3000 x 1024 x 1024 21.7 -> 11.5
+// (12.8), 512 x 4096 x 1024 16.1 -> 11.2 (11.4); the half tile there is 128 x 64 whatever the shape (64 x 128 - rows of
+// 256 bytes in the stage of B - is the slower one: 2048 x 768 x 3072 22.7 against 20.6).
+// Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128.
 int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
-    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || b_row_major || k < 512) return 0;
+    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k < 512) return 0;
     const int64_t cu = compute_units();
     const int64_t m64 = (m + 63) / 64, m128 = (m + 127) / 128, n64 = (n + 63) / 64, n128 = (n + 127) / 128;
     if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above, or (a K beyond its range: 768 x 768 x 16384) K slices
-    if (n > m ? m128 * n64 <= cu : m64 * n128 <= cu) return n > m ? 128064 : 64128;
+    if (b_row_major) {
+        if (m128 * n64 <= cu) return 128064;
+    } else if (n > m ? m128 * n64 <= cu : m64 * n128 <= cu) {
+        return n > m ? 128064 : 64128;
+    }
     if (m128 * n128 <= cu) return 128128;
     return 0;
 }
@@ -2067,14 +2130,12 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             default: break;
         }
     }
-    if constexpr (!B_ROW_MAJOR) {
-        if (variant <= 0 && p.k_slice == 0) {
-            switch (ring_tile(p.M, p.N, p.K, false)) {
-                case 64128: return launch_ring<64, 128, 2, 2, 6, BF16>(p, stream);
-                case 128064: return launch_ring<128, 64, 2, 2, 6, BF16>(p, stream);
-                case 128128: return launch_ring<128, 128, 2, 2, 4, BF16>(p, stream);
-                default: break;
-            }
+    if (variant <= 0 && p.k_slice == 0 && (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0))) {
+        switch (ring_tile(p.M, p.N, p.K, B_ROW_MAJOR)) {
+            case 64128: return launch_ring<64, 128, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
+            case 128064: return launch_ring<128, 64, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
+            case 128128: return launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
+            default: break;
         }
     }
     if (variant <= 0 && p.k_slice == 0) {
@@ -2239,14 +2300,10 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 81:
         case 82:
         case 83:
-            if constexpr (B_ROW_MAJOR) {
-                return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variants need column-major B");
-            } else {
-                if (variant == 80) return launch_ring<128, 128, 2, 2, 4, BF16>(p, stream);  // 4 stages of 32 KB
-                if (variant == 81) return launch_ring<128, 64, 2, 2, 6, BF16>(p, stream);   // 6 stages of 24 KB
-                if (variant == 82) return launch_ring<64, 128, 2, 2, 6, BF16>(p, stream);
-                return launch_ring<128, 128, 2, 4, 5, BF16>(p, stream);  // 8 waves of 64 x 32, 5 stages
-            }
+            if (variant == 80) return launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);  // 4 stages of 32 KB
+            if (variant == 81) return launch_ring<128, 64, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);   // 6 stages of 24 KB
+            if (variant == 82) return launch_ring<64, 128, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
+            return launch_ring<128, 128, 2, 4, 5, BF16, B_ROW_MAJOR>(p, stream);  // 8 waves of 64 x 32, 5 stages
         case 70:
         case 71:
         case 72:

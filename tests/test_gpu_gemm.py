@@ -1022,8 +1022,8 @@ def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, b
     tile - and the whole output agrees with the oracle, plain and with bias + GELU; with those kernels switched off
     (gemm16.wave_k = 1) the older paths give the same result to the same bound."""
     layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
-    if not b_col_major and tile in (64128, 128064, 128128):
-        pytest.skip("the ring kernel takes a column-major B only")
+    if not b_col_major and tile == 64128:
+        tile = 128064  # with B as [K][N] the half tile is 128 x 64 whatever the shape
     assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout) == (1, 0, tile)
     A = _bits16((m, k), 101 + m, bf16)
     B = _bits16((n, k) if b_col_major else (k, n), 103 + n, bf16)
@@ -1049,25 +1049,29 @@ RING_VARIANTS = [80, 81, 82, 83]
 
 @pytest.mark.parametrize("variant", RING_VARIANTS)
 @pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
 @pytest.mark.parametrize("m,n,k", [(1, 1, 8), (33, 36, 8), (128, 128, 64), (300, 520, 72), (256, 384, 1032), (130, 75, 4104),
-                                   (640, 256, 448), (257, 129, 264), (1000, 256, 328), (96, 1000, 200)])
-def test_gemm16_ring_variants_match_oracle(ko, variant, bf16, m, n, k):
+                                   (640, 256, 448), (257, 129, 264), (1000, 256, 328), (96, 1000, 200), (70, 8, 264)])
+def test_gemm16_ring_variants_match_oracle(ko, variant, bf16, b_col_major, m, n, k):
     """The waves of a workgroup walk K together through four to six LDS stages, loads three to five K tiles ahead:
     against the oracle, plain and with the whole epilogue, bit-stable from call to call - fewer K tiles than stages,
     a number of K tiles that is no multiple of the stages, a K that ends inside a K tile, ragged M (the coalesced
-    epilogue with the rows past M left out) and ragged N (the element-wise one)."""
+    epilogue with the rows past M left out) and ragged N (the element-wise one).  B as [N][K], or as [K][N] when N
+    is a multiple of 8."""
+    if not b_col_major and n % 8:
+        pytest.skip("a row-major B off 16-byte rows does not go to these kernels")
     A = _bits16((m, k), 111 + m, bf16)
-    B = _bits16((n, k), 113 + n, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 113 + n, bf16)
     C = _bits16((m, n), 115, bf16)
     bias = _bits16((n,), 117, bf16)
-    kw = dict(dtype=ko.BF16 if bf16 else ko.F16)
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
     ko.set_tuning("gemm16.variant", variant)
     try:
-        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major)
         got = ko.gemm16_host(A, B, m, n, k, **kw)
         assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
         np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, **kw), got)
-        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, C_bits=C, beta=0.5, bias_bits=bias, act=2)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major, C_bits=C, beta=0.5, bias_bits=bias, act=2)
         got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
         assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap + 2.0, k, bf16=bf16)
     finally:
@@ -1095,5 +1099,9 @@ def test_gemm16_ring_variants_are_exact_on_small_integers(ko, variant):
             np.testing.assert_array_equal(out[:m * n].view(np.float16).astype(np.float64).reshape(m, n), want,
                                           err_msg="%dx%dx%d" % (m, n, k))
             assert (out[m * n:] == 0x7bff).all(), "%dx%dx%d: the guard area behind D was written" % (m, n, k)
+            if n % 8 == 0:  # the same product with B handed over as [K][N]
+                got = ko.gemm16_host(Ai.view(np.uint16), np.ascontiguousarray(Bi.T).view(np.uint16), m, n, k,
+                                     b_layout=ko.ROW_MAJOR).view(np.float16)
+                np.testing.assert_array_equal(got.astype(np.float64), want, err_msg="%dx%dx%d, B row-major" % (m, n, k))
     finally:
         ko.set_tuning("gemm16.variant", 0)
