@@ -834,7 +834,7 @@ def main():
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
     ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"],
                     help="one of %s, copy_f32, hbm_ceilings, short_kernels, gemm16_midsize, gemm16_active_cus, softmax_f32_786432x512_unmasked, or a long-row line by name: "
-                         "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache)" % ", ".join(sorted(WORKLOADS)))
+                         "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache); or one 16-bit GEMM shape: gemm_f16_<m>x<n>x<k>" % ", ".join(sorted(WORKLOADS)))
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
     ap.add_argument("--no-all", dest="all", action="store_false")
@@ -864,6 +864,13 @@ def main():
         return
     if args.workload == "softmax_f32_786432x512_unmasked":  # for the traffic counters and traces
         res, _ = bench_softmax(5, args.steps, args.warmup, unmasked=True)
+        print(json.dumps(res))
+        return
+    gemm_line = re.fullmatch(r"gemm_f16_(\d+)x(\d+)x(\d+)", args.workload)
+    if gemm_line and args.workload not in WORKLOADS:  # one 16-bit GEMM shape alone (B column-major), for traces
+        m, n, k = (int(g) for g in gemm_line.groups())
+        res, _ = bench_gemm16(4, min(args.steps, 30), max(args.warmup, 100), vendor, shape=(m, n, k), c_loop=True)
+        res["plan"] = ko.gemm_plan(m, n, k, sixteen_bit=True)
         print(json.dumps(res))
         return
     row_line = re.fullmatch(r"(softmax|layernorm)_f32_(\d+)x(\d+)_(auto|warp|block|nocache)", args.workload)
