@@ -1613,7 +1613,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
     constexpr int SET_BYTES = 32768;                                       // fragment address registers this far apart (see off_a)
     constexpr int OFFSET_SETS = ((STAGES - 1) * STAGE_BYTES) / SET_BYTES + 1;
     constexpr int NCH = BN / 8, RPL = 64 / NCH, B_ROW_BYTES = BN * 2;      // row-major B: chunks per LDS row, rows per wave-level load
-    static_assert(SET_BYTES + (TM > TN ? TM : TN) * 4096 <= 65536 && SET_BYTES + 52 * B_ROW_BYTES < 65536 && RPL % 4 == 0, "");
+    static_assert(SET_BYTES + (TM > TN ? TM : TN) * 4096 <= 65536 && (!B_ROW || (SET_BYTES + 52 * B_ROW_BYTES < 65536 && RPL % 4 == 0)), "");
 
     extern __shared__ u32x4 lds[];
     char *const lds_bytes = reinterpret_cast<char *>(lds);
@@ -2091,7 +2091,9 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
 // 3072 37.1 -> 26.4 (25.0), 3000 x 768 x 3072 35.9 -> 25.3 (21.9), 4096 x 1024 x 1024 16.2 -> 13.2 (13.4); on the half
 // tiles 2048 x 768 x 3072 23.7 -> 17.7 (17.3), 2048 x 1024 x 4096 33.2 -> 25.9 (24.4), 512 x 4096 x 4096 31.4 -> 27.4
 // (24.5), 512 x 4096 x 1024 13.1 -> 10.4 (9.8); with more tiles than compute units the pinned kernel wins (6000 x 768
-// x 3072: 43.4 us against 48.6).  With B as [K][N] (hipBLASLt on that layout in brackets): 3000 x 768 x 3072 45.2 -> 24.2
+// x 3072: 43.4 us against 48.6; 256 x 128 and 128 x 256 tiles of this kernel, three stages of 48 KB, four waves of
+// 128 x 64, came out level with the pinned kernel there - 46.4, 8192 x 1024 x 4096 76 - 80 against 80 - and are not kept).
+// With B as [K][N] (hipBLASLt on that layout in brackets): 3000 x 768 x 3072 45.2 -> 24.2
 // (26.0), 4096 x 1024 x 4096 56.2 -> 40.3 (40.8), 1000 x 4096 x 4096 74.2 -> 43.4 (40.4), 3000 x 1024 x 1024 21.7 -> 11.5
 // (12.8), 512 x 4096 x 1024 16.1 -> 11.2 (11.4); the half tile there is 128 x 64 whatever the shape (64 x 128 - rows of
 // 256 bytes in the stage of B - is the slower one: 2048 x 768 x 3072 22.7 against 20.6).
