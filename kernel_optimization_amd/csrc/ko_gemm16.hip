@@ -1599,8 +1599,11 @@ int launch_wave_k(Params p, hipStream_t stream) {
 // B_ROW: B as [K][N] (rows ldb apart, N and ldb multiples of 8): the K tile of B is 64 rows of BN values and stays
 // row-major in LDS, a wave-level load covers four or eight of its rows with the 16-byte chunks permuted by the row
 // number modulo 4, and the fragments come out of pairs of transposing reads - as in gemm16_wave_k_kernel.
+// K slices: workgroups with blockIdx.y = s take k in [s * k_slice, (s + 1) * k_slice) and leave their fp32 partial
+// products in the workspace (see slice_of, store_partial).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16, bool B_ROW = false>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(const Params p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(const Params whole) {
+    const Params p = slice_of<B_ROW>(whole);
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr int KS = kBK / 16;
@@ -1836,6 +1839,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
 
+    if (p.partial != nullptr) {
+        store_partial<WTM, WTN>(p, acc, lane, m0 + wm * WTM, n0 + wn * WTN);
+        return;
+    }
     // whole tiles, and tiles that only reach past M, take the coalesced epilogue (rows at or past M are not stored)
     u32x4 *region = reinterpret_cast<u32x4 *>(lds_bytes + wave * EPILOGUE_BYTES);
     if (n0 + BN > N)
@@ -1849,9 +1856,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm16_ring_kernel(con
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool BF16, bool B_ROW = false>
 int launch_ring(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = static_cast<size_t>(STAGES) * (BM + BN) * kBK * 2;
-    if (p.K % 8 != 0 || p.k_slice != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a whole K that is a multiple of 8");
+    if (p.K % 8 != 0 || p.k_slice % 8 != 0) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a K (and K slices) that are multiples of 8");
     if (B_ROW && (p.N % 8 != 0 || p.ldb % 8 != 0))
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: the ring variant takes a row-major B whose N and row stride are multiples of 8");
+    const int slices = p.k_slice > 0 ? (p.K + p.k_slice - 1) / p.k_slice : 1;
     auto kernel = gemm16_ring_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, BF16, B_ROW>;
     static std::atomic<uint64_t> configured{0};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured); st != KO_OK) return st;
@@ -1859,7 +1867,7 @@ int launch_ring(Params p, hipStream_t stream) {
     const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * p.tiles_n;
     if (tiles > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: too many tiles for the ring variant");
     p.nblocks = static_cast<int>(tiles);
-    kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, stream>>>(p);
+    kernel<<<dim3(static_cast<unsigned>(p.nblocks), static_cast<unsigned>(slices)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;
 }
@@ -2036,8 +2044,12 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     // 9.1; at K = 1024 the second launch costs what the slices gain)
     if (p.K < (4 * t128 <= cu ? 1536 : 2048)) return plan;
     if (4 * t128 <= cu) {
+        // (128 x 128 tiles when their slices come to three quarters of the compute units or more - they run the ring
+        // kernel, one workgroup per compute unit: 1024 x 512 x 32768 two slices of 64 x 64 tiles 123 us, eight of
+        // 128 x 128 57 (hipBLASLt 50); 512 x 512 x 32768 64 -> 39 (32), 512 x 1024 x 16384 52 -> 36 (27), 256 x 1024 x 16384
+        // 30 -> 23 (19); 256 x 256 x 16384, four such tiles, stays on 16 slices of 64 x 64: 14.7 us)
         const int64_t s128 = capped(cu / t128, 512), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
-        if (s64 >= 2 && s64 * t64 >= s128 * t128) set(s64, 64);
+        if (s64 >= 2 && s64 * t64 >= s128 * t128 && 4 * s128 * t128 < 3 * cu) set(s64, 64);
         else set(s128, 128);
     } else if (t128 <= cu) {
         set(capped(2 * cu / t128, 2048), 128);
@@ -2050,7 +2062,15 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
     Params part = p;
     part.k_slice = plan.k_slice;
     part.partial = workspace;
-    int st = plan.tile == 128  ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream)
+    // 128 x 128 tiles: the ring kernel while the slices are at most one workgroup per compute unit (it is one
+    // workgroup per compute unit; the register pipeline runs two): 1024 x 768 x 16384 in 5 slices 51.7 -> 45.8 us,
+    // 1024 x 1024 x 16384 62.3 -> 55.1, 2048 x 512 x 32768 119 -> 98; with more it loses (1024 x 2304 x 16384, 432 workgroups:
+    // 119 us against 144)
+    const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
+    const bool ring = plan.tile == 128 && tuning(knob_gemm16_wave_k) != 1 && t128 * plan.slices <= compute_units() &&
+                      (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0));
+    int st = ring              ? launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(part, stream)
+             : plan.tile == 128 ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream)
              : plan.tile == 32 ? launch<TileSkinny, BF16, B_ROW_MAJOR>(part, stream)
                                : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
     if (st != KO_OK) return st;
@@ -2099,10 +2119,12 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
 // 256 bytes in the stage of B - is the slower one: 2048 x 768 x 3072 22.7 against 20.6).
 // Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128.
 int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
-    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k < 512) return 0;
+    // (a K beyond 8192 is left to the K slices below, which run this kernel's 128 x 128 tiles: 512 x 2304 x 16384 whole on
+    // 144 tiles of 128 x 64 103 us, in slices 67)
+    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k < 512 || k > 8192) return 0;
     const int64_t cu = compute_units();
     const int64_t m64 = (m + 63) / 64, m128 = (m + 127) / 128, n64 = (n + 63) / 64, n128 = (n + 127) / 128;
-    if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above, or (a K beyond its range: 768 x 768 x 16384) K slices
+    if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above
     if (b_row_major) {
         if (m128 * n64 <= cu) return 128064;
     } else if (n > m ? m128 * n64 <= cu : m64 * n128 <= cu) {
