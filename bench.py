@@ -756,7 +756,7 @@ def _compact(res):
     return out
 
 
-def headline_line(head, cpu, parity, others, copy, info, steps, warmup):
+def headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize=None):
     """The record: one JSON object of at most MAX_LINE_BYTES characters, printed as the last line of stdout.  It
     carries the headline workload in full (roofline, CPU baseline, parity) and six numbers for each of the other
     configurations; everything else goes to gpurun_out/bench_workloads.json and to earlier lines."""
@@ -787,9 +787,12 @@ def headline_line(head, cpu, parity, others, copy, info, steps, warmup):
             line[key] = _sig(head[key])
     by_name = {r["workload"]: r for r in others}
     line["configs"] = [_compact(by_name[n]) for n in CONFIG_LINES if n in by_name]
+    if midsize is not None:  # the 16-bit GEMM on 77 mid-size shapes next to hipBLASLt (rows in the details file)
+        line["gemm16_midsize"] = {"shapes": midsize["shapes"], "median_vs_hipblaslt": _sig(midsize["median_vs_hipblaslt"]),
+                                  "min_vs_hipblaslt": _sig(midsize["min_vs_hipblaslt"])}
     line["details_file"] = "gpurun_out/bench_workloads.json"
     # never let the record outgrow what a reader of the last line keeps: shed the optional parts first
-    for key in ("details_file", "copy_ceiling_frac", "copy_same_bytes_us", "max_abs_diff_vs_hipblaslt"):
+    for key in ("details_file", "copy_ceiling_frac", "copy_same_bytes_us", "max_abs_diff_vs_hipblaslt", "gemm16_midsize"):
         if len(json.dumps(line)) <= MAX_LINE_BYTES:
             break
         line.pop(key, None)
@@ -800,11 +803,13 @@ def headline_line(head, cpu, parity, others, copy, info, steps, warmup):
 
 
 
-def emit_record(head, cpu, parity, others, copy, ceilings, info, steps, warmup, out_dir=None):
+def emit_record(head, cpu, parity, others, copy, ceilings, info, steps, warmup, out_dir=None, midsize=None):
     """Writes everything that was measured to <out_dir>/bench_workloads.json, prints one short line per secondary
     workload, and prints the record as the LAST line of stdout."""
-    line = headline_line(head, cpu, parity, others, copy, info, steps, warmup)
+    line = headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize)
     details = dict(line)
+    if midsize is not None:
+        details["gemm16_midsize"] = midsize
     details["copy_ceiling"] = None if copy is None else {
         "GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"], "workload": copy["workload"],
         "independent_sources": ceilings}
@@ -900,6 +905,7 @@ def main():
     others = []
     copy = None
     ceilings = None
+    midsize = None
     if args.all:
         copy = bench_copy(args.steps, args.warmup)
         ceilings = bench_ceilings(min(args.steps, 10), 3)
@@ -979,8 +985,13 @@ def main():
             res["steps"], res["warmup"] = args.steps, warm
             others.append(res)
 
+        # token counts from 100 to 20000 against transformer weight shapes, next to hipBLASLt (launch loops in C on both
+        # sides; about ten seconds): the summary goes into the record, the rows into the details file
+        if vendor is not None:
+            midsize = bench_gemm16_midsize(min(args.steps, 30), 100, vendor)
+
         head, cpu, parity = headline()
-    emit_record(head, cpu, parity, others, copy, ceilings, info, args.steps, args.warmup)
+    emit_record(head, cpu, parity, others, copy, ceilings, info, args.steps, args.warmup, midsize=midsize)
 
 
 if __name__ == "__main__":

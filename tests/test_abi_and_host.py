@@ -243,8 +243,10 @@ def test_bench_record_is_one_short_last_line(tmp_path, capsys):
     others += [_canned_result("layernorm_f32_%dx%d_block" % (1024 << i, 131072 >> i)) for i in range(40)]
     info = dict(name="AMD Instinct MI355X", arch="gfx950:sramecc+:xnack-", compute_units=256)
     copy = _canned_result("copy_f32_1024MiB")
+    midsize = dict(shapes=77, median_vs_hipblaslt=0.89973, min_vs_hipblaslt=0.65537, max_vs_hipblaslt=1.18,
+                   rows=[dict(m=100, n=1024, k=1024, us=4.4)] * 77)
     line = bench.emit_record(head, cpu, parity, others, copy, {"rows": list(range(1000))}, info, 20, 5,
-                             out_dir=str(tmp_path))
+                             out_dir=str(tmp_path), midsize=midsize)
     out = capsys.readouterr().out.rstrip("\n").split("\n")
     assert len(out) == len(others) + 1
     last = out[-1]
@@ -254,6 +256,8 @@ def test_bench_record_is_one_short_last_line(tmp_path, capsys):
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "parity", "configs"):
         assert key in rec, key
+    assert rec["gemm16_midsize"] == dict(shapes=77, median_vs_hipblaslt=0.8997, min_vs_hipblaslt=0.6554)
+    assert len(json.load(open(tmp_path / "bench_workloads.json"))["gemm16_midsize"]["rows"]) == 77
     assert rec["config"]["workload"] == "masked_softmax_f32_786432x512" and "model" not in rec["config"]
     assert set(rec["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"}
     assert rec["roofline"]["frac"] <= 1.0
