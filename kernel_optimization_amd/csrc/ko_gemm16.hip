@@ -897,9 +897,9 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
 // EDGE_K: K is any multiple of 8 and is padded with zeros up to the next multiple of 128 - a lane whose
 // 16-byte chunk (or, for a row-major B, whose row) lies at or past K fetches 16 zero bytes instead, chosen per
 // load with a compare and two selects, so nothing is read past the end of a row or of the matrix.
-// EDGE_M: M is any multiple of 8; the last row of tiles may reach past it.  A wave-level load covers eight rows of A,
-// so a load whose rows lie at or past M is pointed - a wave-uniform choice, made once per output tile - at the last
-// eight rows of A instead: valid addresses, whose products land in rows of the tile that the epilogue does not store.
+// EDGE_M: any M; the last row of tiles may reach past it.  A lane whose row of A lies at or past M fetches row
+// M - 1 instead - its byte offset from the cursor, one 32-bit register per load, is recomputed once per output tile -
+// a valid address, whose products land in rows of the tile that the epilogue does not store.
 template <class T, bool BF16, bool B_ROW, bool EDGE_K = false, bool EDGE_M = false>
 __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
@@ -966,17 +966,17 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     int ld_kt = 0, ld_t = 0;
     const char *cur_a, *cur_b;
     const int64_t group_stride = static_cast<int64_t>(8 * WAVES) * K * 2;  // bytes between a wave's consecutive loads
-    int64_t a_off[A_LOADS];  // load i of A: bytes from the cursor to its eight rows (wave-uniform)
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = i * group_stride;
+    // EDGE_M: load i of A, this lane: bytes from the cursor (row m0 + 8 * wave, the K tile's first k) to its chunk;
+    // fits 32 bits (at most 256 rows either way, K below 2^22: the launcher checks)
+    int32_t a_lane_off[EDGE_M ? A_LOADS : 1];
     auto set_cursor = [&]() {
         int m0, n0;
         tile_origin(ld_t, m0, n0);
         if constexpr (EDGE_M) {
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
-                const int first = m0 + 8 * (wave + WAVES * i);  // first of the load's eight rows
-                a_off[i] = static_cast<int64_t>((first < p.M ? first : p.M - 8) - (m0 + 8 * wave)) * K * 2;
+                const int row = m0 + 8 * (wave + WAVES * i) + row_in;
+                a_lane_off[i] = (((row < p.M ? row : p.M - 1) - (m0 + 8 * wave)) * K + lane_k) * 2;
             }
         }
         cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
@@ -1001,7 +1001,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // EDGE_K: where load I of the cursor's K tile reads from - its place in A or B, or the zero chunk when the
     // lane's k lies at or past K (for a row-major B the k is the row the load fetches)
     auto source_a = [&](int i) {
-        const char *at = cur_a + a_off[i] + lane_off;
+        const char *at = EDGE_M ? cur_a + a_lane_off[EDGE_M ? i : 0] : cur_a + i * group_stride + lane_off;
         if constexpr (EDGE_K) at = ld_kt * kBK + lane_k < K ? at : zeros;
         return at;
     };
@@ -1262,11 +1262,11 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     }
 }
 
-// EDGE_M: M may be any multiple of 8 from 8 on (the last row of tiles then reaches past M, see the kernel).
+// EDGE_M: any M (the last row of tiles then reaches past M, see the kernel); K below 2^22.
 template <class T, bool BF16, bool B_ROW = false, bool EDGE_M = false>
 int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
-    if ((p.M % (EDGE_M ? 8 : T::BM)) != 0 || p.M < 8 || (p.N % T::BN) != 0 || (p.K % 8) != 0)
+    if ((!EDGE_M && p.M % T::BM != 0) || p.M < 1 || (EDGE_M && p.K >= (1 << 22)) || (p.N % T::BN) != 0 || (p.K % 8) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 8 == 0");
     const bool edge_k = p.K % (2 * kBK) != 0;  // padded with zeros up to a pair of K tiles inside the kernel
     auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true, EDGE_M> : gemm16_pinned_kernel<T, BF16, B_ROW, false, EDGE_M>;
@@ -2198,12 +2198,13 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         // x 256 81 / 71 (58); 4880 x 7768 x 256 52 / 60 (41), x 512 82 / 82; 1351 x 18488 x 256 41 / 45, x 512 65 / 60;
         // 8148 x 1800 x 512 30 / 37 (27); 3000 x 5000 x 256 22 / 29 (22), x 512 34 / 38 (28); 4071 x 2328 x 768
         // (160 big tiles) 32 / 41 (24), 12521 x 989 x 768 40 / 52 (30), 3000 x 5000 x 768 (240) 46 / 48.
-        // A row count that is a multiple of 8 but not of the tile height, on whole tile columns: the pinned kernel
+        // A row count that is not a multiple of the tile height (any: 4093 x 3072 x 768 40.3 -> 26.6 us, at 4096 rows
+        // 25.5), on whole tile columns: the pinned kernel
         // takes it as it is (its last row of tiles fetches rows it has, and stores what lies inside the matrix),
         // so such a shape is neither cut nor taken off that kernel.  3000 x 3072 x 768: 30.0 -> 22.1 us (hipBLASLt
         // 19.5), 12000 x 768 x 3072 84 -> 73, 3000 x 4096 x 4096 112 -> 93, 16000 x 3072 x 768 82 -> 76; on
         // 128 x 256 tiles 6000 x 1024 x 1024 25.5 -> 18.0 (17.8), 6000 x 768 x 3072 55 -> 44.
-        const bool m_edge = p.M % 256 != 0 && p.M % 8 == 0 && p.M >= 8 && p.N % 256 == 0 && p.K >= 2 * kBK;
+        const bool m_edge = p.M % 256 != 0 && p.N % 256 == 0 && p.K >= 2 * kBK && p.K < (1 << 22);
         {
             const int64_t cu = compute_units();
             const bool ragged = p.M % 256 != 0 || p.N % 256 != 0;
@@ -2318,7 +2319,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
         case 53: return launch_direct<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);
         case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
-        case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // M any multiple of 8
+        case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // any M
         case 61: return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         case 80:
         case 81:

@@ -900,10 +900,11 @@ def test_sgemm_forced_slices_keep_a_kernel_that_takes_them(ko):
 @pytest.mark.parametrize("variant", [60, 61])
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("b_col_major", [True, False])
-@pytest.mark.parametrize("m,n,k", [(8, 256, 128), (136, 512, 256), (264, 256, 200), (1000, 768, 384), (3000, 512, 1032)])
-def test_gemm16_pinned_kernel_takes_any_multiple_of_8_rows(ko, variant, bf16, b_col_major, m, n, k):
-    """The pinned kernel with a last row of tiles that reaches past M (M a multiple of 8): its loads of rows at or past M
-    fetch the last eight rows of A instead and its epilogue leaves those rows of the tile alone.  Against the oracle,
+@pytest.mark.parametrize("m,n,k", [(8, 256, 128), (136, 512, 256), (264, 256, 200), (1000, 768, 384), (3000, 512, 1032),
+                                   (1, 256, 128), (257, 256, 136), (1001, 512, 392), (2047, 256, 1024)])
+def test_gemm16_pinned_kernel_takes_any_row_count(ko, variant, bf16, b_col_major, m, n, k):
+    """The pinned kernel with a last row of tiles that reaches past M (any M): its loads of rows at or past M
+    fetch row M - 1 instead and its epilogue leaves those rows of the tile alone.  Against the oracle,
     on 256 x 256 and 128 x 256 tiles, both layouts of B, K that is and is not whole K tiles, with C and beta, and with a
     guard area behind D that must come back untouched."""
     dt = ko.BF16 if bf16 else ko.F16
@@ -933,9 +934,10 @@ def test_gemm16_pinned_kernel_takes_any_multiple_of_8_rows(ko, variant, bf16, b_
         ko.set_tuning("gemm16.variant", 0)
 
 
-@pytest.mark.parametrize("m,n,k", [(3000, 3072, 768), (6000, 1024, 1024), (1240, 2304, 3072), (16000, 3072, 768)])
+@pytest.mark.parametrize("m,n,k", [(3000, 3072, 768), (6000, 1024, 1024), (1240, 2304, 3072), (16000, 3072, 768),
+                                   (4093, 3072, 768), (8191, 1024, 1024), (5001, 2304, 776)])
 def test_gemm16_ragged_rows_through_the_default_dispatch_are_exact(ko, m, n, k):
-    """Row counts that are multiples of 8 but not of the tile height, on the shapes the dispatch sends to the pinned
+    """Row counts that are not multiples of the tile height (of 8 or not), on the shapes the dispatch sends to the pinned
     kernel as they are (256 x 256 tiles, and 128 x 256 tiles): small integers make every sum exact, so any row fetched
     from the wrong place or stored where it does not belong shows."""
     rng = np.random.default_rng(m + k)
