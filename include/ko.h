@@ -172,8 +172,8 @@ int ko_layernorm_16(const void *in, void *out, float *mean, float *rstd, const v
  * Workspace: a problem with a deep K whose output tiles do not fill the chip (tiles for at most half of the
  * compute units and k >= 768, or rounds of tiles that leave many compute units idle and k >= 2048; any n)
  * is cut into slices of K that run side by side; their partial products go
- * through 32 MiB of device memory that the library allocates at the first such call on a (device, stream)
- * pair and keeps until ko_stream_destroy releases it (the default stream's: until the process ends).  Calls on
+ * through the first 32 MiB of a 64 MiB block of device memory that the library allocates at the first such call
+ * on a (device, stream) pair and keeps until ko_stream_destroy releases it (the default stream's: until the process ends).  Calls on
  * different streams therefore never share it.  A first such call made while the stream is being captured into a
  * graph allocates nothing and takes the unsliced kernels; so does every call while 64 live pairs hold a
  * workspace.  Results do not depend on the timing of the slices (summed in slice order), but the sliced and the
@@ -215,8 +215,9 @@ int ko_sgemm_f32_static_scratch(int64_t m, int64_t n, int64_t k, float alpha, co
  * boundaries then) it runs at about 0.6 of the rate.
  * Workspace: like ko_sgemm_f32, a deep K (k >= 2048; k >= 1536 on very few tiles; any n) on few output tiles -
  * of the whole problem or of the parts a ragged shape is cut into - is cut into slices of K whose fp32
- * partial products go through the 32 MiB workspace of the (device, stream) pair, allocated at the first such
- * call on the stream; a first such call inside a graph capture allocates nothing and runs unsliced. */
+ * partial products go through the 64 MiB workspace of the (device, stream) pair, allocated at the first such
+ * call on the stream; a first such call inside a graph capture allocates nothing and runs unsliced.  Beyond k = 8192
+ * that also holds for outputs of up to half a chip's worth of 256 x 256 tiles (n a multiple of 256). */
 int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A, const void *B,
                       int b_layout, float beta, const void *C, void *D, int in_dtype,
                       ko_stream_t stream);

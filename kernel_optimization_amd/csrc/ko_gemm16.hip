@@ -134,6 +134,7 @@ struct Params {
     int k_slice;                // 0: no slices
     float *partial;
     int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
+    int tiles;                  // gemm16_pinned_kernel with K slices: output tiles (nblocks = tiles * slices)
     int xcd_cols_log2;          // blocked tile order: the 8 XCDs' regions lie 2^this side by side (0: one below the other)
     int region_cols;            //                     columns of tiles in a region (unused when they lie one below the other)
 };
@@ -900,7 +901,12 @@ __device__ __forceinline__ void mfma_asm(float16v &acc, const u32x4 &a, const u3
 // EDGE_M: any M; the last row of tiles may reach past it.  A lane whose row of A lies at or past M fetches row
 // M - 1 instead - its byte offset from the cursor, one 32-bit register per load, is recomputed once per output tile -
 // a valid address, whose products land in rows of the tile that the epilogue does not store.
-template <class T, bool BF16, bool B_ROW, bool EDGE_K = false, bool EDGE_M = false>
+// SLICED: K slices.  The workgroups walk p.nblocks = p.tiles * slices pairs (slice, output tile) - tile_of's grid of
+// tiles with the slices' tile grids below each other; pair
+// (s, tile) multiplies k in [s * p.k_slice, (s + 1) * p.k_slice) - p.k_slice a multiple of 128, the last slice
+// padded with zeros when K ends inside it (EDGE_K) - and stores its accumulators as fp32 into partial product s
+// (see Params::partial) instead of the epilogue; p.K stays the whole K, the distance between rows.
+template <class T, bool BF16, bool B_ROW, bool EDGE_K = false, bool EDGE_M = false, bool SLICED = false>
 __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params p) {
     constexpr int BM = T::BM, BN = T::BN, WAVES_M = T::WAVES_M, WAVES_N = T::WAVES_N;
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -927,7 +933,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets address math run on the scalar unit
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int K = p.K;
-    const int KT = EDGE_K ? 2 * ((K + 2 * kBK - 1) / (2 * kBK)) : K / kBK;
+    const int KT = SLICED ? p.k_slice / kBK : EDGE_K ? 2 * ((K + 2 * kBK - 1) / (2 * kBK)) : K / kBK;
     const int grid = gridDim.x;
     const int my_tiles = (p.nblocks - static_cast<int>(blockIdx.x) + grid - 1) / grid;
     const int total = my_tiles * KT;
@@ -952,9 +958,17 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     typedef const __attribute__((address_space(1))) void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
 
-    auto tile_origin = [&](int t, int &m0, int &n0) {
+    auto tile_origin = [&](int t, int &m0, int &n0, int &slice) {
         int tile_m, tile_n;
         tile_of(p, static_cast<int>(blockIdx.x), grid, t, tile_m, tile_n);
+        if constexpr (SLICED) {
+            // the pairs are laid out as a grid of tiles with the slices below each other: row = slice * tiles_m + tile_m
+            const int tiles_m = p.tiles / p.tiles_n;
+            slice = tile_m / tiles_m;
+            tile_m -= slice * tiles_m;
+        } else {
+            slice = 0;
+        }
         m0 = tile_m * BM;
         n0 = tile_n * BN;
     };
@@ -969,9 +983,12 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // EDGE_M: load i of A, this lane: bytes from the cursor (row m0 + 8 * wave, the K tile's first k) to its chunk;
     // fits 32 bits (at most 256 rows either way, K below 2^22: the launcher checks)
     int32_t a_lane_off[EDGE_M ? A_LOADS : 1];
+    int k_end = K;  // EDGE_K: the K tiles of the cursor's output tile count from k = K - k_end
     auto set_cursor = [&]() {
-        int m0, n0;
-        tile_origin(ld_t, m0, n0);
+        int m0, n0, slice;
+        tile_origin(ld_t, m0, n0, slice);
+        const int k0 = SLICED ? slice * p.k_slice : 0;
+        if constexpr (SLICED) k_end = K - k0;
         if constexpr (EDGE_M) {
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
@@ -979,9 +996,9 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
                 a_lane_off[i] = (((row < p.M ? row : p.M - 1) - (m0 + 8 * wave)) * K + lane_k) * 2;
             }
         }
-        cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K);
-        if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(2 * wave) * p.ldb + n0);
-        else cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K);
+        cur_a = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(m0 + 8 * wave) * K + k0);
+        if constexpr (B_ROW) cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(k0 + 2 * wave) * p.ldb + n0);
+        else cur_b = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(n0 + 8 * wave) * K + k0);
     };
     set_cursor();
     const int64_t group_stride_b = B_ROW ? static_cast<int64_t>(2 * WAVES) * p.ldb * 2 : group_stride;
@@ -1002,14 +1019,14 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
     // lane's k lies at or past K (for a row-major B the k is the row the load fetches)
     auto source_a = [&](int i) {
         const char *at = EDGE_M ? cur_a + a_lane_off[EDGE_M ? i : 0] : cur_a + i * group_stride + lane_off;
-        if constexpr (EDGE_K) at = ld_kt * kBK + lane_k < K ? at : zeros;
+        if constexpr (EDGE_K) at = ld_kt * kBK + lane_k < k_end ? at : zeros;
         return at;
     };
     auto source_b = [&](int j) {
         const char *at = cur_b + j * group_stride_b + lane_off_b;
         if constexpr (EDGE_K) {
             const int k = B_ROW ? 2 * (wave + WAVES * j) + (lane >> 5) : lane_k;
-            at = ld_kt * kBK + k < K ? at : zeros;
+            at = ld_kt * kBK + k < k_end ? at : zeros;
         }
         return at;
     };
@@ -1214,11 +1231,21 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
         }
         wait_frags(0);
         if constexpr (last_of_tile) {
-            int m0, n0;
-            tile_origin(t, m0, n0);
+            int m0, n0, slice;
+            tile_origin(t, m0, n0, slice);
             // MFMA results are read by vector ALU instructions next: cover the issue-to-write latency
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-            if constexpr (SPARE) {
+            if constexpr (SLICED) {
+                static_assert(!SLICED || SPARE, "");
+                // the loads in flight (the next pair's first K tiles) are confirmed before the first store, as in
+                // the epilogue below
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                Params mine = p;
+                mine.partial = p.partial + static_cast<int64_t>(slice) * p.M * partial_ld(p.N);
+                store_partial<WTM, WTN>(mine, acc, lane, m0 + wm * WTM, n0 + wn * WTN);
+                clear_acc();
+                stores_in_flight = true;
+            } else if constexpr (SPARE) {
                 constexpr int REGION = WTM * WTN * 2 / 4;  // bytes per wave and pass
                 char *region = lds_bytes + 2 * (A_BYTES + B_BYTES) + wave * REGION;
                 store_tile<WTM, WTN, 1, BF16, false, 4, true, EDGE_M>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
@@ -1263,19 +1290,26 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
 }
 
 // EDGE_M: any M (the last row of tiles then reaches past M, see the kernel); K below 2^22.
-template <class T, bool BF16, bool B_ROW = false, bool EDGE_M = false>
+// SLICED: p.k_slice (a multiple of 128) and p.partial are set: the fp32 partial products of the K slices, no epilogue.
+template <class T, bool BF16, bool B_ROW = false, bool EDGE_M = false, bool SLICED = false>
 int launch_pinned(Params p, hipStream_t stream) {
     constexpr size_t lds_bytes = T::SPARE_EPILOGUE ? 160u * 1024u : 2u * (T::BM + T::BN) * kBK * sizeof(uint16_t);
     if ((!EDGE_M && p.M % T::BM != 0) || p.M < 1 || (EDGE_M && p.K >= (1 << 22)) || (p.N % T::BN) != 0 || (p.K % 8) != 0)
         return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: this persistent variant needs full tiles and K %% 8 == 0");
-    const bool edge_k = p.K % (2 * kBK) != 0;  // padded with zeros up to a pair of K tiles inside the kernel
-    auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true, EDGE_M> : gemm16_pinned_kernel<T, BF16, B_ROW, false, EDGE_M>;
+    if (SLICED && (p.k_slice < 2 * kBK || p.k_slice % (2 * kBK) != 0 || p.partial == nullptr))
+        return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: K slices of this variant are multiples of 128 deep");
+    const int slices = SLICED ? (p.K + p.k_slice - 1) / p.k_slice : 1;
+    // padded with zeros inside the kernel: up to a pair of K tiles, or to the end of the last slice
+    const bool edge_k = SLICED ? p.K % p.k_slice != 0 : p.K % (2 * kBK) != 0;
+    auto kernel = edge_k ? gemm16_pinned_kernel<T, BF16, B_ROW, true, EDGE_M, SLICED>
+                         : gemm16_pinned_kernel<T, BF16, B_ROW, false, EDGE_M, SLICED>;
     static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per instantiation: the devices whose LDS limit is raised
     if (const int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_bytes, configured[edge_k]); st != KO_OK)
         return st;
     p.tiles_n = p.N / T::BN;
     const int tiles_m = (p.M + T::BM - 1) / T::BM;
-    p.nblocks = tiles_m * p.tiles_n;
+    p.tiles = tiles_m * p.tiles_n;
+    p.nblocks = p.tiles * slices;
     int grid = compute_units() / 8 * 8;
     if (grid > p.nblocks) grid = p.nblocks;
     // Blocked tile order when the tile grid divides evenly over 8 XCDs x (grid / 8) workgroups: of the ways to lay
@@ -1287,14 +1321,19 @@ int launch_pinned(Params p, hipStream_t stream) {
     p.xcd_cols_log2 = 0;
     p.region_cols = 0;
     const int per_xcd = grid / 8;
+    // (K slices: the grid of tiles is the slices' grids below each other; a band lies inside a slice or is whole
+    // slices, and the resident block then holds a panel of B per slice and column)
+    const int rows = tiles_m * slices;
     if (tuning(knob_gemm16_mapping) != 1 && grid % 8 == 0) {
         int64_t best = 0;
         for (int lg = 0; lg <= 3; ++lg) {
             const int across = 1 << lg, down = 8 >> lg;
-            if (tiles_m % down != 0 || p.tiles_n % across != 0) continue;
-            const int band = tiles_m / down, region = p.tiles_n / across;
+            if (rows % down != 0 || p.tiles_n % across != 0) continue;
+            const int band = rows / down, region = p.tiles_n / across;
             if (band > per_xcd || per_xcd % band != 0 || region % (per_xcd / band) != 0) continue;
-            const int64_t bytes = static_cast<int64_t>(band) * T::BM + static_cast<int64_t>(per_xcd / band) * T::BN;
+            if (tiles_m % band != 0 && band % tiles_m != 0) continue;
+            const int band_slices = (band + tiles_m - 1) / tiles_m;
+            const int64_t bytes = static_cast<int64_t>(band) * T::BM + static_cast<int64_t>(per_xcd / band) * band_slices * T::BN;
             if (p.band_rows == 0 || bytes < best) {
                 best = bytes;
                 p.band_rows = band;
@@ -2014,7 +2053,8 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     const double out_bytes = 4.0 * p.M * partial_ld(p.N);  // of one partial product
     auto set = [&](int64_t slices, int tile) {
         if (slices < 2) return;
-        const int64_t depth = ((p.K + slices - 1) / slices + kBK - 1) / kBK * kBK;
+        const int64_t unit = tile == 256 ? 2 * kBK : kBK;  // the pinned kernel takes K tiles in pairs
+        const int64_t depth = ((p.K + slices - 1) / slices + unit - 1) / unit * unit;
         slices = (p.K + depth - 1) / depth;
         if (slices < 2 || slices > 65535 || slices * out_bytes > static_cast<double>(workspace_bytes)) return;
         plan.slices = static_cast<int>(slices);
@@ -2023,8 +2063,10 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     };
     const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
     const int64_t t64 = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64);
+    const bool pinned_ok = p.N % 256 == 0 && p.K % 8 == 0 && p.K < (1 << 22);  // the pinned kernel's 256 x 256 tiles
     if (forced >= 2) {
-        set(forced, p.M <= 32 && p.N >= 256 ? 32 : t128 * forced >= cu / 2 ? 128 : 64);
+        if (tuning(knob_gemm16_variant) == 62 && pinned_ok) set(forced, 256);
+        else set(forced, p.M <= 32 && p.N >= 256 ? 32 : t128 * forced >= cu / 2 ? 128 : 64);
         return plan;
     }
     const int64_t fit = static_cast<int64_t>(static_cast<double>(workspace_bytes) / out_bytes);  // slices the workspace holds
@@ -2043,13 +2085,27 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
     // (few tiles: from K = 1536 on - 128 x 128 x 1536 9.9 us whole, 8.7 in three slices; 100 x 100 x 1536 13.2 and
     // 9.1; at K = 1024 the second launch costs what the slices gain)
     if (p.K < (4 * t128 <= cu ? 1536 : 2048)) return plan;
+    // More than a quarter of the compute units' worth of 128 x 128 tiles, at most half of them of 256 x 256, and a K
+    // beyond what the ring kernel takes whole: the pinned kernel's 256 x 256 tiles in as many slices, at least 2048
+    // deep, as give every compute unit at most one (us, hipBLASLt in brackets: 2048 x 4096 x 16384 314 -> 260 (239),
+    // 1536 x 4096 x 16392 384 -> 272 (224), 1024 x 3072 x 16384 168 -> 124 (97), 768 x 3072 x 16384 127 -> 102 (79) - in
+    // four slices 116, in two 199; at K = 8192 the ring kernel's 80 us for 1024 x 4096 become 90)
+    const int64_t t256 = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
+    if (pinned_ok && tuning(knob_gemm16_wave_k) != 1 && 4 * t128 > cu && 2 * t256 <= cu && p.K > 8192) {
+        set(capped(cu / t256, 2048), 256);
+        if (plan.slices > 1) return plan;
+    }
     if (4 * t128 <= cu) {
         // (128 x 128 tiles when their slices come to three quarters of the compute units or more - they run the ring
         // kernel, one workgroup per compute unit: 1024 x 512 x 32768 two slices of 64 x 64 tiles 123 us, eight of
         // 128 x 128 57 (hipBLASLt 50); 512 x 512 x 32768 64 -> 39 (32), 512 x 1024 x 16384 52 -> 36 (27), 256 x 1024 x 16384
         // 30 -> 23 (19); 256 x 256 x 16384, four such tiles, stays on 16 slices of 64 x 64: 14.7 us)
-        const int64_t s128 = capped(cu / t128, 512), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
-        if (s64 >= 2 && s64 * t64 >= s128 * t128 && 4 * s128 * t128 < 3 * cu) set(s64, 64);
+        // (a K beyond what the ring kernel takes whole: slices at least 2048 deep, 3072 from half a million outputs on - the
+        // partial products cost what more workgroups gain: 768 x 768 x 16384 7 slices 39.3 us, 5 37.6; 512 x 1024 x 16384
+        // 8 33.4, 5 31.6; 256 x 1024 x 16384 16 27.3, 8 22.9; 512 x 768 x 12288 10 27.7, 6 23.4)
+        const int64_t min128 = p.K <= 8192 ? 512 : static_cast<int64_t>(p.M) * p.N >= 512 * 1024 ? 3072 : 2048;
+        const int64_t s128 = capped(cu / t128, min128), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
+        if (s64 >= 2 && s64 * t64 >= s128 * t128 && (p.K <= 8192 ? 4 * s128 * t128 < 3 * cu : 2 * s128 * t128 < cu)) set(s64, 64);
         else set(s128, 128);
     } else if (t128 <= cu) {
         set(capped(2 * cu / t128, 2048), 128);
@@ -2069,7 +2125,8 @@ int run_sliced16(const Params &p, const SlicePlan16 &plan, float *workspace, hip
     const int64_t t128 = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
     const bool ring = plan.tile == 128 && tuning(knob_gemm16_wave_k) != 1 && t128 * plan.slices <= compute_units() &&
                       (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0));
-    int st = ring              ? launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(part, stream)
+    int st = plan.tile == 256 ? launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true, true>(part, stream)
+             : ring            ? launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(part, stream)
              : plan.tile == 128 ? launch<TileSmall, BF16, B_ROW_MAJOR>(part, stream)
              : plan.tile == 32 ? launch<TileSkinny, BF16, B_ROW_MAJOR>(part, stream)
                                : launch<TileTiny, BF16, B_ROW_MAJOR>(part, stream);
@@ -2162,11 +2219,11 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             default: break;
         }
     }
-    if (variant <= 0 && p.k_slice == 0) {
+    if ((variant <= 0 || variant == 62) && p.k_slice == 0) {
         // the whole problem, or a part cut off it (the launches of one call follow each other on the stream and may
         // use its workspace one after the other): few tiles and a deep K go out as K slices
         const int64_t big = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + 255) / 256);
-        if (2 * big < compute_units() || p.M <= 32) {
+        if (2 * big <= compute_units() || p.M <= 32 || variant == 62) {
             if (const SlicePlan16 plan = plan_k_slices16(p, kStreamWorkspaceBytes); plan.slices > 1) {
                 void *workspace = nullptr;
                 if (const int st = stream_workspace(stream, &workspace); st != KO_OK) return st;
@@ -2321,6 +2378,8 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 54: return launch_direct<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
         case 60: return launch_pinned<TileBigSpread, BF16, B_ROW_MAJOR, true>(p, stream);  // any M
         case 61: return launch_pinned<TileHalf, BF16, B_ROW_MAJOR, true>(p, stream);
+        case 62:  // the pinned kernel in gemm16.k_slices K slices: reached only when the plan above came out whole
+            return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: variant 62 needs gemm16.k_slices >= 2, N %% 256 == 0 and a workspace");
         case 80:
         case 81:
         case 82:
@@ -2414,7 +2473,8 @@ int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *sl
     p.ldk = p.K;
     const int64_t big = ((m + 255) / 256) * ((n + 255) / 256);
     SlicePlan16 plan;
-    if (2 * big < compute_units() || m <= 32) plan = plan_k_slices16(p, kStreamWorkspaceBytes);  // as launch_variant asks
+    if (2 * big <= compute_units() || m <= 32 || tuning(knob_gemm16_variant) == 62)
+        plan = plan_k_slices16(p, kStreamWorkspaceBytes);  // as launch_variant asks
     *slices = plan.slices;
     *k_slice = plan.k_slice;
     *tile = plan.slices > 1 ? plan.tile : 0;

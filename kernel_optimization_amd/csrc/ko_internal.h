@@ -74,7 +74,10 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
 // stream use it in stream order.  `*workspace` stays null, with KO_OK, where nothing may be allocated (the
 // stream is being captured into a graph and has no workspace yet, 64 live pairs already hold one, the stream is
 // hipStreamPerThread, or the allocation fails): the caller then takes its path without a workspace.
-constexpr size_t kStreamWorkspaceBytes = size_t{32} << 20;
+constexpr size_t kStreamWorkspaceBytes = size_t{64} << 20;
+// What the SGEMM's K slices use of it at most: the size of the static array that stands in for the workspace in the
+// entry point that allocates nothing, so that both entry points plan, and sum, the same slices.
+constexpr size_t kSgemmPartialBytes = size_t{32} << 20;
 int stream_workspace(hipStream_t stream, void **workspace);
 // Frees the workspace of (current device, stream), if it has one.  The caller has synchronised the stream.
 int release_stream_workspace(hipStream_t stream);

@@ -32,10 +32,10 @@
 #include <utility>
 
 // Partial products of the entry point that allocates nothing (ko_sgemm_f32_static_scratch): as large as the
-// workspace the allocating entry point gives a stream.  Every device the library runs on holds its own copy
+// part of a stream's workspace that the allocating entry point uses.  Every device the library runs on holds its own copy
 // until the process ends.  In host code the name is a stand-in, not a device address: host code uses the
 // address that ko::static_scratch() asks the runtime for, once per device.
-static __device__ __align__(256) unsigned char scratch[ko::kStreamWorkspaceBytes];
+static __device__ __align__(256) unsigned char scratch[ko::kSgemmPartialBytes];
 
 namespace ko {
 namespace {
@@ -978,7 +978,7 @@ int sgemm(int64_t m, int64_t n, int64_t k, float alpha, const float *A, const fl
                                 "sgemm: the partial products of %d slices of K (%llu bytes) do not fit the static scratch array (%zu bytes)",
                                 slices, (unsigned long long)need, sizeof(scratch));
                 if (const int st = static_scratch(&workspace); st != KO_OK) return st;
-            } else if (need <= kStreamWorkspaceBytes) {
+            } else if (need <= kSgemmPartialBytes) {
                 if (const int st = stream_workspace(s, &workspace); st != KO_OK) return st;
             }
             if (workspace != nullptr) return run_sliced(p, plan, static_cast<float *>(workspace), s);
@@ -1030,7 +1030,7 @@ int ko::debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_sl
     const float *aligned = reinterpret_cast<const float *>(uintptr_t{256});
     const Params p{aligned, aligned, nullptr, nullptr, static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),
                    1.0f, 0.0f, 0, 0, static_cast<int>(k), 0};
-    const SlicePlan plan = plan_k_slices(p, kStreamWorkspaceBytes);
+    const SlicePlan plan = plan_k_slices(p, kSgemmPartialBytes);
     *slices = plan.slices;
     *k_slice = plan.k_slice;
     *variant = plan.variant;

@@ -2,7 +2,7 @@
 
 A plan is arithmetic on the shape and the number of compute units (256 when no device is visible, which is also what
 gfx950 has), so its invariants can be checked on the CPU: every slice but the last is a whole number of K tiles, the
-slices cover K exactly once, the fp32 partial products fit the 32 MiB workspace, and shapes that fill the chip whole
+slices cover K exactly once, the fp32 partial products fit the workspace (32 MiB of it for the SGEMM, 64 for the 16-bit GEMM), and shapes that fill the chip whole
 are left whole.
 """
 import itertools
@@ -11,12 +11,13 @@ import pytest
 
 import kernel_optimization_amd as ko
 
-WORKSPACE = 32 << 20
+WORKSPACE = 32 << 20      # what the SGEMM uses of a stream's workspace
+WORKSPACE16 = 64 << 20    # the whole of it
 SIZES = [8, 31, 32, 64, 100, 107, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
 DEPTHS = [64, 512, 767, 768, 1300, 1535, 1536, 2047, 2048, 4096, 8192, 16384, 65536, 262144]
 
 
-def _check(m, n, k, plan, k_tile, min_k, row_pad=1):
+def _check(m, n, k, plan, k_tile, min_k, row_pad=1, workspace=WORKSPACE):
     slices, k_slice, _ = plan
     assert slices >= 1
     if slices == 1:
@@ -24,7 +25,7 @@ def _check(m, n, k, plan, k_tile, min_k, row_pad=1):
     assert k >= min_k, (m, n, k, plan)
     assert k_slice > 0 and k_slice % k_tile == 0, (m, n, k, plan)
     assert (slices - 1) * k_slice < k <= slices * k_slice, (m, n, k, plan)   # no empty slice, none missing
-    assert slices * m * (-(-n // row_pad) * row_pad) * 4 <= WORKSPACE, (m, n, k, plan)
+    assert slices * m * (-(-n // row_pad) * row_pad) * 4 <= workspace, (m, n, k, plan)
 
 
 @pytest.mark.parametrize("m,n", list(itertools.product(SIZES, SIZES)))
@@ -42,11 +43,14 @@ def test_sgemm_plans_cover_k_once_and_fit_the_workspace(m, n):
 def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
     for k in DEPTHS:
         plan = ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=b_layout)
-        _check(m, n, k, plan, k_tile=64, min_k=1536, row_pad=4)   # rows of partial products: whole groups of 4
+        _check(m, n, k, plan, k_tile=64, min_k=1536, row_pad=4, workspace=WORKSPACE16)   # rows of partial products: whole groups of 4
         if plan[0] > 1:
-            assert plan[2] in (128, 64, 32)
+            assert plan[2] in (256, 128, 64, 32)
             if plan[2] == 32:
                 assert m <= 32
+            if plan[2] == 256:   # the pinned kernel: whole tile columns, K tiles in pairs, at most one pair per compute unit
+                assert n % 256 == 0 and k > 8192 and plan[1] % 128 == 0 and plan[1] >= 2048
+                assert plan[0] * -(-m // 256) * (n // 256) <= 256 < 4 * -(-m // 128) * -(-n // 128)
             continue
         # one launch: whole, or K split over the waves of workgroups that own one small output tile each - B
         # column-major, or row-major with rows of whole 16-byte chunks; a multiple of 8 deep (as every K the operator
@@ -70,7 +74,15 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(1024, 1024, 8192)[0] == 1
     assert ko.gemm_plan(4096, 4096, 4096)[0] == 1
     assert ko.gemm_plan(256, 256, 512)[0] == 1
-    assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (7, 2368, 128)
+    assert ko.gemm_plan(768, 768, 16384, sixteen_bit=True) == (5, 3328, 128)
+    assert ko.gemm_plan(256, 1024, 16384, sixteen_bit=True) == (8, 2048, 128)
+    assert ko.gemm_plan(256, 256, 16384, sixteen_bit=True) == (16, 1024, 64)
+    # beyond a quarter of a chip's worth of 128 x 128 tiles and K = 8192: the pinned kernel's tiles in slices
+    assert ko.gemm_plan(768, 3072, 16384, sixteen_bit=True) == (7, 2432, 256)
+    assert ko.gemm_plan(2048, 4096, 16384, sixteen_bit=True) == (2, 8192, 256)
+    assert ko.gemm_plan(2048, 4096, 16384, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (2, 8192, 256)
+    assert ko.gemm_plan(2048, 4096, 8192, sixteen_bit=True)[0] == 1
+    assert ko.gemm_plan(1000, 1000, 16384, sixteen_bit=True)[2] == 128    # not whole tile columns
     assert ko.gemm_plan(512, 520, 16384, sixteen_bit=True, b_layout=ko.ROW_MAJOR)[0] > 1
     # few tiles, column-major B, K up to 8192: one launch that splits K over the waves of a workgroup
     assert ko.gemm_plan(512, 512, 8192, sixteen_bit=True) == (1, 0, 32032)

@@ -1107,3 +1107,87 @@ def test_gemm16_ring_variants_are_exact_on_small_integers(ko, variant):
                 np.testing.assert_array_equal(got.astype(np.float64), want, err_msg="%dx%dx%d, B row-major" % (m, n, k))
     finally:
         ko.set_tuning("gemm16.variant", 0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b_col_major", [True, False])
+@pytest.mark.parametrize("m,n,k,slices", [(256, 256, 256, 2), (300, 512, 648, 2), (1, 256, 1032, 3), (513, 768, 2056, 5),
+                                           (1000, 256, 904, 7), (256, 1024, 8, 2)])
+def test_gemm16_pinned_kernel_in_k_slices_matches_oracle(ko, bf16, b_col_major, m, n, k, slices):
+    """The 256 x 256 tiles of the pinned kernel as pairs (K slice, output tile), fp32 partial products summed by the
+    second kernel: against the oracle, plain and with the whole epilogue, bit-stable from call to call - any row count
+    (the last row of tiles fetches rows that exist), a K that ends inside the last slice (padded with zeros), slices
+    that come out fewer than asked for, more pairs than one per XCD and fewer."""
+    A = _bits16((m, k), 211 + m, bf16)
+    B = _bits16((n, k) if b_col_major else (k, n), 213 + n, bf16)
+    C = _bits16((m, n), 215, bf16)
+    bias = _bits16((n,), 217, bf16)
+    kw = dict(dtype=ko.BF16 if bf16 else ko.F16, b_layout=ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR)
+    ko.set_tuning("gemm16.variant", 62)
+    ko.set_tuning("gemm16.k_slices", slices)
+    try:
+        planned, depth, tile = ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=kw["b_layout"])
+        if k >= 256:
+            assert tile == 256 and 2 <= planned <= slices and depth % 128 == 0 and (planned - 1) * depth < k <= planned * depth
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major)
+        if k < 256:  # one slice at most: the call says so
+            with pytest.raises(ko.KoError):
+                ko.gemm16_host(A, B, m, n, k, **kw)
+            return
+        got = ko.gemm16_host(A, B, m, n, k, **kw)
+        assert_gemm16_close(_to_f64(got, bf16), ref64, ap, k, bf16=bf16)
+        np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, **kw), got)
+        _, ref64, ap = oracle.gemm16(A, B, m, n, k, bf16=bf16, b_col_major=b_col_major, C_bits=C, beta=0.5, bias_bits=bias, act=2)
+        got = ko.gemm16_host(A, B, m, n, k, C_bits=C, beta=0.5, bias_bits=bias, act=2, **kw)
+        assert_gemm16_act_close(_to_f64(got, bf16), ref64, ap + 2.0, k, bf16=bf16)
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+        ko.set_tuning("gemm16.k_slices", 0)
+
+
+def test_gemm16_pinned_kernel_in_k_slices_is_exact_on_small_integers(ko):
+    """Entries in -2 .. 2, sums below 2^11: a K tile left out, taken twice, read before it landed or added to the wrong
+    slice shows as a wrong integer; a guard area behind D stays as it was.  Pair counts that divide over the 8 XCDs
+    (blocked tile order) and that do not, two rounds of pairs per workgroup (257 x 4096 in 15 slices: 480 pairs), both
+    layouts of B."""
+    rng = np.random.default_rng(62)
+    ko.set_tuning("gemm16.variant", 62)
+    try:
+        for m, n, k, slices in ((512, 1024, 1024, 4), (700, 768, 2432, 7), (2048, 2048, 512, 2), (257, 4096, 1920, 15), (256, 256, 32768, 16),
+                                (1500, 3072, 768, 3)):
+            ko.set_tuning("gemm16.k_slices", slices)
+            Ai = rng.integers(-2, 3, (m, k)).astype(np.float16)
+            Bi = rng.integers(-2, 3, (n, k)).astype(np.float16)  # [n][k]
+            Ai[rng.random((m, k)) > 64.0 / k] = 0
+            want = Ai.astype(np.float64) @ Bi.astype(np.float64).T
+            dA, dB = ko.DeviceBuffer.from_numpy(Ai.view(np.uint16)), ko.DeviceBuffer.from_numpy(Bi.view(np.uint16))
+            guard = 4096
+            dD = ko.DeviceBuffer.from_numpy(np.full(m * n + guard, 0x7bff, np.uint16))
+            ko.gemm16(m, n, k, dA, dB, dD)
+            ko.synchronize()
+            out = dD.download(np.uint16, (m * n + guard,))
+            np.testing.assert_array_equal(out[:m * n].view(np.float16).astype(np.float64).reshape(m, n), want,
+                                          err_msg="%dx%dx%d in %d slices" % (m, n, k, slices))
+            assert (out[m * n:] == 0x7bff).all(), "%dx%dx%d: the guard area behind D was written" % (m, n, k)
+            got = ko.gemm16_host(Ai.view(np.uint16), np.ascontiguousarray(Bi.T).view(np.uint16), m, n, k,
+                                 b_layout=ko.ROW_MAJOR).view(np.float16)
+            np.testing.assert_array_equal(got.astype(np.float64), want, err_msg="%dx%dx%d, B row-major" % (m, n, k))
+    finally:
+        ko.set_tuning("gemm16.variant", 0)
+        ko.set_tuning("gemm16.k_slices", 0)
+
+
+@pytest.mark.parametrize("m,n,k,b_col_major", [(1000, 1280, 8200, True), (1100, 1024, 8456, False), (520, 2304, 9216, True)])
+def test_gemm16_deep_k_on_mid_size_outputs_goes_out_as_pinned_slices(ko, m, n, k, b_col_major):
+    """What the default dispatch does with more 128 x 128 tiles than a quarter of the compute units, at most half of them of
+    256 x 256 tiles and K beyond 8192: sampled rows (every column) against the oracle, and bit-stable."""
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    planned, depth, tile = ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout)
+    assert tile == 256 and planned >= 2 and depth >= 2048 and depth % 128 == 0
+    A = _bits16((m, k), 311, False)
+    B = _bits16((n, k) if b_col_major else (k, n), 313, False)
+    got = ko.gemm16_host(A, B, m, n, k, b_layout=layout)
+    rows = np.unique(np.concatenate([np.arange(0, m, 41), [255, 256, m - 1]]))
+    _, ref64, ap = oracle.gemm16(A[rows], B, len(rows), n, k, b_col_major=b_col_major)
+    assert_gemm16_close(_to_f64(got[rows], False), ref64, ap, k)
+    np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, b_layout=layout), got)
