@@ -2319,7 +2319,12 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             const int64_t tiles = rows_top * tn, rounds = tiles / cu;
             if (rounds >= 1 && tiles % cu != 0) {
                 const int64_t rows1 = rounds * cu / tn;  // whole tile rows within the full rounds
-                if (rows1 >= 1 && 6 * (rows_top - rows1) * tn <= cu) rows_top = rows1;
+                const int64_t rest = (rows_top - rows1) * tn;
+                // (up to a quarter of a round when the rows cut off then are one pass of the ring kernel's 128 x 128
+                // tiles: 20000 x 1024 x 4096, 316 tiles, 199 -> 171 us; 20000 x 1024 x 1024 53.6 -> 47.0)
+                const bool ring_rest = p.K >= 1024 && p.K <= 8192 && 4 * rest <= cu && tuning(knob_gemm16_wave_k) != 1 &&
+                                       (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0));
+                if (rows1 >= 1 && (6 * rest <= cu || ring_rest)) rows_top = rows1;
             }
             if (rows_top * 256 < p.M && 2 * rows_top * tn >= cu) {
                 const int64_t m1 = rows_top * 256;

@@ -935,11 +935,12 @@ def test_gemm16_pinned_kernel_takes_any_row_count(ko, variant, bf16, b_col_major
 
 
 @pytest.mark.parametrize("m,n,k", [(3000, 3072, 768), (6000, 1024, 1024), (1240, 2304, 3072), (16000, 3072, 768),
-                                   (4093, 3072, 768), (8191, 1024, 1024), (5001, 2304, 776)])
+                                   (4093, 3072, 768), (8191, 1024, 1024), (5001, 2304, 776), (19500, 1024, 1032)])
 def test_gemm16_ragged_rows_through_the_default_dispatch_are_exact(ko, m, n, k):
     """Row counts that are not multiples of the tile height (of 8 or not), on the shapes the dispatch sends to the pinned
     kernel as they are (256 x 256 tiles, and 128 x 256 tiles): small integers make every sum exact, so any row fetched
-    from the wrong place or stored where it does not belong shows."""
+    from the wrong place or stored where it does not belong shows.  19500 x 1024: 308 tiles on 256 compute units - the
+    52 below the full round are cut off and go to the ring kernel's 128 x 128 tiles."""
     rng = np.random.default_rng(m + k)
     A = rng.integers(-3, 4, (m, k)).astype(np.float16)
     B = rng.integers(-3, 4, (n, k)).astype(np.float16)
