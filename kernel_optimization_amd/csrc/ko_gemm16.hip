@@ -1352,14 +1352,15 @@ int launch_pinned(Params p, hipStream_t stream) {
 // matrix): every kernel above walks K in steps that all waves of a workgroup take together - a barrier per K tile,
 // one or two K tiles in flight per workgroup - and with a workgroup or less per compute unit such a step costs its
 // latencies (0.4 us per 64 k on 64 x 64 tiles, whatever the arithmetic).  Here a workgroup owns one (32 TM) x (32 TN)
-// output tile (32 x 32 to 128 x 64) and wave w multiplies K tiles w, w + WAVES, ... of it: the whole tile over its own share of K, out of two
+// output tile (32 x 32 to 128 x 64) and wave w multiplies the w-th of WAVES ranges of K tiles of it: the whole tile over its own share of K, out of two
 // LDS stages of its own that it fills with direct-to-LDS loads (eight rows of 128 bytes per wave-level load, as
 // in the kernels above) - no barrier in the loop, WAVES times fewer steps in a row, and two K tiles per wave in
 // flight.  At the end the waves leave their fp32 tiles in LDS and the workgroup adds them in wave order (the same
 // bits from call to call) and applies alpha, beta * C, the bias and the activation once.
 // Any M, N and any K that is a multiple of 8: a row at or past M (N) is fetched from the last row instead and its
-// results are not stored; a 16-byte chunk at or past K - in the last K tile, or in a K tile past the end that a
-// wave's second stage asks for - is fetched from sixteen zero bytes, chosen per load with a compare and two selects.
+// results are not stored; a 16-byte chunk at or past the end of the wave's range of K - in the last K tile, or in a K
+// tile past the range that a wave's second stage asks for - is fetched from sixteen zero bytes, chosen per load with a
+// compare and two selects.
 // B_ROW: B as [K][N] (rows ldb apart, N and ldb multiples of 8).  A wave's K tile of B is 64 rows of 32 TN values and
 // stays row-major in LDS; a wave-level load covers 1 KB of it (16, 8 or 4 rows), the 16-byte chunk a lane fetches
 // is permuted with the row number modulo 4 - as far as the row has chunks for it - and the fragments come out of
@@ -1369,10 +1370,11 @@ template <int TM, int TN, int WAVES, bool BF16, bool B_ROW = false>
 __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params p) {
     constexpr int WTM = 32 * TM, WTN = 32 * TN;
     constexpr int KS = kBK / 16;
+    constexpr int STAGES = 2;
     constexpr int A_LOADS = WTM / 8, B_LOADS = WTN / 8, LOADS = A_LOADS + B_LOADS;
-    constexpr int A_BYTES = WTM * kBK * 2, STAGE_BYTES = (WTM + WTN) * kBK * 2, WAVE_BYTES = 2 * STAGE_BYTES;
+    constexpr int A_BYTES = WTM * kBK * 2, STAGE_BYTES = (WTM + WTN) * kBK * 2, WAVE_BYTES = STAGES * STAGE_BYTES;
     constexpr int LDP = WTN + 4;  // floats between the rows of a wave's fp32 tile in LDS
-    static_assert(KS == 4 && LOADS <= 31, "two K tiles of loads must fit the 6-bit counter");
+    static_assert(KS == 4 && (STAGES - 1) * LOADS <= 63 && STAGES >= 2, "the loads in flight must fit the 6-bit counter");
     static_assert(WTM * LDP * 4 <= WAVE_BYTES && WAVES * WAVE_BYTES <= 160 * 1024, "");
     static_assert(TM * TN <= 8 && TM + TN <= 6, "");
 
@@ -1390,8 +1392,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
     const int m0 = (tile / p.tiles_n) * WTM, n0 = (tile % p.tiles_n) * WTN;
     const int M = p.M, N = p.N, K = p.K;
     const int64_t ldk = p.ldk;
+    // wave w takes the K tiles [w * per, (w + 1) * per), a range of its own.  (Dealt round-robin - w, w + WAVES, ... - the
+    // waves of a workgroup walk through adjacent 128-byte pieces of every row together, and weights that come from memory
+    // stream more slowly: 8 x 8192 x 8192 31.3 us against 28.6, 8 x 4096 x 4096 11.2 against 10.1; problems that live in
+    // the L2s are level, within 3 %.  A read-only loop with this kernel's loads - eight rows of 128 bytes per wave-level
+    // load - over the same 134 MB: 4.6 TB/s round-robin, 5.9 in ranges.  Three or four stages per wave on a K tile
+    // of A cut down to 8 rows gained nothing over two.)  p.band_rows == 0 deals round-robin, for comparison.
     const int KT = (K + kBK - 1) / kBK;
-    const int my_tiles = wave < KT ? (KT - wave + WAVES - 1) / WAVES : 0;
+    const bool ranges = p.band_rows != 0;
+    const int per = (KT + WAVES - 1) / WAVES;
+    const int k_first = ranges ? wave * per * kBK : wave * kBK;             // first k of this wave's K tiles
+    const int k_step = ranges ? kBK : WAVES * kBK;                          // from one of them to the next
+    // ranges: where this wave's range ends - chunks at or past it are fetched as zeros
+    const int k_end = ranges && k_first + per * kBK < K ? k_first + per * kBK : K;
+    const int my_tiles = k_first < k_end ? (k_end - k_first + k_step - 1) / k_step : 0;
 
     typedef const __attribute__((address_space(1))) void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
@@ -1408,7 +1422,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
         const int r = m0 + 8 * i + row_in;
-        src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + wave * kBK + lane_k[i & 1]);
+        src_a[i] = reinterpret_cast<const char *>(p.A + static_cast<int64_t>(r < M ? r : M - 1) * ldk + k_first + lane_k[i & 1]);
     }
     // row-major B: NCH chunks per LDS row, RPL rows per wave-level load; lane l fills position l % NCH of row
     // l / NCH of its load's rows, with chunk (l % NCH) ^ b_swz(row) of that row of the tile
@@ -1422,31 +1436,31 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
             static_assert(RPL % 4 == 0, "");
             const int c = n0 + 8 * ((lane % NCH) ^ b_swz(b_krow));
             b_inside = c < N;
-            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(wave * kBK + RPL * j + b_krow) * p.ldb + (b_inside ? c : 0));
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(k_first + RPL * j + b_krow) * p.ldb + (b_inside ? c : 0));
         } else {
             const int r = n0 + 8 * j + row_in;
-            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + wave * kBK + lane_k[j & 1]);
+            src_b[j] = reinterpret_cast<const char *>(p.B + static_cast<int64_t>(r < N ? r : N - 1) * ldk + k_first + lane_k[j & 1]);
         }
     }
-    int ld_k0 = wave * kBK;  // first k of the K tile to fetch next
+    int ld_k0 = k_first;  // first k of the K tile to fetch next
     char *const wave_lds = lds_bytes + wave * WAVE_BYTES;
-    const int64_t b_tile_step = B_ROW ? static_cast<int64_t>(WAVES * kBK) * p.ldb * 2 : WAVES * kBK * 2;  // bytes to this wave's next K tile
+    const int64_t b_tile_step = B_ROW ? static_cast<int64_t>(k_step) * p.ldb * 2 : k_step * 2;  // bytes to this wave's next K tile
     auto issue = [&](int stage) {
-        const bool in0 = ld_k0 + lane_k[0] < K, in1 = ld_k0 + lane_k[1] < K;
+        const bool in0 = ld_k0 + lane_k[0] < k_end, in1 = ld_k0 + lane_k[1] < k_end;
         char *dst = wave_lds + stage * STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) {
             __builtin_amdgcn_global_load_lds((gptr_t)((i & 1 ? in1 : in0) ? src_a[i] : zeros), (lptr_t)(dst + 1024 * i), 16, 0, 0);
-            src_a[i] += WAVES * kBK * 2;
+            src_a[i] += k_step * 2;
         }
 #pragma unroll
         for (int j = 0; j < B_LOADS; ++j) {
             bool in = j & 1 ? in1 : in0;
-            if constexpr (B_ROW) in = b_inside && ld_k0 + RPL * j + b_krow < K;
+            if constexpr (B_ROW) in = b_inside && ld_k0 + RPL * j + b_krow < k_end;
             __builtin_amdgcn_global_load_lds((gptr_t)(in ? src_b[j] : zeros), (lptr_t)(dst + A_BYTES + 1024 * j), 16, 0, 0);
             src_b[j] += b_tile_step;
         }
-        ld_k0 += WAVES * kBK;
+        ld_k0 += k_step;
     };
 
     // LDS byte addresses of this lane's fragments (stage 0, block 0) for the four K steps
@@ -1522,12 +1536,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
     using C1 = std::integral_constant<int, 1>;
     using C2 = std::integral_constant<int, 2>;
     using C3 = std::integral_constant<int, 3>;
-    // One K tile out of stage S; the loads of the K tile after next go out as soon as the stage's last fragments
-    // are in registers.  Loads complete in order: with two K tiles' worth in flight, all but the last LOADS done
-    // means that this stage has landed.
+    // One K tile out of stage S; the loads of the K tile STAGES further on go out as soon as the stage's last fragments
+    // are in registers.  Loads complete in order: with STAGES K tiles' worth in flight, all but the last
+    // (STAGES - 1) LOADS done means that this stage has landed.
     auto k_tile = [&](auto stage_c) {
         constexpr int S = decltype(stage_c)::value;
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 1) * LOADS) : "memory");
         read_frags(C0{}, C0{}, stage_c);
         read_frags(C1{}, C1{}, stage_c);
         wait_frags(0);
@@ -1542,12 +1556,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm16_wave_k_kernel(const Params 
         multiply(0);
         multiply(1);
     };
-    issue(0);
-    issue(1);
-    for (int t = 0; t < my_tiles; t += 2) {
-        k_tile(C0{});
-        k_tile(C1{});  // past this wave's last K tile: a stage of zeros
-    }
+    static_for<STAGES>([&](auto s_c) { issue(decltype(s_c)::value); });
+    for (int t = 0; t < my_tiles; t += STAGES) static_for<STAGES>(k_tile);  // past this wave's last K tile: stages of zeros
     // the loads still in flight (K tiles past the end: zeros) must land before the stages are written over
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -1616,6 +1626,7 @@ int launch_wave_k(Params p, hipStream_t stream) {
     const int64_t tiles = static_cast<int64_t>((p.M + 32 * TM - 1) / (32 * TM)) * p.tiles_n;
     if (tiles > 0x7fffffff) return fail(KO_ERR_UNSUPPORTED_SHAPE, "gemm16: too many tiles for the wave-K variant");
     p.nblocks = static_cast<int>(tiles);
+    p.band_rows = tuning(knob_gemm16_mapping) == 2 ? 0 : 1;  // knob gemm16.mapping = 2: K tiles dealt round-robin
     kernel<<<dim3(static_cast<unsigned>(p.nblocks)), dim3(64 * WAVES), lds_bytes, stream>>>(p);
     KO_CHECK_LAUNCH();
     return KO_OK;
