@@ -498,6 +498,28 @@ def bench_gemm16_midsize(steps, warmup, vendor):
                 min_vs_hipblaslt=ratios[0] if ratios else None, max_vs_hipblaslt=ratios[-1] if ratios else None, rows=rows)
 
 
+# weight-gradient shapes: a layer's weight (M x N) against batch x sequence (K), and a decoding step's few rows
+DEEP_K_SHAPES = ((768, 768, 16384), (768, 3072, 16384), (3072, 768, 16384), (768, 2304, 16384), (1024, 1024, 16384),
+                 (1024, 4096, 16384), (4096, 1024, 16384), (4096, 4096, 16384), (1024, 3072, 12288), (2048, 4096, 16384),
+                 (1536, 2304, 16384), (2048, 2048, 32768), (512, 512, 32768), (256, 1024, 16384), (1024, 4096, 8192),
+                 (8, 8192, 8192), (32, 8192, 8192), (8, 4096, 4096), (8, 28672, 4096))
+
+
+def bench_gemm16_deep_k(steps, warmup, vendor):
+    """The 16-bit GEMM on a deep K against few or mid-size outputs (weight gradients), and on a handful of rows against
+    large weights (decoding), next to hipBLASLt on the same buffers; with the planner's decision."""
+    rows = []
+    for m, n, k in DEEP_K_SHAPES:
+        res, _ = bench_gemm16(4, steps, warmup, vendor, shape=(m, n, k), c_loop=True)
+        slices, k_slice, tile = ko.gemm_plan(m, n, k, sixteen_bit=True)
+        rows.append(dict(m=m, n=n, k=k, us=res["kernel_us"], tflops=res["flops"] / res["kernel_us"] / 1e6,
+                         hipblaslt_us=res["flops"] / res["hipblaslt_tflops"] / 1e6 if "hipblaslt_tflops" in res else None,
+                         vs_hipblaslt=res.get("vs_hipblaslt"), k_slices=slices, k_slice=k_slice, slice_tile=tile))
+    ratios = sorted(r["vs_hipblaslt"] for r in rows if r["vs_hipblaslt"])
+    return dict(steps=steps, warmup=warmup, shapes=len(rows), median_vs_hipblaslt=ratios[len(ratios) // 2] if ratios else None,
+                min_vs_hipblaslt=ratios[0] if ratios else None, max_vs_hipblaslt=ratios[-1] if ratios else None, rows=rows)
+
+
 def bench_gemm16_active_cus(steps, warmup):
     """Time per K tile of the 256 x 256 kernel of the 16-bit GEMM by how many compute units have a tile: K = 4096
     (64 K tiles per output tile), N = 3072 (12 tile columns), M from 256 to 16384."""
@@ -838,7 +860,7 @@ def main():
                     help="untimed launches before the timed ones; the device takes a few hundred short launches "
                          "to settle its clocks, so the microsecond-scale secondary workloads use at least 300")
     ap.add_argument("--workload", default=inputs.CONFIGS[HEADLINE]["name"],
-                    help="one of %s, copy_f32, hbm_ceilings, short_kernels, gemm16_midsize, gemm16_active_cus, softmax_f32_786432x512_unmasked, or a long-row line by name: "
+                    help="one of %s, copy_f32, hbm_ceilings, short_kernels, gemm16_midsize, gemm16_deep_k, gemm16_active_cus, softmax_f32_786432x512_unmasked, or a long-row line by name: "
                          "(softmax|layernorm)_f32_<rows>x<cols>_(auto|warp|block|nocache); or one 16-bit GEMM shape: gemm_f16_<m>x<n>x<k>" % ", ".join(sorted(WORKLOADS)))
     ap.add_argument("--all", dest="all", action="store_true", default=True,
                     help="also measure the other four configurations (default)")
@@ -857,6 +879,9 @@ def main():
         return
     if args.workload == "hbm_ceilings":  # the whole streaming sweep, for profiles/
         print(json.dumps(bench_ceilings(min(args.steps, 10), 3, full=True)))
+        return
+    if args.workload == "gemm16_deep_k":  # the sweep behind profiles/gemm16_deep_k.md
+        print(json.dumps(bench_gemm16_deep_k(min(args.steps, 30), max(args.warmup, 60), vendor)))
         return
     if args.workload == "gemm16_midsize":  # the sweep behind profiles/gemm16_midsize.md
         print(json.dumps(bench_gemm16_midsize(min(args.steps, 30), max(args.warmup, 100), vendor)))
