@@ -57,6 +57,11 @@ def test_operators_replay_from_a_hip_graph(ko):
     a5, b5, d5 = ko.DeviceBuffer(m5 * k5 * 2), ko.DeviceBuffer(n5 * k5 * 2), ko.DeviceBuffer(m5 * n5 * 2)
     ko.fill_uniform_16(a5, m5 * k5, 513)
     ko.fill_uniform_16(b5, n5 * k5, 514)
+    m7, n7, k7 = 1000, 1280, 8200  # 16-bit, a mid-size output and K beyond 8192: the pinned kernel's tiles in K slices
+    a7, b7, d7 = ko.DeviceBuffer(m7 * k7 * 2), ko.DeviceBuffer(n7 * k7 * 2), ko.DeviceBuffer(m7 * n7 * 2)
+    ko.fill_uniform_16(a7, m7 * k7, 516)
+    ko.fill_uniform_16(b7, n7 * k7, 517)
+    assert ko.gemm_plan(m7, n7, k7, sixteen_bit=True)[2] == 256
     rows6, cols6 = 8, 131072  # a few long rows: cut into pieces that hand partial results over through the workspace
     x6 = ko.DeviceBuffer.from_numpy(inputs.normal_f32((rows6, cols6), 515, 0.0, 4.0))
     s6, l6 = ko.DeviceBuffer(rows6 * cols6 * 4), ko.DeviceBuffer(rows6 * cols6 * 4)
@@ -83,23 +88,24 @@ def test_operators_replay_from_a_hip_graph(ko):
         ko.set_tuning("gemm16.wave_k", 0)
         ko.softmax(x6, s6, rows6, cols6, stream=stream)
         ko.layernorm(s6, l6, rows6, cols6, stream=stream)
+        ko.gemm16(m7, n7, k7, a7, b7, d7, stream=stream)
 
     def outputs():
         return (dl.download(np.uint32, (rows, cols)), dmean.download(np.uint32, (rows,)),
                 d16.download(np.uint16, (m, n)), d32.download(np.uint32, (m, n)), d2.download(np.uint16, (m2, n2)),
                 d3.download(np.uint16, (m3, n3)), d4.download(np.uint32, (m4, n4)), d5.download(np.uint16, (m5, n5)),
-                l6.download(np.uint32, (rows6, cols6)))
+                l6.download(np.uint32, (rows6, cols6)), d7.download(np.uint16, (m7, n7)))
 
     def clear():
         for buf, nbytes in ((ds, rows * cols * 4), (dl, rows * cols * 4), (dmean, rows * 4), (d16, m * n * 2), (d32, m * n * 4),
                             (d2, m2 * n2 * 2), (d3, m3 * n3 * 2), (d4, m4 * n4 * 4), (d5, m5 * n5 * 2),
-                            (s6, rows6 * cols6 * 4), (l6, rows6 * cols6 * 4)):
+                            (s6, rows6 * cols6 * 4), (l6, rows6 * cols6 * 4), (d7, m7 * n7 * 2)):
             buf.upload(np.zeros(nbytes, np.uint8))
 
     chain()
     stream.synchronize()
     want = outputs()
-    assert want[0].any() and want[2].any() and want[3].any() and want[6].any() and want[7].any() and want[8].any()
+    assert want[0].any() and want[2].any() and want[3].any() and want[6].any() and want[7].any() and want[8].any() and want[9].any()
 
     graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
     assert hip.hipStreamBeginCapture(stream.handle, 0) == 0  # hipStreamCaptureModeGlobal
