@@ -502,7 +502,7 @@ def bench_gemm16_midsize(steps, warmup, vendor):
 DEEP_K_SHAPES = ((768, 768, 16384), (768, 3072, 16384), (3072, 768, 16384), (768, 2304, 16384), (1024, 1024, 16384),
                  (1024, 4096, 16384), (4096, 1024, 16384), (4096, 4096, 16384), (1024, 3072, 12288), (2048, 4096, 16384),
                  (1536, 2304, 16384), (2048, 2048, 32768), (512, 512, 32768), (256, 1024, 16384), (1024, 4096, 8192),
-                 (8, 8192, 8192), (32, 8192, 8192), (8, 4096, 4096), (8, 28672, 4096))
+                 (8, 8192, 8192), (32, 8192, 8192), (8, 4096, 4096), (8, 28672, 4096), (32, 32000, 4096), (8, 128256, 4096))
 
 
 def bench_gemm16_deep_k(steps, warmup, vendor):

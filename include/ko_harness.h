@@ -85,7 +85,9 @@ int ko_debug_stream_workspace_count(int *count);
  * problem; 16-bit GEMM: 128 or 64, the tile edge, or 32 for 32 x 256 tiles).  The 16-bit GEMM with B in layout
  * b_layout (KO_ROW_MAJOR / KO_COL_MAJOR) has one more answer for a problem of few tiles: slices = 1 and tile =
  * 1000 * rows + columns - one launch whose workgroups own one output tile of that size and either split K over
- * their waves (32032, 32064, 64064) or walk K together through a deep ring of LDS stages (64128, 128064, 128128);
+ * their waves (32032, 32064, 64064) or walk K together through a deep ring of LDS stages (64128, 128064, 128128;
+ * 1032064: 32 x 64 tiles of that kernel for a problem of at most 32 rows); slices > 1 with tile = 256: the pinned
+ * kernel's 256 x 256 tiles in K slices;
  * tile = 0: none of this.  Touches no device memory and launches nothing. */
 int ko_debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
 int ko_debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile);

@@ -2185,13 +2185,22 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
 // (26.0), 4096 x 1024 x 4096 56.2 -> 40.3 (40.8), 1000 x 4096 x 4096 74.2 -> 43.4 (40.4), 3000 x 1024 x 1024 21.7 -> 11.5
 // (12.8), 512 x 4096 x 1024 16.1 -> 11.2 (11.4); the half tile there is 128 x 64 whatever the shape (64 x 128 - rows of
 // 256 bytes in the stage of B - is the slower one: 2048 x 768 x 3072 22.7 against 20.6).
-// Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128.
+// Returns 0, or 1000 * rows + columns of the tile: 64128, 128064, 128128; 1032064 for the 32 x 64 tiles of a problem of
+// at most 32 rows (the million tells them from the other kernel's 32 x 64).
 int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     // (a K beyond 8192 is left to the K slices below, which run this kernel's 128 x 128 tiles: 512 x 2304 x 16384 whole on
     // 144 tiles of 128 x 64 103 us, in slices 67)
-    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k < 512 || k > 8192) return 0;
+    if (tuning(knob_gemm16_wave_k) == 1 || tuning(knob_gemm16_k_slices) != 0 || k < 512) return 0;
     const int64_t cu = compute_units();
     const int64_t m64 = (m + 63) / 64, m128 = (m + 127) / 128, n64 = (n + 63) / 64, n128 = (n + 127) / 128;
+    // At most 32 rows against more columns than the kernel above takes (a decoding step against a vocabulary or a wide
+    // feed-forward weight): 32 x 64 tiles, two waves, two workgroups per compute unit, however many rounds - the time is
+    // the weights' way out of memory, and rows of A that a taller tile would fetch again and again are not.  Before
+    // -> now (hipBLASLt), us: 8 x 28672 x 4096 52.3 -> 42.7 (37.5), 32 x 32000 x 4096 58.5 -> 51.2 (43.6), 8 x 128256 x 4096
+    // 237 -> 177 (151), 8 x 50304 x 1024 27.2 -> 23.7 (18.5); 32 x 128 tiles with six stages (one workgroup per compute
+    // unit) 47.6 / 56.1 / 181 / 24.0, with three 61 / 70 / 190 / 20.7.
+    if (m <= 32 && n64 > cu) return 1032064;
+    if (k > 8192) return 0;
     if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above
     if (b_row_major) {
         if (m128 * n64 <= cu) return 128064;
@@ -2224,6 +2233,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
     }
     if (variant <= 0 && p.k_slice == 0 && (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0))) {
         switch (ring_tile(p.M, p.N, p.K, B_ROW_MAJOR)) {
+            case 1032064: return launch_ring<32, 64, 1, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
             case 64128: return launch_ring<64, 128, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
             case 128064: return launch_ring<128, 64, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
             case 128128: return launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
@@ -2404,6 +2414,7 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             if (variant == 81) return launch_ring<128, 64, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);   // 6 stages of 24 KB
             if (variant == 82) return launch_ring<64, 128, 2, 2, 6, BF16, B_ROW_MAJOR>(p, stream);
             return launch_ring<128, 128, 2, 4, 5, BF16, B_ROW_MAJOR>(p, stream);  // 8 waves of 64 x 32, 5 stages
+        case 84: return launch_ring<32, 64, 1, 2, 6, BF16, B_ROW_MAJOR>(p, stream);  // two waves of 32 x 32, 6 stages of 12 KB
         case 70:
         case 71:
         case 72:

@@ -55,8 +55,10 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
         # one launch: whole, or K split over the waves of workgroups that own one small output tile each - B
         # column-major, or row-major with rows of whole 16-byte chunks; a multiple of 8 deep (as every K the operator
         # takes); at most one such tile per compute unit, and the smallest tile for which that holds
-        assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064, 128128)
-        if plan[2]:
+        assert plan[1] == 0 and plan[2] in (0, 32032, 32064, 64064, 64128, 128064, 128128, 1032064)
+        if plan[2] == 1032064:   # at most 32 rows against more columns than 64-wide tiles for every compute unit
+            assert m <= 32 and -(-n // 64) > 256 and k >= 512 and k % 8 == 0 and (b_layout == ko.COL_MAJOR or n % 8 == 0)
+        elif plan[2]:
             tm, tn = divmod(plan[2], 1000)
             assert -(-m // tm) * -(-n // tn) <= 256 and k % 8 == 0
             if plan[2] in (32032, 32064, 64064):   # K over the waves of a workgroup
@@ -100,6 +102,11 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(100, 1028, 1024, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 0)  # rows of B off 16 bytes
     assert ko.gemm_plan(2048, 2048, 2048, sixteen_bit=True)[0] == 1
     assert ko.gemm_plan(16384, 3072, 768, sixteen_bit=True)[0] == 1
+    # a decoding step against a vocabulary: 32 x 64 tiles of the ring kernel, however many rounds
+    assert ko.gemm_plan(8, 128256, 4096, sixteen_bit=True) == (1, 0, 1032064)
+    assert ko.gemm_plan(32, 32000, 4096, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 1032064)
+    assert ko.gemm_plan(8, 8192, 8192, sixteen_bit=True) == (1, 0, 32032)
+    assert ko.gemm_plan(33, 32000, 4096, sixteen_bit=True)[2] != 1032064
     # operand rows off 16-byte boundaries are sliced like the others
     assert ko.gemm_plan(282, 31, 13104)[0] > 1
     assert ko.gemm_plan(282, 31, 13104, sixteen_bit=True)[0] > 1

@@ -1017,7 +1017,8 @@ def test_gemm16_wave_k_variants_are_exact_on_small_integers(ko, variant):
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("m,n,k,tile", [(100, 1024, 1024, 32032), (512, 768, 3072, 32064), (1000, 1024, 4096, 64064),
                                         (8, 4096, 4096, 32032), (200, 2304, 768, 32064), (750, 1000, 1032, 64064),
-                                        (2040, 704, 2056, 64128), (500, 4000, 1032, 128064), (3000, 1000, 520, 128128)])
+                                        (2040, 704, 2056, 64128), (500, 4000, 1032, 128064), (3000, 1000, 520, 128128),
+                                        (8, 16448, 1032, 1032064), (30, 17000, 520, 1032064)])
 @pytest.mark.parametrize("b_col_major", [True, False])
 def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, bf16, b_col_major):
     """A few hundred to a few thousand rows against a weight matrix: the dispatch sends them to the kernel that
@@ -1046,8 +1047,9 @@ def test_gemm16_small_problems_through_the_default_dispatch(ko, m, n, k, tile, b
 
 
 # a deep ring of LDS stages: 80 = 128 x 128 tiles (4 waves, 4 stages), 81 = 128 x 64, 82 = 64 x 128 (6 stages),
-# 83 = 128 x 128 with 8 waves and 5 stages
-RING_VARIANTS = [80, 81, 82, 83]
+# 83 = 128 x 128 with 8 waves and 5 stages, 84 = 32 x 64 (2 waves, 6 stages: what a problem of at most 32 rows and
+# many columns takes)
+RING_VARIANTS = [80, 81, 82, 83, 84]
 
 
 @pytest.mark.parametrize("variant", RING_VARIANTS)
