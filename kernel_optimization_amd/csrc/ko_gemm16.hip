@@ -2201,6 +2201,12 @@ int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     // unit) 47.6 / 56.1 / 181 / 24.0, with three 61 / 70 / 190 / 20.7.
     if (m <= 32 && n64 > cu) return 1032064;
     if (k > 8192) return 0;
+    // One row of tiles against more columns than compute units (64 or 128 rows against a vocabulary): this kernel in
+    // several rounds, where the persistent kernels' 256 x 256 tiles are mostly rows that do not exist
+    // (64 x 128256 x 4096 258 -> 187 us (hipBLASLt 174), 128 x 128256 x 4096 274 -> 215 (204), 64 x 50304 x 1024 31.8 -> 27.8
+    // (21.7); 128 x 50304 x 1024 stays: 31.9 against 33.6)
+    if (m > 32 && m <= 64 && n128 > cu && !b_row_major) return 64128;
+    if (m > 32 && m <= 128 && n128 > cu && k >= 2048) return 128128;
     if (m64 * n64 <= cu) return 0;  // few tiles: the kernel above
     if (b_row_major) {
         if (m128 * n64 <= cu) return 128064;

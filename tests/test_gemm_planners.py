@@ -60,13 +60,16 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
             assert m <= 32 and -(-n // 64) > 256 and k >= 512 and k % 8 == 0 and (b_layout == ko.COL_MAJOR or n % 8 == 0)
         elif plan[2]:
             tm, tn = divmod(plan[2], 1000)
-            assert -(-m // tm) * -(-n // tn) <= 256 and k % 8 == 0
+            # at most one such tile per compute unit - or one row of ring tiles, however many
+            assert (-(-m // tm) * -(-n // tn) <= 256 or (m <= tm and plan[2] in (64128, 128128))) and k % 8 == 0
             if plan[2] in (32032, 32064, 64064):   # K over the waves of a workgroup
                 assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and 128 <= k <= 8192
                 assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
             else:                                   # a deep ring of LDS stages: when the small tiles are too many
                 assert (b_layout == ko.COL_MAJOR or (n % 8 == 0 and plan[2] != 64128)) and 512 <= k <= 8192
                 assert -(-m // 64) * -(-n // 64) > 256
+                if -(-m // tm) * -(-n // tn) > 256:
+                    assert (plan[2] == 64128 and b_layout == ko.COL_MAJOR) or (plan[2] == 128128 and k >= 2048)
 
 
 def test_measured_decisions_stay_put():
@@ -107,6 +110,11 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(32, 32000, 4096, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 1032064)
     assert ko.gemm_plan(8, 8192, 8192, sixteen_bit=True) == (1, 0, 32032)
     assert ko.gemm_plan(33, 32000, 4096, sixteen_bit=True)[2] != 1032064
+    assert ko.gemm_plan(64, 128256, 4096, sixteen_bit=True) == (1, 0, 64128)
+    assert ko.gemm_plan(64, 128256, 4096, sixteen_bit=True, b_layout=ko.ROW_MAJOR) == (1, 0, 128128)
+    assert ko.gemm_plan(128, 128256, 4096, sixteen_bit=True) == (1, 0, 128128)
+    assert ko.gemm_plan(128, 50304, 1024, sixteen_bit=True)[2] == 0
+    assert ko.gemm_plan(256, 128256, 4096, sixteen_bit=True)[2] == 0
     # operand rows off 16-byte boundaries are sliced like the others
     assert ko.gemm_plan(282, 31, 13104)[0] > 1
     assert ko.gemm_plan(282, 31, 13104, sixteen_bit=True)[0] > 1

@@ -1194,3 +1194,22 @@ def test_gemm16_deep_k_on_mid_size_outputs_goes_out_as_pinned_slices(ko, m, n, k
     _, ref64, ap = oracle.gemm16(A[rows], B, len(rows), n, k, b_col_major=b_col_major)
     assert_gemm16_close(_to_f64(got[rows], False), ref64, ap, k)
     np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, b_layout=layout), got)
+
+
+@pytest.mark.parametrize("m,n,k,b_col_major,tile", [(40, 33000, 520, True, 64128), (100, 32776, 2056, True, 128128),
+                                                    (60, 32776, 2056, False, 128128)])
+def test_gemm16_one_row_of_tiles_against_many_columns(ko, m, n, k, b_col_major, tile):
+    """64 or 128 rows against more columns than compute units have 128-wide tiles for: the ring kernel in several
+    rounds.  The whole output against the oracle, plain and with bias + GELU, bit-stable."""
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout) == (1, 0, tile)
+    A = _bits16((m, k), 401 + m, False)
+    B = _bits16((n, k) if b_col_major else (k, n), 403, False)
+    bias = _bits16((n,), 405, False)
+    _, ref64, ap = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major)
+    got = ko.gemm16_host(A, B, m, n, k, b_layout=layout)
+    assert_gemm16_close(_to_f64(got, False), ref64, ap, k)
+    np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, b_layout=layout), got)
+    _, ref64b, apb = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bias_bits=bias, act=1)
+    got = ko.gemm16_host(A, B, m, n, k, bias_bits=bias, act=1, b_layout=layout)
+    assert_gemm16_act_close(_to_f64(got, False), ref64b, apb + 2.0, k)
