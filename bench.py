@@ -778,7 +778,7 @@ def _compact(res):
     return out
 
 
-def headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize=None):
+def headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize=None, deep_k=None):
     """The record: one JSON object of at most MAX_LINE_BYTES characters, printed as the last line of stdout.  It
     carries the headline workload in full (roofline, CPU baseline, parity) and six numbers for each of the other
     configurations; everything else goes to gpurun_out/bench_workloads.json and to earlier lines."""
@@ -812,9 +812,13 @@ def headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize=
     if midsize is not None:  # the 16-bit GEMM on 77 mid-size shapes next to hipBLASLt (rows in the details file)
         line["gemm16_midsize"] = {"shapes": midsize["shapes"], "median_vs_hipblaslt": _sig(midsize["median_vs_hipblaslt"]),
                                   "min_vs_hipblaslt": _sig(midsize["min_vs_hipblaslt"])}
+    if deep_k is not None:  # and on weight-gradient and decoding shapes
+        line["gemm16_deep_k"] = {"shapes": deep_k["shapes"], "median_vs_hipblaslt": _sig(deep_k["median_vs_hipblaslt"]),
+                                 "min_vs_hipblaslt": _sig(deep_k["min_vs_hipblaslt"])}
     line["details_file"] = "gpurun_out/bench_workloads.json"
     # never let the record outgrow what a reader of the last line keeps: shed the optional parts first
-    for key in ("details_file", "copy_ceiling_frac", "copy_same_bytes_us", "max_abs_diff_vs_hipblaslt", "gemm16_midsize"):
+    for key in ("details_file", "copy_ceiling_frac", "copy_same_bytes_us", "max_abs_diff_vs_hipblaslt", "gemm16_deep_k",
+                "gemm16_midsize"):
         if len(json.dumps(line)) <= MAX_LINE_BYTES:
             break
         line.pop(key, None)
@@ -825,13 +829,15 @@ def headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize=
 
 
 
-def emit_record(head, cpu, parity, others, copy, ceilings, info, steps, warmup, out_dir=None, midsize=None):
+def emit_record(head, cpu, parity, others, copy, ceilings, info, steps, warmup, out_dir=None, midsize=None, deep_k=None):
     """Writes everything that was measured to <out_dir>/bench_workloads.json, prints one short line per secondary
     workload, and prints the record as the LAST line of stdout."""
-    line = headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize)
+    line = headline_line(head, cpu, parity, others, copy, info, steps, warmup, midsize, deep_k)
     details = dict(line)
     if midsize is not None:
         details["gemm16_midsize"] = midsize
+    if deep_k is not None:
+        details["gemm16_deep_k"] = deep_k
     details["copy_ceiling"] = None if copy is None else {
         "GB/s": copy["roofline"]["achieved"], "frac_of_peak": copy["roofline"]["frac"], "workload": copy["workload"],
         "independent_sources": ceilings}
@@ -930,7 +936,7 @@ def main():
     others = []
     copy = None
     ceilings = None
-    midsize = None
+    midsize = deep_k = None
     if args.all:
         copy = bench_copy(args.steps, args.warmup)
         ceilings = bench_ceilings(min(args.steps, 10), 3)
@@ -1014,9 +1020,10 @@ def main():
         # sides; about ten seconds): the summary goes into the record, the rows into the details file
         if vendor is not None:
             midsize = bench_gemm16_midsize(min(args.steps, 30), 100, vendor)
+            deep_k = bench_gemm16_deep_k(min(args.steps, 30), 60, vendor)
 
         head, cpu, parity = headline()
-    emit_record(head, cpu, parity, others, copy, ceilings, info, args.steps, args.warmup, midsize=midsize)
+    emit_record(head, cpu, parity, others, copy, ceilings, info, args.steps, args.warmup, midsize=midsize, deep_k=deep_k)
 
 
 if __name__ == "__main__":

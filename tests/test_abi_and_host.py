@@ -245,8 +245,10 @@ def test_bench_record_is_one_short_last_line(tmp_path, capsys):
     copy = _canned_result("copy_f32_1024MiB")
     midsize = dict(shapes=77, median_vs_hipblaslt=0.89973, min_vs_hipblaslt=0.65537, max_vs_hipblaslt=1.18,
                    rows=[dict(m=100, n=1024, k=1024, us=4.4)] * 77)
+    deep_k = dict(shapes=21, median_vs_hipblaslt=0.84512, min_vs_hipblaslt=0.75311, max_vs_hipblaslt=0.95,
+                  rows=[dict(m=768, n=3072, k=16384, us=96.0)] * 21)
     line = bench.emit_record(head, cpu, parity, others, copy, {"rows": list(range(1000))}, info, 20, 5,
-                             out_dir=str(tmp_path), midsize=midsize)
+                             out_dir=str(tmp_path), midsize=midsize, deep_k=deep_k)
     out = capsys.readouterr().out.rstrip("\n").split("\n")
     assert len(out) == len(others) + 1
     last = out[-1]
@@ -258,6 +260,8 @@ def test_bench_record_is_one_short_last_line(tmp_path, capsys):
         assert key in rec, key
     assert rec["gemm16_midsize"] == dict(shapes=77, median_vs_hipblaslt=0.8997, min_vs_hipblaslt=0.6554)
     assert len(json.load(open(tmp_path / "bench_workloads.json"))["gemm16_midsize"]["rows"]) == 77
+    assert rec["gemm16_deep_k"] == dict(shapes=21, median_vs_hipblaslt=0.8451, min_vs_hipblaslt=0.7531)
+    assert len(json.load(open(tmp_path / "bench_workloads.json"))["gemm16_deep_k"]["rows"]) == 21
     assert rec["config"]["workload"] == "masked_softmax_f32_786432x512" and "model" not in rec["config"]
     assert set(rec["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"}
     assert rec["roofline"]["frac"] <= 1.0
