@@ -2111,12 +2111,17 @@ SlicePlan16 plan_k_slices16(const Params &p, size_t workspace_bytes) {
         // kernel, one workgroup per compute unit: 1024 x 512 x 32768 two slices of 64 x 64 tiles 123 us, eight of
         // 128 x 128 57 (hipBLASLt 50); 512 x 512 x 32768 64 -> 39 (32), 512 x 1024 x 16384 52 -> 36 (27), 256 x 1024 x 16384
         // 30 -> 23 (19); 256 x 256 x 16384, four such tiles, stays on 16 slices of 64 x 64: 14.7 us)
-        // (a K beyond what the ring kernel takes whole: slices at least 2048 deep, 3072 from half a million outputs on - the
-        // partial products cost what more workgroups gain: 768 x 768 x 16384 7 slices 39.3 us, 5 37.6; 512 x 1024 x 16384
+        // (the partial products cost what more workgroups gain: 768 x 768 x 16384 7 slices 39.3 us, 5 37.6; 512 x 1024 x 16384
         // 8 33.4, 5 31.6; 256 x 1024 x 16384 16 27.3, 8 22.9; 512 x 768 x 12288 10 27.7, 6 23.4)
-        const int64_t min128 = p.K <= 8192 ? 512 : static_cast<int64_t>(p.M) * p.N >= 512 * 1024 ? 3072 : 2048;
-        const int64_t s128 = capped(cu / t128, min128), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
-        if (s64 >= 2 && s64 * t64 >= s128 * t128 && (p.K <= 8192 ? 4 * s128 * t128 < 3 * cu : 2 * s128 * t128 < cu)) set(s64, 64);
+        // Measured on the ring kernel's tiles, us by slices: 768 x 768 x 8192 4: 23.3, 5: 28.4, 8: 31.6; 1412 x 440 x 8952
+        // 2: 43.5, 4: 31.3, 5: 33.1; 1856 x 320 x 6144 3: 21.7, 4: 22.6, 6: 30.1; 1024 x 512 x 32768 6: 64.8, 8: 56.7.  So:
+        // three quarters of the compute units' worth of workgroups - all of them when the slices are still 4096 deep -
+        // in slices at least 2048 deep, or a quarter of K while K is at most 8192 (and 1024).
+        const int64_t s_fill = cu / t128, s_most = (3 * cu + 2 * t128) / (4 * t128);
+        const int64_t quarter = p.K / 4 > 1024 ? p.K / 4 : 1024;
+        const int64_t min128 = p.K <= 8192 ? quarter : 2048;
+        const int64_t s128 = capped(p.K / s_fill >= 4096 ? s_fill : s_most, min128), s64 = t64 <= cu ? capped(cu / t64, 512) : 1;
+        if (s64 >= 2 && s64 * t64 >= s128 * t128 && 2 * s128 * t128 < cu) set(s64, 64);
         else set(s128, 128);
     } else if (t128 <= cu) {
         set(capped(2 * cu / t128, 2048), 128);
@@ -2166,8 +2171,12 @@ int wave_k_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     const int64_t cu = compute_units();
     const int64_t m32 = (m + 31) / 32, m64 = (m + 63) / 64, n32 = (n + 31) / 32, n64 = (n + 63) / 64;
     if (m32 * n32 <= cu) return k >= 128 ? 32032 : 0;
-    if (m32 * n64 <= cu) return k >= 256 ? 32064 : 0;
-    if (m64 * n64 <= cu) return k >= 1024 ? 64064 : 0;
+    // (the larger tiles up to a K where K slices of the ring kernel's 128 x 128 tiles take over: 1856 x 320 x 6144 27.1 us
+    // here, 21.7 in three slices; 768 x 768 x 8192 28.7 / 23.3; 1536 x 512 x 6144 29.1 / 22.4; 2048 x 256 x 8192 on 32 x 64
+    // tiles 24.4 / 21.0; at K = 4096 level - 768 x 768 16.7 / 16.8, 1024 x 1024 18.5 / 22.8)
+    if (m32 * n64 <= cu) return k >= 256 && k < 8192 ? 32064 : 0;
+    // (with at most three quarters of the compute units' worth of tiles from K = 5120 on: 1868 x 303 x 5720 34.3 / 23.6)
+    if (m64 * n64 <= cu) return k >= 1024 && k < (4 * m64 * n64 <= 3 * cu ? 5120 : 6144) ? 64064 : 0;
     return 0;
 }
 

@@ -94,6 +94,15 @@ def test_measured_decisions_stay_put():
     assert ko.gemm_plan(100, 1024, 1024, sixteen_bit=True) == (1, 0, 32032)
     assert ko.gemm_plan(512, 1024, 4096, sixteen_bit=True) == (1, 0, 32064)
     assert ko.gemm_plan(1000, 1024, 4096, sixteen_bit=True) == (1, 0, 64064)
+    # ... up to a K where K slices of the ring kernel's 128 x 128 tiles are faster: at most three quarters of the compute
+    # units' worth of workgroups, slices a quarter of K deep or more
+    assert ko.gemm_plan(768, 768, 8192, sixteen_bit=True) == (4, 2048, 128)
+    assert ko.gemm_plan(1856, 320, 6144, sixteen_bit=True) == (4, 1536, 128)
+    assert ko.gemm_plan(1868, 303, 5720, sixteen_bit=True)[0] == 4       # 150 tiles of 64 x 64: sliced from K = 5120 on
+    assert ko.gemm_plan(1024, 1024, 5720, sixteen_bit=True) == (1, 0, 64064)   # 256 of them: from 6144 on
+    assert ko.gemm_plan(2048, 256, 8192, sixteen_bit=True) == (4, 2048, 128)
+    assert ko.gemm_plan(1412, 440, 8952, sixteen_bit=True) == (4, 2240, 128)
+    assert ko.gemm_plan(1024, 512, 32768, sixteen_bit=True) == (8, 4096, 128)
     # too many small tiles for that, at most one tile of 128 x 128 (or half of one) per compute unit: the ring kernel
     assert ko.gemm_plan(2048, 768, 3072, sixteen_bit=True) == (1, 0, 64128)
     assert ko.gemm_plan(512, 4096, 4096, sixteen_bit=True) == (1, 0, 128064)
