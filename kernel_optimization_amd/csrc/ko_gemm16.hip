@@ -2209,7 +2209,10 @@ int ring_tile(int64_t m, int64_t n, int64_t k, bool b_row_major) {
     // 237 -> 177 (151), 8 x 50304 x 1024 27.2 -> 23.7 (18.5); 32 x 128 tiles with six stages (one workgroup per compute
     // unit) 47.6 / 56.1 / 181 / 24.0, with three 61 / 70 / 190 / 20.7.
     if (m <= 32 && n64 > cu) return 1032064;
-    if (k > 8192) return 0;
+    // (a K beyond 8192 only where neither two slices fit a round nor the pinned kernel's slices apply - more than half
+    // a chip's worth of 128 x 128 tiles, N not whole 256 x 256 tiles: 311 x 7983 x 8216 in two slices of the register
+    // pipeline 111 us, whole here 97; x 12000 143 / 128)
+    if (k > 8192 && !(k <= 16384 && n % 256 != 0 && m128 * n128 <= cu && 2 * m128 * n128 > cu)) return 0;
     // One row of tiles against more columns than compute units (64 or 128 rows against a vocabulary): this kernel in
     // several rounds, where the persistent kernels' 256 x 256 tiles are mostly rows that do not exist
     // (64 x 128256 x 4096 258 -> 187 us (hipBLASLt 174), 128 x 128256 x 4096 274 -> 215 (204), 64 x 50304 x 1024 31.8 -> 27.8
@@ -2392,6 +2395,11 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
             // 128 x 128 tiles 16.3 us).
             const int64_t want = static_cast<int64_t>(compute_units()) * 3 / 2;
             const int64_t tm128 = (p.M + 127) / 128, tn128 = (p.N + 127) / 128, tn64 = (p.N + 63) / 64;
+            // up to one and a half rounds of 128 x 128 tiles: the ring kernel in two rounds still beats the register
+            // pipeline (657 x 7834 x 1544, 372 tiles: 49.2 -> 43.1 us; hipBLASLt 28.0)
+            if (tm128 * tn128 > compute_units() && 2 * tm128 * tn128 <= 3 * compute_units() && p.K >= 512 && p.K <= 16384 &&
+                tuning(knob_gemm16_wave_k) != 1 && (!B_ROW_MAJOR || (p.N % 8 == 0 && p.ldb % 8 == 0)))
+                return launch_ring<128, 128, 2, 2, 4, BF16, B_ROW_MAJOR>(p, stream);
             // from one 128 x 128 tile per compute unit on when K is deep: the longer main loop then outweighs the
             // idle second slot (2048^3: 30.1 us against 31.3 with 128 x 64 tiles; 4096 x 1024 x 4096: 50.9 against 53.0)
             if (tm128 * tn128 >= want || (tm128 * tn128 >= compute_units() && p.K >= 2048))

@@ -66,7 +66,9 @@ def test_gemm16_plans_cover_k_once_and_fit_the_workspace(m, n, b_layout):
                 assert (b_layout == ko.COL_MAJOR or n % 8 == 0) and 128 <= k <= 8192
                 assert plan[2] == 32032 or -(-m // 32) * -(-n // 32) > 256
             else:                                   # a deep ring of LDS stages: when the small tiles are too many
-                assert (b_layout == ko.COL_MAJOR or (n % 8 == 0 and plan[2] != 64128)) and 512 <= k <= 8192
+                assert (b_layout == ko.COL_MAJOR or (n % 8 == 0 and plan[2] != 64128)) and 512 <= k <= 16384
+                if k > 8192:   # only where two slices do not fit a round and the pinned kernel's slices do not apply
+                    assert plan[2] == 128128 and n % 256 != 0 and 2 * -(-m // 128) * -(-n // 128) > 256
                 assert -(-m // 64) * -(-n // 64) > 256
                 if -(-m // tm) * -(-n // tn) > 256:
                     assert (plan[2] == 64128 and b_layout == ko.COL_MAJOR) or (plan[2] == 128128 and k >= 2048)

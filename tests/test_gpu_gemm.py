@@ -1213,3 +1213,20 @@ def test_gemm16_one_row_of_tiles_against_many_columns(ko, m, n, k, b_col_major, 
     _, ref64b, apb = oracle.gemm16(A, B, m, n, k, b_col_major=b_col_major, bias_bits=bias, act=1)
     got = ko.gemm16_host(A, B, m, n, k, bias_bits=bias, act=1, b_layout=layout)
     assert_gemm16_act_close(_to_f64(got, False), ref64b, apb + 2.0, k)
+
+
+@pytest.mark.parametrize("m,n,k,b_col_major,tile", [(657, 7834, 520, True, 0), (640, 7840, 776, False, 0),
+                                                    (311, 7983, 8200, True, 128128), (300, 7984, 8456, False, 128128)])
+def test_gemm16_ring_kernel_beyond_one_round_and_beyond_k_8192(ko, m, n, k, b_col_major, tile):
+    """Up to one and a half rounds of 128 x 128 tiles on a shape that is not whole 256 x 256 tiles (the plan query says 0:
+    the choice falls in the later rules of the dispatch), and more than half a round of them at a K beyond 8192:
+    sampled rows (every column) against the oracle, and bit-stable."""
+    layout = ko.COL_MAJOR if b_col_major else ko.ROW_MAJOR
+    assert ko.gemm_plan(m, n, k, sixteen_bit=True, b_layout=layout) == (1, 0, tile)
+    A = _bits16((m, k), 501, False)
+    B = _bits16((n, k) if b_col_major else (k, n), 503, False)
+    got = ko.gemm16_host(A, B, m, n, k, b_layout=layout)
+    rows = np.unique(np.concatenate([np.arange(0, m, 29), [127, 128, m - 1]]))
+    _, ref64, ap = oracle.gemm16(A[rows], B, len(rows), n, k, b_col_major=b_col_major)
+    assert_gemm16_close(_to_f64(got[rows], False), ref64, ap, k)
+    np.testing.assert_array_equal(ko.gemm16_host(A, B, m, n, k, b_layout=layout), got)
