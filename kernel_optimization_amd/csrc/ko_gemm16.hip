@@ -215,6 +215,10 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
     const float alpha = p.alpha;
     const bool use_c = p.C != nullptr && p.beta != 0.0f;
     const bool plain = !use_c && p.bias == nullptr && p.act == KO_ACT_NONE;  // D = alpha * acc
+    // rows of D that start on 64-byte boundaries: a wave's row segments are whole 64-byte sectors then, and streaming
+    // stores pay; off them the segments end inside sectors that a neighbour's store completes, and the L2 should get
+    // the chance to put the two together
+    const bool whole_sectors = (ldd & 31) == 0;
 
     if (!EDGE) {
         // Full tiles: each wave transposes its own tile through LDS (free now: the last
@@ -293,7 +297,10 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 const int gn = col0 + c * 8;
                 // streaming store: D is written once and not read again by this kernel (`sc1 nt`, which helps the
                 // row kernels, measured no different here: 74.3 against 73.8 us)
-                if (!GUARD_M || gm < M) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
+                if (!GUARD_M || gm < M) {
+                    if (whole_sectors) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
+                    else *reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn) = v;
+                }
             }
         }
         return;
@@ -2420,6 +2427,8 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 11: return launch<TileTiny, BF16, B_ROW_MAJOR>(p, stream);
         case 12: return launch<TileSmallN, BF16, B_ROW_MAJOR>(p, stream);
         case 13: return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
+        case 14: return launch<Tiling<128, 128, 2, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);  // one register stage: 32 KB of LDS
+        case 15: return launch<Tiling<64, 64, 2, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
         case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);
