@@ -2427,8 +2427,6 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
         case 11: return launch<TileTiny, BF16, B_ROW_MAJOR>(p, stream);
         case 12: return launch<TileSmallN, BF16, B_ROW_MAJOR>(p, stream);
         case 13: return launch<TileSkinny, BF16, B_ROW_MAJOR>(p, stream);
-        case 14: return launch<Tiling<128, 128, 2, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);  // one register stage: 32 KB of LDS
-        case 15: return launch<Tiling<64, 64, 2, 2, 1, true, 1>, BF16, B_ROW_MAJOR>(p, stream);
         case 30: return launch_direct<TileBig, BF16, B_ROW_MAJOR, false>(p, stream);
         case 50: return launch_direct<TileBig, BF16, B_ROW_MAJOR, true>(p, stream);
         case 52: return launch_direct<TileBigSpare, BF16, B_ROW_MAJOR, true>(p, stream);

@@ -153,6 +153,10 @@ __device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc
     // acc[i][j][r] is D[m][n] with m = 8*(r/4) + 4*(lane/32) + r%4, n = lane%32 inside
     // the 32x32 tile: for a fixed r the 32 lanes of a half-wave write 128 contiguous bytes.
     const float alpha = p.alpha, beta = p.beta;
+    // streaming stores while rows of D start on 64-byte boundaries (a half-wave's 128 bytes are two whole sectors then);
+    // off them the ends of a row segment share their sectors with a neighbour's, and go through the L2 to meet there
+    // (4096 x 4072 x 128: 60.5 us streamed, against 54.4 at N = 4064)
+    const bool whole_sectors = (N & 15) == 0;
     // The choice between "with C" and "without" is made once, not per element, and the 32 x 32 sub-tiles
     // are written one after the other (the addresses of all of them at once would not fit the registers).
     auto store_all = [&](auto with_c) {
@@ -169,7 +173,8 @@ __device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc
                         const int64_t off = static_cast<int64_t>(m) * N + n;
                         float v = alpha * acc[i][j][r];
                         if constexpr (decltype(with_c)::value) v += beta * p.C[off];
-                        __builtin_nontemporal_store(v, &p.D[off]);
+                        if (whole_sectors) __builtin_nontemporal_store(v, &p.D[off]);
+                        else p.D[off] = v;
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
