@@ -205,9 +205,10 @@ __device__ __forceinline__ void tile_of(const Params &p, int b, int grid, int t,
 // (the caller has loads in flight that it wants confirmed while they are still the only ones outstanding).
 // GUARD_M (full-tile form): the tile may reach past row M - rows at or past M hold the products of rows fetched from
 // elsewhere in A: they take no C and are not stored.
-template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1, bool WAIT_VM = false, bool GUARD_M = false>
-__device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
-                                           int lane, int row0, int col0) {
+// STREAM (full-tile form): the stores are streaming (non-temporal) ones - see store_tile below, which chooses.
+template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS, bool WAIT_VM, bool GUARD_M, bool STREAM>
+__device__ __forceinline__ void store_tile_as(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
+                                              int lane, int row0, int col0) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     const int M = p.M, N = p.N;
     const int64_t ldd = p.ldd;
@@ -215,10 +216,6 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
     const float alpha = p.alpha;
     const bool use_c = p.C != nullptr && p.beta != 0.0f;
     const bool plain = !use_c && p.bias == nullptr && p.act == KO_ACT_NONE;  // D = alpha * acc
-    // rows of D that start on 64-byte boundaries: a wave's row segments are whole 64-byte sectors then, and streaming
-    // stores pay; off them the segments end inside sectors that a neighbour's store completes, and the L2 should get
-    // the chance to put the two together
-    const bool whole_sectors = (ldd & 31) == 0;
 
     if (!EDGE) {
         // Full tiles: each wave transposes its own tile through LDS (free now: the last
@@ -295,10 +292,8 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
                 if (erow(row) & 1) v = u32x4{v[2], v[3], v[0], v[1]};
                 const int gm = row0 + part * PROWS + row;
                 const int gn = col0 + c * 8;
-                // streaming store: D is written once and not read again by this kernel (`sc1 nt`, which helps the
-                // row kernels, measured no different here: 74.3 against 73.8 us)
                 if (!GUARD_M || gm < M) {
-                    if (whole_sectors) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
+                    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn));
                     else *reinterpret_cast<u32x4_rows *>(p.D + gm * ldd + gn) = v;
                 }
             }
@@ -343,6 +338,23 @@ __device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM 
             }
         }
     }
+}
+
+// The epilogue with the kind of store that the rows of D ask for, chosen once per tile (the two forms are two copies of
+// the code: a choice per store inside the loop cost the 16384 x 3072 x 768 problem 6 us - and the persistent kernels,
+// whose tiles are whole 256-column ones of rows that as a rule start on such boundaries, keep the one streaming copy).  D is written once and not read
+// again, and while its rows start on 64-byte boundaries a wave's 128-byte row segments are whole sectors and streaming
+// (non-temporal) stores are the faster ones (that problem, on operand sets that rotate through more than the caches
+// hold: 77 us against 85 with plain stores).  Off such boundaries the segments end inside sectors that a neighbouring
+// wave or tile completes; streamed out, each part goes to memory on its own, and the kernel takes a third longer
+// (4096 x 11928 x 64: 44.1 us, with plain stores - which meet in the L2 - 35.0; 9329 x 4948 x 32 44.3 / 34.6).
+template <int WTM, int WTN, int SWIZZLE, bool BF16, bool EDGE, int PARTS = 1, bool WAIT_VM = false, bool GUARD_M = false>
+__device__ __forceinline__ void store_tile(const Params &p, float16v (&acc)[WTM / 32][WTN / 32], u32x4 *region,
+                                           int lane, int row0, int col0) {
+    if (EDGE || (p.ldd & 31) == 0)
+        store_tile_as<WTM, WTN, SWIZZLE, BF16, EDGE, PARTS, WAIT_VM, GUARD_M, true>(p, acc, region, lane, row0, col0);
+    else
+        store_tile_as<WTM, WTN, SWIZZLE, BF16, EDGE, PARTS, WAIT_VM, GUARD_M, false>(p, acc, region, lane, row0, col0);
 }
 
 // Tiling of one kernel instantiation.
@@ -846,7 +858,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_persistent_kernel(const Par
             int m0, n0;
             tile_origin(t, m0, n0);
             // stage `cur` is free (every wave is past the barrier); stage cur^1 holds the next tile's first K tile
-            store_tile<WTM, WTN, SWIZZLE, BF16, false, EPI_PARTS>(
+            store_tile_as<WTM, WTN, SWIZZLE, BF16, false, EPI_PARTS, false, false, true>(
                 p, acc, lds + cur * STAGE + wave * (WTM * WTN / 8 / EPI_PARTS), lane, m0 + wm * WTM, n0 + wn * WTN);
             clear_acc();
             lds_barrier();  // the next step loads into stage `cur`
@@ -1255,7 +1267,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
             } else if constexpr (SPARE) {
                 constexpr int REGION = WTM * WTN * 2 / 4;  // bytes per wave and pass
                 char *region = lds_bytes + 2 * (A_BYTES + B_BYTES) + wave * REGION;
-                store_tile<WTM, WTN, 1, BF16, false, 4, true, EDGE_M>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                store_tile_as<WTM, WTN, 1, BF16, false, 4, true, EDGE_M, true>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
                                                                       m0 + wm * WTM, n0 + wn * WTN);
                 clear_acc();
                 stores_in_flight = true;
@@ -1264,7 +1276,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm16_pinned_kernel(const Params 
                 static_assert(REGION * (WAVES / 2) <= A_BYTES && REGION * (WAVES / 2) <= B_BYTES, "");
                 char *region = wave < WAVES / 2 ? lds_bytes + S * A_BYTES + wave * REGION
                                                 : lds_bytes + 2 * A_BYTES + S * B_BYTES + (wave - WAVES / 2) * REGION;
-                store_tile<WTM, WTN, 1, BF16, false, EPI_PARTS, false, EDGE_M>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
+                store_tile_as<WTM, WTN, 1, BF16, false, EPI_PARTS, false, EDGE_M, true>(p, acc, reinterpret_cast<u32x4 *>(region), lane,
                                                                                m0 + wm * WTM, n0 + wn * WTN);
                 clear_acc();
                 lds_barrier();  // every wave is done with its transpose region in stage S

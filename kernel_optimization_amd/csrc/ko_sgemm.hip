@@ -159,7 +159,7 @@ __device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc
     const bool whole_sectors = (N & 15) == 0;
     // The choice between "with C" and "without" is made once, not per element, and the 32 x 32 sub-tiles
     // are written one after the other (the addresses of all of them at once would not fit the registers).
-    auto store_all = [&](auto with_c) {
+    auto store_all = [&](auto with_c, auto streaming) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -173,7 +173,7 @@ __device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc
                         const int64_t off = static_cast<int64_t>(m) * N + n;
                         float v = alpha * acc[i][j][r];
                         if constexpr (decltype(with_c)::value) v += beta * p.C[off];
-                        if (whole_sectors) __builtin_nontemporal_store(v, &p.D[off]);
+                        if constexpr (decltype(streaming)::value) __builtin_nontemporal_store(v, &p.D[off]);
                         else p.D[off] = v;
                     }
                 }
@@ -181,8 +181,13 @@ __device__ __forceinline__ void reduce_and_store(const Params &p, float16v (&acc
             }
         }
     };
-    if (p.C != nullptr && beta != 0.0f) store_all(std::true_type{});
-    else store_all(std::false_type{});
+    if (p.C != nullptr && beta != 0.0f) {
+        if (whole_sectors) store_all(std::true_type{}, std::true_type{});
+        else store_all(std::true_type{}, std::false_type{});
+    } else {
+        if (whole_sectors) store_all(std::false_type{}, std::true_type{});
+        else store_all(std::false_type{}, std::false_type{});
+    }
 }
 
 // VEC: K % 4 == 0, N % 4 == 0 and 16-byte aligned A and B (128-bit global loads);
