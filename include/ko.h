@@ -114,8 +114,10 @@ int ko_event_destroy(ko_event_t event);
  * row r belongs to sequence r / rows_per_seq and every column
  * j >= valid_len[seq] takes the value -10000 before the softmax.
  * Workspace: a few long rows (fewer rows than a quarter of the compute units, 256 KB and more each) run as two
- * launches that pass partial results through the (device, stream) workspace described at ko_sgemm_f32; the same
- * holds for ko_layernorm_f32 and the 16-bit forms.  Without a workspace (first such call inside a graph capture)
+ * launches that pass partial results through 1 MiB of device memory that belongs to the (device, stream) pair -
+ * an allocation of its own next to the GEMMs' workspace described at ko_sgemm_f32, made at the first such call,
+ * kept and released the same way, under the same rules for graphs; the same holds for ko_layernorm_f32 and the
+ * 16-bit forms.  Without a workspace (first such call inside a graph capture)
  * they run as one launch, one workgroup per row. */
 int ko_softmax_f32(const float *in, float *out, int64_t rows, int64_t cols,
                    const int32_t *valid_len, int64_t rows_per_seq, ko_stream_t stream);

@@ -79,6 +79,10 @@ constexpr size_t kStreamWorkspaceBytes = size_t{64} << 20;
 // entry point that allocates nothing, so that both entry points plan, and sum, the same slices.
 constexpr size_t kSgemmPartialBytes = size_t{32} << 20;
 int stream_workspace(hipStream_t stream, void **workspace);
+// The same for the row operators, which pass a few kilobytes of per-piece statistics: a small allocation of the pair's
+// own (kStreamSmallWorkspaceBytes), made, kept and released like the large one and independent of it.
+constexpr size_t kStreamSmallWorkspaceBytes = size_t{1} << 20;
+int stream_small_workspace(hipStream_t stream, void **workspace);
 // Frees the workspace of (current device, stream), if it has one.  The caller has synchronised the stream.
 int release_stream_workspace(hipStream_t stream);
 // How many (device, stream) pairs hold a workspace right now.

@@ -1164,8 +1164,8 @@ int launch_pieces(const Args<IO> &a) {
     piece = (piece + THREADS - 1) / THREADS * THREADS;  // whole trips of the workgroup; the last piece is the short one
     parts = (nvec + piece - 1) / piece;
     void *workspace = nullptr;
-    if (const int st = stream_workspace(a.stream, &workspace); st != KO_OK) return st;
-    if (workspace == nullptr || static_cast<size_t>(a.rows) * (parts * sizeof(wave::Welford) + sizeof(float)) > kStreamWorkspaceBytes)
+    if (const int st = stream_small_workspace(a.stream, &workspace); st != KO_OK) return st;
+    if (workspace == nullptr || static_cast<size_t>(a.rows) * (parts * sizeof(wave::Welford) + sizeof(float)) > kStreamSmallWorkspaceBytes)
         return -1;
     wave::Welford *triplets = static_cast<wave::Welford *>(workspace);
     const dim3 grid(static_cast<unsigned>(parts), static_cast<unsigned>(a.rows));

@@ -68,26 +68,31 @@ int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &d
 }
 
 namespace {
-struct WorkspaceEntry { int device; hipStream_t stream; void *memory; };
+// what a (device, stream) pair holds: the GEMMs' workspace, the row operators' small one, or both
+struct WorkspaceEntry { int device; hipStream_t stream; void *memory; void *small; };
 constexpr int kMaxWorkspaces = 64;
 WorkspaceEntry g_workspaces[kMaxWorkspaces];
 int g_workspaces_used = 0;
 std::mutex g_workspaces_lock;
 }  // namespace
 
-int stream_workspace(hipStream_t stream, void **workspace) {
+namespace {
+// The pair's workspace of the asked kind, allocated if it has none yet and nothing forbids it.
+int workspace_of(hipStream_t stream, bool small, void **workspace) {
     *workspace = nullptr;
     // one handle value stands for a different stream in every host thread: no workspace can belong to it
     if (stream == hipStreamPerThread) return KO_OK;
     int dev = 0;
     KO_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> guard(g_workspaces_lock);
+    int at = -1;
     for (int i = 0; i < g_workspaces_used; ++i)
-        if (g_workspaces[i].device == dev && g_workspaces[i].stream == stream) {
-            *workspace = g_workspaces[i].memory;
-            return KO_OK;
-        }
-    if (g_workspaces_used == kMaxWorkspaces) return KO_OK;
+        if (g_workspaces[i].device == dev && g_workspaces[i].stream == stream) at = i;
+    if (at >= 0 && (small ? g_workspaces[at].small : g_workspaces[at].memory) != nullptr) {
+        *workspace = small ? g_workspaces[at].small : g_workspaces[at].memory;
+        return KO_OK;
+    }
+    if (at < 0 && g_workspaces_used == kMaxWorkspaces) return KO_OK;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
         (void)hipGetLastError();
@@ -97,29 +102,39 @@ int stream_workspace(hipStream_t stream, void **workspace) {
     void *memory = nullptr;
     // no memory, or an allocation is not allowed right now (another stream of the process is being captured):
     // the caller goes without a workspace this time
-    if (hipMalloc(&memory, kStreamWorkspaceBytes) != hipSuccess || memory == nullptr) {
+    if (hipMalloc(&memory, small ? kStreamSmallWorkspaceBytes : kStreamWorkspaceBytes) != hipSuccess || memory == nullptr) {
         (void)hipGetLastError();
         return KO_OK;
     }
-    g_workspaces[g_workspaces_used++] = WorkspaceEntry{dev, stream, memory};
+    if (at < 0) {
+        at = g_workspaces_used++;
+        g_workspaces[at] = WorkspaceEntry{dev, stream, nullptr, nullptr};
+    }
+    (small ? g_workspaces[at].small : g_workspaces[at].memory) = memory;
     *workspace = memory;
     return KO_OK;
 }
+}  // namespace
+
+int stream_workspace(hipStream_t stream, void **workspace) { return workspace_of(stream, false, workspace); }
+int stream_small_workspace(hipStream_t stream, void **workspace) { return workspace_of(stream, true, workspace); }
 
 int release_stream_workspace(hipStream_t stream) {
     int dev = 0;
     KO_HIP(hipGetDevice(&dev));
-    void *memory = nullptr;
+    void *memory = nullptr, *small = nullptr;
     {
         std::lock_guard<std::mutex> guard(g_workspaces_lock);
         for (int i = 0; i < g_workspaces_used; ++i)
             if (g_workspaces[i].device == dev && g_workspaces[i].stream == stream) {
                 memory = g_workspaces[i].memory;
+                small = g_workspaces[i].small;
                 g_workspaces[i] = g_workspaces[--g_workspaces_used];
                 break;
             }
     }
     if (memory != nullptr) KO_HIP(hipFree(memory));
+    if (small != nullptr) KO_HIP(hipFree(small));
     return KO_OK;
 }
 

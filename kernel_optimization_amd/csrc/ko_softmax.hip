@@ -849,8 +849,8 @@ int launch_pieces(const Args<IO> &a) {
     piece = (piece + THREADS - 1) / THREADS * THREADS;  // whole trips of the workgroup; the last piece is the short one
     parts = (nvec + piece - 1) / piece;
     void *workspace = nullptr;
-    if (const int st = stream_workspace(a.stream, &workspace); st != KO_OK) return st;
-    if (workspace == nullptr || static_cast<size_t>(a.rows) * parts * sizeof(PiecePair) > kStreamWorkspaceBytes) return -1;
+    if (const int st = stream_small_workspace(a.stream, &workspace); st != KO_OK) return st;
+    if (workspace == nullptr || static_cast<size_t>(a.rows) * parts * sizeof(PiecePair) > kStreamSmallWorkspaceBytes) return -1;
     PiecePair *pairs = static_cast<PiecePair *>(workspace);
     const dim3 grid(static_cast<unsigned>(parts), static_cast<unsigned>(a.rows));
     softmax_pieces_stats_kernel<IO, THREADS, MASKED><<<grid, dim3(THREADS), 0, a.stream>>>(a.in, a.cols, a.valid_len,

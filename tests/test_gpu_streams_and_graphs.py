@@ -182,7 +182,7 @@ def _workspaces(ko):
 
 
 def test_stream_destroy_releases_the_workspace(ko):
-    """ko_stream_destroy frees the 32 MiB workspace a K-sliced call gave the stream: a process that creates and
+    """ko_stream_destroy frees the workspace a K-sliced call gave the stream: a process that creates and
     destroys more streams than the workspace table has entries (64) keeps the sliced path - same bits as on the
     first stream - and holds no more workspaces afterwards than before."""
     ko.set_tuning("gemm16.wave_k", 1)  # (by default the 16-bit GEMM splits K over the waves of a workgroup here, in one launch)
@@ -227,6 +227,48 @@ def _stream_destroy_releases_the_workspace(ko):
         np.testing.assert_array_equal(got16, first16, err_msg="stream %d" % i)
     ref = A.astype(np.float64) @ B.astype(np.float64)
     assert np.abs(first.view(np.float32) - ref).max() <= 2 * k * 2.0 ** -24 * (np.abs(A) @ np.abs(B)).max()
+
+
+def test_row_operators_hold_a_small_workspace_of_their_own(ko):
+    """A stream that only ever cuts a few long rows into pieces holds 1 MiB, not the GEMMs' 64 MiB: free device memory
+    drops by a few MiB at most on the first such call, by the large workspace when a K-sliced GEMM follows on the
+    same stream (the table still counts one pair), and ko_stream_destroy gives both back."""
+    hip = _hip_runtime()
+    hip.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    rows, cols = 8, 131072
+    x = ko.DeviceBuffer.from_numpy(inputs.normal_f32((rows, cols), 611, 0.0, 4.0))
+    y, z = ko.DeviceBuffer(rows * cols * 4), ko.DeviceBuffer(rows * cols * 4)
+    m, n, k = 256, 256, 2048
+    assert ko.gemm_plan(m, n, k)[0] > 1
+    dA, dB, dD = ko.DeviceBuffer(m * k * 4), ko.DeviceBuffer(k * n * 4), ko.DeviceBuffer(m * n * 4)
+    ko.fill_uniform_f32(dA, m * k, 612)
+    ko.fill_uniform_f32(dB, k * n, 613)
+    ko.softmax(x, y, rows, cols)           # the default stream: the reference result, in pieces as well
+    ko.synchronize()
+    want = y.download(np.uint32, (rows, cols))
+    stream = ko.Stream()
+    ko.synchronize()
+    base, free0 = _workspaces(ko), free_bytes()
+    ko.softmax(x, z, rows, cols, stream=stream)
+    ko.layernorm(z, y, rows, cols, stream=stream)
+    stream.synchronize()
+    assert _workspaces(ko) == base + 1
+    free1 = free_bytes()
+    assert free0 - free1 <= 8 << 20, "the row operators took %d bytes" % (free0 - free1)
+    np.testing.assert_array_equal(z.download(np.uint32, (rows, cols)), want)
+    ko.sgemm(m, n, k, dA, dB, dD, stream=stream)
+    stream.synchronize()
+    assert _workspaces(ko) == base + 1
+    assert free1 - free_bytes() >= 60 << 20
+    stream.close()
+    assert _workspaces(ko) == base
+    assert free_bytes() >= free0 - (1 << 20)
 
 
 def test_operators_from_two_threads_on_two_streams(ko):
