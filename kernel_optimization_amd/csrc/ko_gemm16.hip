@@ -34,6 +34,16 @@
 #include <type_traits>
 #include <utility>
 
+// This file is compiled four times, once per combination of operand type and layout of B - the kernels of one
+// combination take over a minute to compile: by itself for binary16 operands and a column-major B, together with the
+// entry points, and through ko_gemm16_f16_row.hip, ko_gemm16_bf16_col.hip and ko_gemm16_bf16_row.hip, which set the
+// three macros and include it.  Each part defines its gemm16_run<BF16, B_ROW_MAJOR>.
+#ifndef KO_GEMM16_BF16
+#define KO_GEMM16_BF16 0
+#define KO_GEMM16_B_ROW 0
+#define KO_GEMM16_ENTRY 1
+#endif
+
 namespace ko {
 namespace {
 
@@ -113,31 +123,7 @@ __device__ __forceinline__ void lds_barrier() {
 // Orders this wave's earlier LDS writes before its later LDS reads.
 __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-struct Params {
-    const uint16_t *A;
-    const uint16_t *B;
-    const uint16_t *C;
-    uint16_t *D;
-    int M, N, K;
-    float alpha, beta;
-    int tiles_n;
-    int nblocks;
-    int band_rows;              // persistent kernels: > 0 selects the blocked tile order (see tile_of)
-    int block_cols;
-    const uint16_t *bias;       // [N] or null: added to every row before the activation
-    int act;                    // KO_ACT_*
-    int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
-    int ldb;                    // row-major B: elements between its rows (N, or more likewise)
-    // K slices (gemm16_kernel only): workgroups with blockIdx.y = s multiply k in [s * k_slice, (s + 1) * k_slice) and
-    // write their M x N partial product as fp32 (no alpha, C, bias or activation; rows partial_ld(N) floats apart)
-    // behind partial + s * M * partial_ld(N)
-    int k_slice;                // 0: no slices
-    float *partial;
-    int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
-    int tiles;                  // gemm16_pinned_kernel with K slices: output tiles (nblocks = tiles * slices)
-    int xcd_cols_log2;          // blocked tile order: the 8 XCDs' regions lie 2^this side by side (0: one below the other)
-    int region_cols;            //                     columns of tiles in a region (unused when they lie one below the other)
-};
+using Params = Gemm16Params;  // (ko_internal.h: the four parts this file is compiled into share it)
 
 // x/2 (1 + tanh u) = x / (1 + exp(-2u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written as
 // x * rcp(1 + 2^(x (c1 + c2 x^2))), c1 = -2 sqrt(2/pi) log2(e), c2 = 0.044715 c1: two multiplies, one FMA,
@@ -2470,8 +2456,14 @@ int launch_variant(const Params &p, hipStream_t stream, bool col_cut = true, int
 }
 
 }  // namespace
+
+template <>
+int gemm16_run<KO_GEMM16_BF16 != 0, KO_GEMM16_B_ROW != 0>(const Gemm16Params &p, hipStream_t stream) {
+    return launch_variant<KO_GEMM16_BF16 != 0, KO_GEMM16_B_ROW != 0>(p, stream);
+}
 }  // namespace ko
 
+#if KO_GEMM16_ENTRY
 KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
                                          const void *B, int b_layout, float beta, const void *C, const void *bias,
                                          int activation, void *D, int in_dtype, ko_stream_t stream) {
@@ -2507,9 +2499,8 @@ KO_EXPORT int ko_gemm_f16f32acc_bias_act(int64_t m, int64_t n, int64_t k, float 
         KO_CHECK_LAUNCH();
         return KO_OK;
     }
-    if (in_dtype == KO_F16)
-        return b_layout == KO_COL_MAJOR ? launch_variant<false, false>(p, s) : launch_variant<false, true>(p, s);
-    return b_layout == KO_COL_MAJOR ? launch_variant<true, false>(p, s) : launch_variant<true, true>(p, s);
+    if (in_dtype == KO_F16) return b_layout == KO_COL_MAJOR ? gemm16_run<false, false>(p, s) : gemm16_run<false, true>(p, s);
+    return b_layout == KO_COL_MAJOR ? gemm16_run<true, false>(p, s) : gemm16_run<true, true>(p, s);
 }
 
 KO_EXPORT int ko_gemm_f16f32acc(int64_t m, int64_t n, int64_t k, float alpha, const void *A,
@@ -2549,3 +2540,4 @@ int ko::debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *sl
     *tile = plan.slices > 1 ? plan.tile : 0;
     return KO_OK;
 }
+#endif  // KO_GEMM16_ENTRY

@@ -88,6 +88,41 @@ int release_stream_workspace(hipStream_t stream);
 // How many (device, stream) pairs hold a workspace right now.
 int stream_workspace_count();
 
+// The 16-bit GEMM's problem as its kernels take it (csrc/ko_gemm16.hip, compiled in four parts).
+struct Gemm16Params {
+    const uint16_t *A;
+    const uint16_t *B;
+    const uint16_t *C;
+    uint16_t *D;
+    int M, N, K;
+    float alpha, beta;
+    int tiles_n;
+    int nblocks;
+    int band_rows;              // persistent kernels: > 0 selects the blocked tile order (see tile_of)
+    int block_cols;
+    const uint16_t *bias;       // [N] or null: added to every row before the activation
+    int act;                    // KO_ACT_*
+    int ldd;                    // elements between rows of C and D (N, or more when they are a column range of a wider matrix)
+    int ldb;                    // row-major B: elements between its rows (N, or more likewise)
+    // K slices (gemm16_kernel only): workgroups with blockIdx.y = s multiply k in [s * k_slice, (s + 1) * k_slice) and
+    // write their M x N partial product as fp32 (no alpha, C, bias or activation; rows partial_ld(N) floats apart)
+    // behind partial + s * M * partial_ld(N)
+    int k_slice;                // 0: no slices
+    float *partial;
+    int ldk;                    // gemm16_kernel: elements between rows of A and of a column-major B (K of the whole problem)
+    int tiles;                  // gemm16_pinned_kernel with K slices: output tiles (nblocks = tiles * slices)
+    int xcd_cols_log2;          // blocked tile order: the 8 XCDs' regions lie 2^this side by side (0: one below the other)
+    int region_cols;            //                     columns of tiles in a region (unused when they lie one below the other)
+};
+// One call of the 16-bit GEMM on operands of one type and one layout of B: defined by the part of ko_gemm16.hip that
+// is compiled for that combination.
+template <bool BF16, bool B_ROW_MAJOR>
+int gemm16_run(const Gemm16Params &p, hipStream_t stream);
+template <> int gemm16_run<false, false>(const Gemm16Params &p, hipStream_t stream);
+template <> int gemm16_run<false, true>(const Gemm16Params &p, hipStream_t stream);
+template <> int gemm16_run<true, false>(const Gemm16Params &p, hipStream_t stream);
+template <> int gemm16_run<true, true>(const Gemm16Params &p, hipStream_t stream);
+
 // What the GEMM planners decide for a shape, for the harness (ko_harness_hooks_t::sgemm_plan, gemm16_plan).
 int debug_sgemm_plan(int64_t m, int64_t n, int64_t k, int *slices, int *k_slice, int *variant);
 int debug_gemm16_plan(int64_t m, int64_t n, int64_t k, int b_layout, int *slices, int *k_slice, int *tile);
